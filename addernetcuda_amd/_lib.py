@@ -1,0 +1,96 @@
+"""ctypes binding of libaddernet_hip.so (the C ABI declared in include/addernet_hip.h)."""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libaddernet_hip.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"{LIB_PATH} is missing: build it with `python -m addernetcuda_amd.build` "
+        "(hipcc, gfx950). There is no fallback implementation.")
+
+lib = ctypes.CDLL(LIB_PATH)
+
+_i, _l, _f, _p, _sz = ctypes.c_int, ctypes.c_long, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+_szp = ctypes.POINTER(ctypes.c_size_t)
+
+_SIGNATURES = {
+    "adder_strerror": (ctypes.c_char_p, [_i]),
+    "adder_last_hip_error": (ctypes.c_char_p, []),
+    "adder_abi_version": (_i, []),
+    "adder_out_dim": (_i, [_i, _i, _i, _i]),
+    "adder_conv2d_fwd_f32": (_i, [_p, _p, _p] + [_i] * 9 + [_p]),
+    "adder_conv2d_bwd_workspace_bytes": (_i, [_i] * 9 + [_szp]),
+    "adder_conv2d_bwd_f32": (_i, [_p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
+    "adder_col_fwd_f32": (_i, [_p, _p, _p, _i, _l, _i, _p]),
+    "adder_col_bwd_workspace_bytes": (_i, [_i, _l, _i, _szp]),
+    "adder_col_bwd_f32": (_i, [_p, _p, _p, _p, _p, _i, _l, _i, _p, _sz, _p]),
+    "adder_col_gradw_f32": (_i, [_p, _p, _p, _p, _i, _l, _i, _p, _sz, _p]),
+    "adder_col_gradx_f32": (_i, [_p, _p, _p, _p, _i, _l, _i, _p]),
+    "adder_norm_scale_workspace_bytes": (_i, [_l, _szp]),
+    "adder_grad_norm_scale_f32": (_i, [_p, _l, _f, _f, _p, _sz, _p]),
+}
+for _name, (_res, _args) in _SIGNATURES.items():
+    _fn = getattr(lib, _name)
+    _fn.restype, _fn.argtypes = _res, _args
+
+EXPORTED = tuple(_SIGNATURES)
+
+
+def check(status, what):
+    """Turn a negative adder_status into the RuntimeError the reference's AT_ASSERTM would raise."""
+    if status != 0:
+        msg = lib.adder_strerror(status).decode()
+        if status == -5:
+            msg += ": " + lib.adder_last_hip_error().decode()
+        raise RuntimeError(f"{what}: {msg}")
+
+
+def require_gpu_f32(t, name):
+    """CHECK_INPUT of adder_cuda.cpp:33-35 (device + contiguity) plus the dtype the kernels assume."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"{name} must be float32, got {t.dtype}")
+
+
+def same_device(*tensors):
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise RuntimeError("all tensors must be on the same device")
+    return dev
+
+
+def stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def conv_dims(x_shape, w_shape, stride, padding):
+    N, Ci, H, W = x_shape
+    Co, Ciw, kh, kw = w_shape
+    if Ci != Ciw:
+        raise RuntimeError(f"input has {Ci} channels but the weight expects {Ciw}")
+    Ho, Wo = lib.adder_out_dim(H, kh, padding, stride), lib.adder_out_dim(W, kw, padding, stride)
+    if Ho <= 0 or Wo <= 0:
+        raise RuntimeError(f"empty output for input {tuple(x_shape)}, kernel {kh}x{kw}, "
+                           f"stride {stride}, padding {padding}")
+    return (N, Ci, H, W, Co, kh, kw, stride, padding), Ho, Wo
+
+
+def conv2d_bwd_workspace(dims, device):
+    need = ctypes.c_size_t(0)
+    check(lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)), "adder_conv2d_bwd_workspace_bytes")
+    # torch's caching allocator hands out >=512-byte aligned blocks and is graph-capture safe
+    return torch.empty(max(need.value, 256), dtype=torch.uint8, device=device), need.value

@@ -1,0 +1,195 @@
+// C ABI of libaddernet_hip.so: argument validation and dispatch.  Every check
+// that can fail does so before the first HIP call, so the error paths can be
+// exercised on a machine without a GPU.
+#include "common.hpp"
+
+#include <string>
+
+namespace adder {
+
+static thread_local std::string g_last_hip_error;
+
+int record_hip_error(hipError_t e) {
+    g_last_hip_error = hipGetErrorString(e);
+    return ADDER_ERR_HIP;
+}
+
+int check_launch() {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? ADDER_OK : record_hip_error(e);
+}
+
+static const long kMaxElems = 0x7fffffffL;
+
+static int make_dims(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, ConvDims &d) {
+    if (N <= 0 || Ci <= 0 || H <= 0 || W <= 0 || Co <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || pad < 0)
+        return ADDER_ERR_BAD_SHAPE;
+    if (H + 2 * pad < kh || W + 2 * pad < kw) return ADDER_ERR_BAD_SHAPE;
+    d = ConvDims{N, Ci, H, W, Co, kh, kw, stride, pad, (H - kh + 2 * pad) / stride + 1,
+                 (W - kw + 2 * pad) / stride + 1};
+    const long nx = (long)N * Ci * H * W, ny = (long)N * Co * d.Ho * d.Wo, nw = (long)Co * Ci * kh * kw;
+    if (nx > kMaxElems || ny > kMaxElems || nw > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    return ADDER_OK;
+}
+
+static bool overlaps(const void *a, size_t na, const void *b, size_t nb) {
+    if (!a || !b) return false;
+    const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+    return pa < pb + nb && pb < pa + na;
+}
+
+}  // namespace adder
+
+using namespace adder;
+
+extern "C" {
+
+const char *adder_strerror(int status) {
+    switch (status) {
+        case ADDER_OK: return "ok";
+        case ADDER_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case ADDER_ERR_BAD_SHAPE: return "non-positive or inconsistent dimension";
+        case ADDER_ERR_TOO_LARGE: return "tensor exceeds 2^31-1 elements";
+        case ADDER_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case ADDER_ERR_HIP: return "HIP runtime error";
+        case ADDER_ERR_ALIAS: return "an output overlaps an input";
+        default: return "unknown status";
+    }
+}
+
+const char *adder_last_hip_error(void) { return g_last_hip_error.c_str(); }
+
+int adder_abi_version(void) { return 1; }
+
+int adder_out_dim(int h, int k, int pad, int stride) {
+    if (h <= 0 || k <= 0 || pad < 0 || stride <= 0 || h + 2 * pad < k) return 0;
+    return (h - k + 2 * pad) / stride + 1;
+}
+
+int adder_conv2d_fwd_f32(const float *x, const float *w, float *y, int N, int Ci, int H, int W, int Co,
+                         int kh, int kw, int stride, int pad, void *stream) {
+    if (!x || !w || !y) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo;
+    if (overlaps(y, ny, x, nx) || overlaps(y, ny, w, nw)) return ADDER_ERR_ALIAS;
+    return launch_fwd(x, w, y, d, static_cast<hipStream_t>(stream));
+}
+
+int adder_conv2d_bwd_workspace_bytes(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
+                                     int pad, size_t *bytes) {
+    if (!bytes) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    *bytes = grad_w_workspace_bytes(d);
+    return ADDER_OK;
+}
+
+int adder_conv2d_bwd_f32(const float *gy, const float *x, const float *w, float *gx, float *gw, float eta,
+                         void *ws, size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream) {
+    if (!gy || !x || !w) return ADDER_ERR_NULL_POINTER;
+    if (!gx && !gw) return ADDER_ERR_NULL_POINTER;
+    if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo;
+    if (overlaps(gx, nx, x, nx) || overlaps(gx, nx, w, nw) || overlaps(gx, nx, gy, ny) ||
+        overlaps(gw, nw, x, nx) || overlaps(gw, nw, w, nw) || overlaps(gw, nw, gy, ny) ||
+        overlaps(gw, nw, gx, nx))
+        return ADDER_ERR_ALIAS;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (gw) {
+        const size_t need = grad_w_workspace_bytes(d);
+        if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
+        if (overlaps(ws, need, x, nx) || overlaps(ws, need, w, nw) || overlaps(ws, need, gy, ny) ||
+            overlaps(ws, need, gx, nx) || overlaps(ws, need, gw, nw))
+            return ADDER_ERR_ALIAS;
+    }
+    if (gx)
+        if (int rc = launch_grad_x(gy, x, w, gx, d, s)) return rc;
+    if (gw)
+        if (int rc = launch_grad_w(gy, x, w, gw, eta, ws, ws_bytes, d, s)) return rc;
+    return ADDER_OK;
+}
+
+static int check_col(int K, long NL, int Co) {
+    if (K <= 0 || NL <= 0 || Co <= 0) return ADDER_ERR_BAD_SHAPE;
+    if ((long)K * NL > kMaxElems || (long)Co * NL > kMaxElems || (long)Co * K > kMaxElems)
+        return ADDER_ERR_TOO_LARGE;
+    return ADDER_OK;
+}
+
+int adder_col_fwd_f32(const float *Xcol, const float *Wcol, float *out, int K, long NL, int Co, void *stream) {
+    if (!Xcol || !Wcol || !out) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_col(K, NL, Co)) return rc;
+    const size_t nx = sizeof(float) * (size_t)K * NL, nw = sizeof(float) * (size_t)Co * K,
+                 ny = sizeof(float) * (size_t)Co * NL;
+    if (overlaps(out, ny, Xcol, nx) || overlaps(out, ny, Wcol, nw)) return ADDER_ERR_ALIAS;
+    return launch_col_fwd(Xcol, Wcol, out, K, NL, Co, static_cast<hipStream_t>(stream));
+}
+
+int adder_col_bwd_workspace_bytes(int K, long NL, int Co, size_t *bytes) {
+    if (!bytes) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_col(K, NL, Co)) return rc;
+    *bytes = col_grad_w_workspace_bytes(K, NL, Co);
+    return ADDER_OK;
+}
+
+static int col_alias(const float *gy, const float *X, const float *Wm, const float *gW, const float *gX, int K,
+                     long NL, int Co) {
+    const size_t nx = sizeof(float) * (size_t)K * NL, nw = sizeof(float) * (size_t)Co * K,
+                 ny = sizeof(float) * (size_t)Co * NL;
+    if (overlaps(gW, nw, X, nx) || overlaps(gW, nw, Wm, nw) || overlaps(gW, nw, gy, ny) ||
+        overlaps(gX, nx, X, nx) || overlaps(gX, nx, Wm, nw) || overlaps(gX, nx, gy, ny) ||
+        overlaps(gX, nx, gW, nw))
+        return ADDER_ERR_ALIAS;
+    return ADDER_OK;
+}
+
+int adder_col_gradw_f32(const float *gy, const float *Xcol, const float *Wcol, float *gW, int K, long NL,
+                        int Co, void *ws, size_t ws_bytes, void *stream) {
+    if (!gy || !Xcol || !Wcol || !gW) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_col(K, NL, Co)) return rc;
+    if (int rc = col_alias(gy, Xcol, Wcol, gW, nullptr, K, NL, Co)) return rc;
+    if (ws_bytes < col_grad_w_workspace_bytes(K, NL, Co)) return ADDER_ERR_WORKSPACE;
+    return launch_col_grad_w(gy, Xcol, Wcol, gW, K, NL, Co, ws, static_cast<hipStream_t>(stream));
+}
+
+int adder_col_gradx_f32(const float *gy, const float *Xcol, const float *Wcol, float *gX, int K, long NL,
+                        int Co, void *stream) {
+    if (!gy || !Xcol || !Wcol || !gX) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_col(K, NL, Co)) return rc;
+    if (int rc = col_alias(gy, Xcol, Wcol, nullptr, gX, K, NL, Co)) return rc;
+    return launch_col_grad_x(gy, Xcol, Wcol, gX, K, NL, Co, static_cast<hipStream_t>(stream));
+}
+
+int adder_col_bwd_f32(const float *gy, const float *Xcol, const float *Wcol, float *gW, float *gX, int K,
+                      long NL, int Co, void *ws, size_t ws_bytes, void *stream) {
+    if (!gy || !Xcol || !Wcol || !gW || !gX) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_col(K, NL, Co)) return rc;
+    if (int rc = col_alias(gy, Xcol, Wcol, gW, gX, K, NL, Co)) return rc;
+    if (ws_bytes < col_grad_w_workspace_bytes(K, NL, Co)) return ADDER_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = launch_col_grad_x(gy, Xcol, Wcol, gX, K, NL, Co, s)) return rc;
+    return launch_col_grad_w(gy, Xcol, Wcol, gW, K, NL, Co, ws, s);
+}
+
+int adder_norm_scale_workspace_bytes(long n, size_t *bytes) {
+    if (!bytes) return ADDER_ERR_NULL_POINTER;
+    if (n <= 0) return ADDER_ERR_BAD_SHAPE;
+    *bytes = norm_scale_workspace_bytes(n);
+    return ADDER_OK;
+}
+
+int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps, void *ws, size_t ws_bytes, void *stream) {
+    if (!g) return ADDER_ERR_NULL_POINTER;
+    if (n <= 0 || !(eta >= 0.f) || !(eps > 0.f)) return ADDER_ERR_BAD_SHAPE;
+    if (!ws || ws_bytes < norm_scale_workspace_bytes(n) || (reinterpret_cast<uintptr_t>(ws) & 255))
+        return ADDER_ERR_WORKSPACE;
+    return launch_norm_scale(g, n, eta, eps, ws, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,92 @@
+// Shared device/host helpers for the gfx950 AdderNet kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/addernet_hip.h"
+
+namespace adder {
+
+// Wave-uniform read-only data (weights) is fetched through the scalar cache:
+// a load from the constant address space with a uniform address becomes
+// s_load_dword*, and the value is then used directly as the SGPR operand of the
+// vector subtract, so weights cost neither VGPRs nor LDS bandwidth.
+typedef const __attribute__((address_space(4))) float *uniform_f32_ptr;
+
+__device__ __forceinline__ uniform_f32_ptr as_uniform(const float *p) {
+    return (uniform_f32_ptr)p;
+}
+
+// hardtanh of adder.cu:17 (x<-1 -> -1, x<=1 -> x, else 1) is one v_med3_f32.
+__device__ __forceinline__ float hardtanh(float v) {
+    return __builtin_amdgcn_fmed3f(v, -1.0f, 1.0f);
+}
+
+__host__ __device__ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ constexpr long ceil_div_l(long a, long b) { return (a + b - 1) / b; }
+__host__ __device__ constexpr int round_up(int a, int b) { return ceil_div(a, b) * b; }
+
+// Read `CNT` consecutive floats from LDS, `ALIGN` (1, 2 or 4 floats) being the
+// alignment the caller guarantees for `p`; widest ds_read that alignment allows.
+template <int CNT, int ALIGN>
+__device__ __forceinline__ void lds_read_strip(const float *p, float (&dst)[CNT]) {
+    int e = 0;
+    if constexpr (ALIGN >= 4) {
+#pragma unroll
+        for (; e + 4 <= CNT; e += 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(p + e);
+            dst[e] = v.x; dst[e + 1] = v.y; dst[e + 2] = v.z; dst[e + 3] = v.w;
+        }
+    }
+    if constexpr (ALIGN >= 2) {
+#pragma unroll
+        for (; e + 2 <= CNT; e += 2) {
+            const float2 v = *reinterpret_cast<const float2 *>(p + e);
+            dst[e] = v.x; dst[e + 1] = v.y;
+        }
+    }
+#pragma unroll
+    for (; e < CNT; ++e) dst[e] = p[e];
+}
+
+// Sum over the 64 lanes of a wave; every lane receives the total.
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+struct ConvDims {
+    int N, Ci, H, W, Co, kh, kw, stride, pad, Ho, Wo;
+    __host__ __device__ int K() const { return Ci * kh * kw; }
+};
+
+// ---- host-side launch plumbing -------------------------------------------------
+int record_hip_error(hipError_t e);  // stores the message, returns ADDER_ERR_HIP
+int check_launch();                  // hipGetLastError -> status
+
+// Launchers implemented in the kernel translation units.
+int launch_fwd(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s);
+int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
+                  hipStream_t s);
+size_t grad_w_workspace_bytes(const ConvDims &d);
+int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta,
+                  void *ws, size_t ws_bytes, const ConvDims &d, hipStream_t s);
+
+size_t norm_scale_workspace_bytes(long n);
+int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);
+
+int launch_col_fwd(const float *X, const float *W, float *out, int K, long NL, int Co, hipStream_t s);
+size_t col_grad_w_workspace_bytes(int K, long NL, int Co);
+int launch_col_grad_w(const float *gy, const float *X, const float *W, float *gW, int K, long NL,
+                      int Co, void *ws, hipStream_t s);
+int launch_col_grad_x(const float *gy, const float *X, const float *W, float *gX, int K, long NL,
+                      int Co, hipStream_t s);
+
+}  // namespace adder

@@ -1,0 +1,226 @@
+// Forward AdderNet convolution, NCHW in -> NCHW out, implicit im2col.
+//   y[n,co,ho,wo] = - sum_{ci,i,j} | w[co,ci,i,j] - xpad[n,ci,ho*s+i-p,wo*s+j-p] |
+// Replaces adder_cuda/adder.cu:19-70 (CONV) together with the unfold + permute
+// copies of adder.py:32-33,38-39 that feed it.
+//
+// The inner operation is two fp32 VALU instructions per (co,k,position) term
+// -- v_sub_f32 d, s_w, v_x ; v_sub_f32 acc, acc, |d| -- and cannot use FMA or
+// MFMA, so the kernels are built to keep everything else off the vector ALU:
+//   * lanes own output positions, weights are wave-uniform and arrive through
+//     the scalar cache as SGPR operands (no VGPRs, no LDS bandwidth);
+//   * the haloed input tile of a workgroup is staged once in LDS with the
+//     padding zeros materialised, and each lane reads its (TN+2)-wide strips
+//     with ds_read_b128/b64 at immediate offsets;
+//   * each lane keeps TM x TN accumulators so one strip read feeds 9*TM*TN terms.
+#include "common.hpp"
+#include "tile3x3.hpp"
+
+namespace adder {
+
+// ---------------------------------------------------------------------------
+// Generic kernel: any kernel size / stride / padding / channel count.
+// One output position per lane, TM output channels per lane, input read
+// straight from global memory with bounds checks.
+// ---------------------------------------------------------------------------
+template <int TM>
+__global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restrict__ x,
+                                                          const float *__restrict__ w,
+                                                          float *__restrict__ y, ConvDims d) {
+    const int total = d.N * d.Ho * d.Wo;
+    int pos = blockIdx.x * 256 + threadIdx.x;
+    const bool active = pos < total;
+    if (!active) pos = total - 1;
+    const int wo = pos % d.Wo;
+    const int ho = (pos / d.Wo) % d.Ho;
+    const int n = pos / (d.Wo * d.Ho);
+    const int co0 = blockIdx.y * TM;
+    const int K = d.K();
+    uniform_f32_ptr wc = as_uniform(w);
+
+    float acc[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) acc[m] = 0.f;
+
+    int wrow[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) wrow[m] = min(co0 + m, d.Co - 1) * K;
+
+    const float *xn = x + (size_t)n * d.Ci * d.H * d.W;
+    for (int ci = 0; ci < d.Ci; ++ci) {
+        for (int i = 0; i < d.kh; ++i) {
+            const int hi = ho * d.stride + i - d.pad;
+            const bool hv = hi >= 0 && hi < d.H;
+            for (int j = 0; j < d.kw; ++j) {
+                const int wi = wo * d.stride + j - d.pad;
+                const bool v = hv && wi >= 0 && wi < d.W;
+                const float xv = v ? xn[((size_t)ci * d.H + hi) * d.W + wi] : 0.f;
+                const int k = (ci * d.kh + i) * d.kw + j;
+#pragma unroll
+                for (int m = 0; m < TM; ++m) acc[m] -= fabsf(wc[wrow[m] + k] - xv);
+            }
+        }
+    }
+    if (active) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+            if (co0 + m < d.Co) y[(((size_t)n * d.Co + co0 + m) * d.Ho + ho) * d.Wo + wo] = acc[m];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Tiled kernel for 3x3, stride 1, pad 1 (Ho = H, Wo = W).
+//
+// A workgroup owns NIMG images x a TH x TW patch of output positions and
+// TM*COW output channels.  TW = TN*SPR: each lane owns a strip of TN adjacent
+// outputs in one row, SPR strips side by side.  The 64*POSW position lanes are
+// replicated COW times, each replica ("co-wave group") taking its own TM
+// output channels and sharing the LDS tile.
+//
+// LDS tile: [img][cc][TH+2][PITCH] floats, double buffered over chunks of CC
+// input channels.  Column 0 of a row is input column w0-1, so a lane's strip
+// starts at column strip*TN, which is 16-byte aligned for TN = 4.
+// ---------------------------------------------------------------------------
+template <class C>
+__global__ __launch_bounds__(C::NTHREADS) void fwd_3x3s1_kernel(const float *__restrict__ x,
+                                                                const float *__restrict__ w,
+                                                                float *__restrict__ y, int N, int Ci,
+                                                                int H, int W, int Co, int tilesH,
+                                                                int tilesW) {
+    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ;
+    extern __shared__ __align__(16) float smem[];
+
+    int b = blockIdx.x;
+    const int tw = b % tilesW; b /= tilesW;
+    const int th = b % tilesH; b /= tilesH;
+    const int n0 = b * C::NIMG;
+    const int h0 = th * C::TH, w0 = tw * C::TW;
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int pw = wave % C::POSW, cw = wave / C::POSW;
+    int p = pw * 64 + lane;
+    const bool lane_ok = p < C::LANES;
+    if (!lane_ok) p = C::LANES - 1;
+    const int strip = p % C::SPR;
+    const int row = (p / C::SPR) % C::TH;
+    const int img = p / (C::SPR * C::TH);
+    const int co_base = (blockIdx.y * C::COW + cw) * TM;
+    const int K = Ci * 9;
+    uniform_f32_ptr wc = as_uniform(w);
+
+    // wave-uniform weight row offsets (clamped so tail channels read valid memory)
+    int wrow[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m)
+        wrow[m] = __builtin_amdgcn_readfirstlane(min(co_base + m, Co - 1) * K);
+
+    float acc[TM][TN];
+#pragma unroll
+    for (int m = 0; m < TM; ++m)
+#pragma unroll
+        for (int t = 0; t < TN; ++t) acc[m][t] = 0.f;
+
+    const int lane_off = img * C::CC * C::PLANE + row * C::PITCH + strip * TN;
+    const int nchunks = ceil_div(Ci, C::CC);
+
+    TileStage<C> st;
+    tile_fetch<C>(st, x, 0, Ci, n0, N, h0, w0, H, W);
+    tile_commit<C>(st, smem);
+    __syncthreads();
+
+    for (int c = 0; c < nchunks; ++c) {
+        const int ci0 = c * C::CC;
+        if (c + 1 < nchunks) tile_fetch<C>(st, x, ci0 + C::CC, Ci, n0, N, h0, w0, H, W);
+
+        const float *lbase = smem + (c & 1) * C::BUF + lane_off;
+        const int ccnt = min(C::CC, Ci - ci0);
+#pragma unroll 1
+        for (int cc = 0; cc < ccnt; cc += CQ) {
+            float xr[CQ][3][TN + 2];
+#pragma unroll
+            for (int q = 0; q < CQ; ++q)
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + (cc + q) * C::PLANE + i * C::PITCH, xr[q][i]);
+            const int kofs = (ci0 + cc) * 9;
+#pragma unroll
+            for (int m = 0; m < TM; ++m) {
+                float wv[CQ * 9];
+#pragma unroll
+                for (int e = 0; e < CQ * 9; ++e) wv[e] = wc[wrow[m] + kofs + e];
+#pragma unroll
+                for (int q = 0; q < CQ; ++q)
+#pragma unroll
+                    for (int i = 0; i < 3; ++i)
+#pragma unroll
+                        for (int j = 0; j < 3; ++j)
+#pragma unroll
+                            for (int t = 0; t < TN; ++t)
+                                acc[m][t] -= fabsf(wv[q * 9 + i * 3 + j] - xr[q][i][t + j]);
+            }
+        }
+
+        if (c + 1 < nchunks) tile_commit<C>(st, smem + ((c + 1) & 1) * C::BUF);
+        __syncthreads();
+    }
+
+    const int n = n0 + img, ho = h0 + row, wo = w0 + strip * TN;
+    if (lane_ok && n < N && ho < H) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const int co = co_base + m;
+            if (co < Co) {
+                float *dst = y + (((size_t)n * Co + co) * H + ho) * W + wo;
+                if (TN % 4 == 0 && wo + TN <= W) {
+#pragma unroll
+                    for (int t = 0; t < TN; t += 4)
+                        *reinterpret_cast<float4 *>(dst + t) =
+                            make_float4(acc[m][t], acc[m][t + 1], acc[m][t + 2], acc[m][t + 3]);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < TN; ++t)
+                        if (wo + t < W) dst[t] = acc[m][t];
+                }
+            }
+        }
+    }
+}
+
+template <class C>
+static int launch_fwd_3x3s1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+    const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
+    const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
+    const int gy = ceil_div(d.Co, C::TM * C::COW);
+    if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
+    static bool attr_set = false;
+    if (!attr_set && C::LDS_BYTES > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3s1_kernel<C>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return record_hip_error(e);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(fwd_3x3s1_kernel<C>, dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w,
+                       y, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW);
+    return check_launch();
+}
+
+//                      TN SPR TH NIMG TM COW CC CQ
+using FwdW32 = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1>;   // 32-wide maps, whole image per workgroup
+using FwdW16 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1>;   // 16-wide maps, one image per workgroup
+using FwdW8  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1>;    // 8-wide maps, one image x 32 channels per workgroup
+
+int launch_fwd(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+    const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
+    if (k3s1p1 && d.W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+        if (d.W > 16) return launch_fwd_3x3s1<FwdW32>(x, w, y, d, s);
+        if (d.W > 8) return launch_fwd_3x3s1<FwdW16>(x, w, y, d, s);
+        return launch_fwd_3x3s1<FwdW8>(x, w, y, d, s);
+    }
+    constexpr int TM = 8;
+    const long total = (long)d.N * d.Ho * d.Wo;
+    hipLaunchKernelGGL(fwd_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Co, TM)),
+                       dim3(256), 0, s, x, w, y, d);
+    return check_launch();
+}
+
+}  // namespace adder

@@ -1,0 +1,235 @@
+// Input gradient of the AdderNet convolution, NCHW, gather form (no atomics):
+//   gx[n,ci,hi,wi] = sum_{co,i,j} hardtanh(w[co,ci,i,j] - x[n,ci,hi,wi]) * gy[n,co,ho,wo]
+//   with ho = (hi + p - i)/s, wo = (wi + p - j)/s when those divide exactly and
+//   fall inside the output; taps that land in the padding are dropped.
+// Replaces the grad_i half of adder_cuda/adder.cu:194-272 (CONV_BACKWARD),
+// adder.cu:133-192 (CONV_INPUT), and the permute + F.fold (col2im) autograd
+// runs after them for adder.py:32-33.  hardtanh is adder.cu:17.
+//
+// Three fp32 VALU instructions per term: v_sub (SGPR weight - own x),
+// v_med3 (clamp), v_fma (times gy).  Lanes own input positions, so x and the
+// accumulators stay in registers for the whole kernel, weights are SGPR
+// operands, and the haloed gy tile is staged in LDS with zeros outside the
+// output so invalid taps vanish without predication.
+#include "common.hpp"
+#include "tile3x3.hpp"
+
+namespace adder {
+
+// ---------------------------------------------------------------------------
+// Generic kernel: any kernel size / stride / padding.
+// ---------------------------------------------------------------------------
+template <int TM>
+__global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__restrict__ gy,
+                                                             const float *__restrict__ x,
+                                                             const float *__restrict__ w,
+                                                             float *__restrict__ gx, ConvDims d) {
+    const int total = d.N * d.H * d.W;
+    int pos = blockIdx.x * 256 + threadIdx.x;
+    const bool active = pos < total;
+    if (!active) pos = total - 1;
+    const int wi = pos % d.W;
+    const int hi = (pos / d.W) % d.H;
+    const int n = pos / (d.W * d.H);
+    const int ci0 = blockIdx.y * TM;
+    const int KK = d.kh * d.kw;
+    const int K = d.Ci * KK;
+    uniform_f32_ptr wc = as_uniform(w);
+
+    float xr[TM], acc[TM];
+    int wofs[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) {
+        const int ci = min(ci0 + m, d.Ci - 1);
+        xr[m] = x[(((size_t)n * d.Ci + ci) * d.H + hi) * d.W + wi];
+        acc[m] = 0.f;
+        wofs[m] = ci * KK;
+    }
+    const float *gn = gy + (size_t)n * d.Co * d.Ho * d.Wo;
+    for (int co = 0; co < d.Co; ++co) {
+        for (int i = 0; i < d.kh; ++i) {
+            const int th = hi + d.pad - i;
+            const int ho = th / d.stride;
+            const bool hv = th >= 0 && ho * d.stride == th && ho < d.Ho;
+            for (int j = 0; j < d.kw; ++j) {
+                const int tw = wi + d.pad - j;
+                const int wo = tw / d.stride;
+                const bool v = hv && tw >= 0 && wo * d.stride == tw && wo < d.Wo;
+                const float g = v ? gn[((size_t)co * d.Ho + ho) * d.Wo + wo] : 0.f;
+                const int kofs = co * K + i * d.kw + j;
+#pragma unroll
+                for (int m = 0; m < TM; ++m)
+                    acc[m] = fmaf(hardtanh(wc[kofs + wofs[m]] - xr[m]), g, acc[m]);
+            }
+        }
+    }
+    if (active) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+            if (ci0 + m < d.Ci) gx[(((size_t)n * d.Ci + ci0 + m) * d.H + hi) * d.W + wi] = acc[m];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Tiled kernel for 3x3, stride 1, pad 1.  Same tile geometry as the forward
+// kernel with the roles swapped: the LDS tile holds gy (chunks of CC output
+// channels, reduction axis), a lane owns TN input positions x TM input
+// channels, COW wave groups take different input channels.
+//   gx[hi,wi] += hardtanh(w[co,ci,i,j] - x[hi,wi]) * gy[hi+1-i, wi+1-j]
+// In tile coordinates (row 0 = h0-1, column 0 = w0-1) that is row+2-i, t+2-j.
+// ---------------------------------------------------------------------------
+template <class C>
+__global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *__restrict__ gy,
+                                                                   const float *__restrict__ x,
+                                                                   const float *__restrict__ w,
+                                                                   float *__restrict__ gx, int N, int Ci,
+                                                                   int H, int W, int Co, int tilesH,
+                                                                   int tilesW) {
+    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ;
+    extern __shared__ __align__(16) float smem[];
+
+    int b = blockIdx.x;
+    const int tw = b % tilesW; b /= tilesW;
+    const int th = b % tilesH; b /= tilesH;
+    const int n0 = b * C::NIMG;
+    const int h0 = th * C::TH, w0 = tw * C::TW;
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int pw = wave % C::POSW, cw = wave / C::POSW;
+    int p = pw * 64 + lane;
+    const bool lane_ok = p < C::LANES;
+    if (!lane_ok) p = C::LANES - 1;
+    const int strip = p % C::SPR;
+    const int row = (p / C::SPR) % C::TH;
+    const int img = p / (C::SPR * C::TH);
+    const int ci_base = (blockIdx.y * C::COW + cw) * TM;
+    const int K = Ci * 9;
+    uniform_f32_ptr wc = as_uniform(w);
+
+    const int n = n0 + img, hi = h0 + row, wi0 = w0 + strip * TN;
+    const bool pos_ok = lane_ok && n < N && hi < H;
+    const int nc = min(n, N - 1), hc = min(hi, H - 1);
+
+    // own x values and accumulators live in registers for the whole kernel
+    float xr[TM][TN], acc[TM][TN];
+    int wofs[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) {
+        const int ci = min(ci_base + m, Ci - 1);
+        wofs[m] = __builtin_amdgcn_readfirstlane(ci * 9);
+        const float *src = x + (((size_t)nc * Ci + ci) * H + hc) * W;
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            xr[m][t] = src[min(wi0 + t, W - 1)];
+            acc[m][t] = 0.f;
+        }
+    }
+
+    const int lane_off = img * C::CC * C::PLANE + row * C::PITCH + strip * TN;
+    const int nchunks = ceil_div(Co, C::CC);
+
+    TileStage<C> st;
+    tile_fetch<C>(st, gy, 0, Co, n0, N, h0, w0, H, W);
+    tile_commit<C>(st, smem);
+    __syncthreads();
+
+    for (int c = 0; c < nchunks; ++c) {
+        const int co0 = c * C::CC;
+        if (c + 1 < nchunks) tile_fetch<C>(st, gy, co0 + C::CC, Co, n0, N, h0, w0, H, W);
+
+        const float *lbase = smem + (c & 1) * C::BUF + lane_off;
+        const int ccnt = min(C::CC, Co - co0);
+#pragma unroll 1
+        for (int cc = 0; cc < ccnt; cc += CQ) {
+            float gr[CQ][3][TN + 2];
+#pragma unroll
+            for (int q = 0; q < CQ; ++q)
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + (cc + q) * C::PLANE + i * C::PITCH, gr[q][i]);
+#pragma unroll
+            for (int q = 0; q < CQ; ++q) {
+                const int kofs = (co0 + cc + q) * K;
+#pragma unroll
+                for (int m = 0; m < TM; ++m) {
+                    float wv[9];
+#pragma unroll
+                    for (int e = 0; e < 9; ++e) wv[e] = wc[kofs + wofs[m] + e];
+#pragma unroll
+                    for (int i = 0; i < 3; ++i)
+#pragma unroll
+                        for (int j = 0; j < 3; ++j)
+#pragma unroll
+                            for (int t = 0; t < TN; ++t)
+                                acc[m][t] = fmaf(hardtanh(wv[i * 3 + j] - xr[m][t]), gr[q][2 - i][t + 2 - j],
+                                                 acc[m][t]);
+                }
+            }
+        }
+
+        if (c + 1 < nchunks) tile_commit<C>(st, smem + ((c + 1) & 1) * C::BUF);
+        __syncthreads();
+    }
+
+    if (pos_ok) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const int ci = ci_base + m;
+            if (ci < Ci) {
+                float *dst = gx + (((size_t)n * Ci + ci) * H + hi) * W + wi0;
+                if (TN % 4 == 0 && wi0 + TN <= W) {
+#pragma unroll
+                    for (int t = 0; t < TN; t += 4)
+                        *reinterpret_cast<float4 *>(dst + t) =
+                            make_float4(acc[m][t], acc[m][t + 1], acc[m][t + 2], acc[m][t + 3]);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < TN; ++t)
+                        if (wi0 + t < W) dst[t] = acc[m][t];
+                }
+            }
+        }
+    }
+}
+
+template <class C>
+static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, float *gx,
+                               const ConvDims &d, hipStream_t s) {
+    const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
+    const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
+    const int gyd = ceil_div(d.Ci, C::TM * C::COW);
+    if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
+    static bool attr_set = false;
+    if (!attr_set && C::LDS_BYTES > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return record_hip_error(e);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(grad_x_3x3s1_kernel<C>, dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
+                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW);
+    return check_launch();
+}
+
+//                        TN SPR TH NIMG TM COW CC CQ
+using GxW32 = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1>;
+using GxW16 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1>;
+using GxW8  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1>;
+
+int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
+                  hipStream_t s) {
+    const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
+    if (k3s1p1 && d.W % 4 == 0 && (reinterpret_cast<uintptr_t>(gy) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(gx) & 15) == 0) {
+        if (d.W > 16) return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s);
+        if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s);
+        return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s);
+    }
+    constexpr int TM = 8;
+    const long total = (long)d.N * d.H * d.W;
+    hipLaunchKernelGGL(grad_x_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Ci, TM)),
+                       dim3(256), 0, s, gy, x, w, gx, d);
+    return check_launch();
+}
+
+}  // namespace adder

@@ -1,0 +1,125 @@
+/*
+ * addernet_hip.h -- C ABI of libaddernet_hip.so (AdderNet convolution for gfx950).
+ *
+ * Plain pointers and sizes only: every pointer is a DEVICE pointer to a dense,
+ * row-major fp32 array, `stream` is a hipStream_t passed as void* (NULL = the
+ * default stream).  Every function returns 0 on success or a negative
+ * adder_status; nothing aborts, nothing allocates, nothing synchronises.  All
+ * launches are asynchronous on `stream` and safe to record into a HIP graph
+ * (no memset nodes: scratch is cleared by kernels).
+ *
+ * The entry points replace the reference's native boundary, i.e. the four
+ * pybind functions of adder_cuda/adder_cuda.cpp:88-93 and the host launchers
+ * behind them (adder_cuda/adder.cu:274-465), plus the PyTorch glue the
+ * reference runs around them (adder.py:22-41 im2col/col2im, adder.py:78 scaling).
+ */
+#ifndef ADDERNET_HIP_H
+#define ADDERNET_HIP_H
+
+#include <stddef.h>
+
+#if defined(__GNUC__)
+#define ADDER_API __attribute__((visibility("default")))
+#else
+#define ADDER_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum adder_status {
+    ADDER_OK = 0,
+    ADDER_ERR_NULL_POINTER = -1,   /* a required pointer is NULL                         */
+    ADDER_ERR_BAD_SHAPE = -2,      /* non-positive or inconsistent dimension             */
+    ADDER_ERR_TOO_LARGE = -3,      /* a tensor exceeds 2^31-1 elements                   */
+    ADDER_ERR_WORKSPACE = -4,      /* workspace missing, misaligned or too small         */
+    ADDER_ERR_HIP = -5,            /* a HIP call failed; see adder_last_hip_error()      */
+    ADDER_ERR_ALIAS = -6           /* an output overlaps an input                        */
+} adder_status;
+
+/* Text for a status code (static storage). */
+ADDER_API const char *adder_strerror(int status);
+/* hipGetErrorString of the last HIP failure seen by the calling thread ("" if none). */
+ADDER_API const char *adder_last_hip_error(void);
+/* ABI version: bumped on any signature change. */
+ADDER_API int adder_abi_version(void);
+
+/* Output extent floor((h - k + 2p)/s) + 1; replaces adder.py:26-31. Returns <=0 if invalid. */
+ADDER_API int adder_out_dim(int h, int k, int pad, int stride);
+
+/* ------------------------------------------------------------------------
+ * Fused NCHW path (what adder2d itself uses).
+ *   x  (N, Ci, H, W)        w  (Co, Ci, kh, kw)        y, gy (N, Co, Ho, Wo)
+ * Zero padding; padded taps count as x = 0 (they add -|w| to y and -w*gy to
+ * grad_w) exactly as F.unfold makes them do in adder.py:32.
+ * ---------------------------------------------------------------------- */
+
+/* y = -sum_{ci,i,j} |w - x_patch|.  Replaces adder2d_function + adder.forward
+ * (adder.py:22-41, 44-60) and ADDER_CONV (adder_cuda.cpp:37-46, adder.cu:19-70,
+ * 274-320) including the unfold / permute copies around it.  y is overwritten. */
+ADDER_API int adder_conv2d_fwd_f32(const float *x, const float *w, float *y,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream);
+
+/* Bytes of scratch adder_conv2d_bwd_f32 needs for these dimensions. */
+ADDER_API int adder_conv2d_bwd_workspace_bytes(int N, int Ci, int H, int W, int Co, int kh, int kw,
+                                     int stride, int pad, size_t *bytes);
+
+/* Backward of the layer.  Replaces adder.backward (adder.py:62-80), ADDER_BACKWARD
+ * (adder_cuda.cpp:74-86, adder.cu:194-272, 404-465), the fold that autograd runs
+ * after it and the Python-side scaling of adder.py:78.
+ *   gx (N, Ci, H, W)   = fold( sum_co hardtanh(w - x) * gy )        overwritten; may be NULL
+ *   gw (Co, Ci, kh, kw) = sum_{n,l} (x - w) * gy                    overwritten; may be NULL
+ *   eta > 0: gw <- gw / max(||gw||_2, 1e-12) * sqrt(Co*Ci*kh*kw) * eta   (reference: eta = 0.2)
+ *   eta == 0: gw is left raw.
+ * ws / ws_bytes: scratch of at least adder_conv2d_bwd_workspace_bytes, 256-byte aligned. */
+ADDER_API int adder_conv2d_bwd_f32(const float *gy, const float *x, const float *w,
+                         float *gx, float *gw, float eta,
+                         void *ws, size_t ws_bytes,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Column-matrix path: the literal signatures of the reference extension.
+ *   Xcol (K, NL)   Wcol (Co, K)   out, gy (Co, NL)   gW (Co, K)   gX (K, NL)
+ * The reference ACCUMULATES into gW / gX (atomicAdd into caller-zeroed
+ * buffers, adder.cu:125,186,266-267; adder.py:66-67); so do these.
+ * ---------------------------------------------------------------------- */
+
+/* ADDER_CONV (adder_cuda.cpp:37-46; adder.cu:19-70, 274-320). out is overwritten. */
+ADDER_API int adder_col_fwd_f32(const float *Xcol, const float *Wcol, float *out,
+                      int K, long NL, int Co, void *stream);
+
+/* Scratch for the three column-matrix backward entry points. */
+ADDER_API int adder_col_bwd_workspace_bytes(int K, long NL, int Co, size_t *bytes);
+
+/* ADDER_BACKWARD (adder_cuda.cpp:74-86; adder.cu:194-272, 404-465): gW += ..., gX += ... */
+ADDER_API int adder_col_bwd_f32(const float *gy, const float *Xcol, const float *Wcol,
+                      float *gW, float *gX, int K, long NL, int Co,
+                      void *ws, size_t ws_bytes, void *stream);
+
+/* ADDER_CONV_WEIGHT (adder_cuda.cpp:48-59; adder.cu:72-131, 322-355): gW += sum_nl (X - W) * gy */
+ADDER_API int adder_col_gradw_f32(const float *gy, const float *Xcol, const float *Wcol,
+                        float *gW, int K, long NL, int Co,
+                        void *ws, size_t ws_bytes, void *stream);
+
+/* ADDER_CONV_INPUT (adder_cuda.cpp:61-72; adder.cu:133-192, 357-402): gX += sum_co hardtanh(W - X) * gy.
+ * Follows the arithmetic the reference states in adder_cuda/test_cuda.py:57-60, not the
+ * un-parenthesised macro expansion at adder.cu:170. */
+ADDER_API int adder_col_gradx_f32(const float *gy, const float *Xcol, const float *Wcol,
+                        float *gX, int K, long NL, int Co, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Adaptive learning-rate scaling, in place (adder.py:78):
+ *   g <- g / max(||g||_2, eps) * sqrt(n) * eta
+ * ws must hold adder_norm_scale_workspace_bytes(n) bytes.
+ * ---------------------------------------------------------------------- */
+ADDER_API int adder_norm_scale_workspace_bytes(long n, size_t *bytes);
+ADDER_API int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps,
+                              void *ws, size_t ws_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ADDERNET_HIP_H */
