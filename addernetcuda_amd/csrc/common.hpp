@@ -79,6 +79,15 @@ size_t grad_w_workspace_bytes(const ConvDims &d);
 int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta,
                   void *ws, size_t ws_bytes, const ConvDims &d, hipStream_t s);
 
+// 1x1 / pad 0 / stride 1-2 kernels (conv1x1.hip)
+bool conv1x1_supported(const ConvDims &d, const void *a, const void *b);
+int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s);
+int launch_grad_x_1x1(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
+                      hipStream_t s);
+int grad_w_1x1_slots(const ConvDims &d);
+int launch_grad_w_1x1(const float *gy, const float *x, float *part, float *sgpart, int slots,
+                      const ConvDims &d, hipStream_t s);
+
 size_t norm_scale_workspace_bytes(long n);
 int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);
 

@@ -1,0 +1,300 @@
+// 1x1 AdderNet convolution, pad 0, stride S = 1 or 2 (the ResNet downsample
+// path, resnet20.py:66-70): the same three operations as the 3x3 kernels with
+// K = Ci, so there is no halo and no LDS tile -- every lane reads its own
+// float4 of the source row and keeps a TM x TN register tile; weights are
+// wave-uniform SGPR operands.
+//   forward  y[n,co,ho,wo]  = -sum_ci |w[co,ci] - x[n,ci,ho*S,wo*S]|
+//   grad_x   gx[n,ci,hi,wi] =  sum_co hardtanh(w[co,ci] - x) * gy[n,co,hi/S,wi/S]  on the sampled
+//                              grid, exactly 0 on the positions stride 2 skips
+//   grad_w   gw[co,ci]      =  sum x*gy - w * sum gy   (partials folded per wave, summed in fp64)
+// Replaces adder.cu:19-70 / 194-272 for these shapes together with the
+// unfold/fold copies of adder.py:32-33,38-39.
+#include "common.hpp"
+
+namespace adder {
+
+// A lane owns 4/S adjacent outputs of one output row: one aligned float4 of the source row.
+template <int S>
+struct Lane1x1 {
+    static constexpr int TN = 4 / S;
+    int n, ho, wo0;   // first output of the lane
+    bool ok;
+    __device__ __forceinline__ Lane1x1(int g, int groups, int gpr, int Ho) {
+        ok = g < groups;
+        if (!ok) g = groups - 1;
+        const int q = g % gpr;
+        ho = (g / gpr) % Ho;
+        n = g / (gpr * Ho);
+        wo0 = q * TN;
+    }
+};
+
+template <int S, int TM>
+__global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                      float *__restrict__ y, int N, int Ci, int H, int W,
+                                                      int Co, int Ho, int Wo, int gpr, int groups) {
+    constexpr int TN = 4 / S;
+    const Lane1x1<S> L(blockIdx.x * 256 + threadIdx.x, groups, gpr, Ho);
+    const int co0 = blockIdx.y * TM;
+    uniform_f32_ptr wc = as_uniform(w);
+    int wrow[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) wrow[m] = min(co0 + m, Co - 1) * Ci;
+    float acc[TM][TN];
+#pragma unroll
+    for (int m = 0; m < TM; ++m)
+#pragma unroll
+        for (int t = 0; t < TN; ++t) acc[m][t] = 0.f;
+
+    const size_t plane = (size_t)H * W;
+    const float *xp = x + (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
+    int ci = 0;
+    for (; ci + 4 <= Ci; ci += 4) {
+        float4 xv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xv[e] = *reinterpret_cast<const float4 *>(xp + (size_t)(ci + e) * plane);
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float wv = wc[wrow[m] + ci + e];
+                const float xs[4] = {xv[e].x, xv[e].y, xv[e].z, xv[e].w};
+#pragma unroll
+                for (int t = 0; t < TN; ++t) acc[m][t] -= fabsf(wv - xs[t * S]);
+            }
+    }
+    for (; ci < Ci; ++ci) {
+        const float4 v = *reinterpret_cast<const float4 *>(xp + (size_t)ci * plane);
+        const float xs[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const float wv = wc[wrow[m] + ci];
+#pragma unroll
+            for (int t = 0; t < TN; ++t) acc[m][t] -= fabsf(wv - xs[t * S]);
+        }
+    }
+    if (L.ok) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            if (co0 + m >= Co) continue;
+            float *dst = y + (((size_t)L.n * Co + co0 + m) * Ho + L.ho) * Wo + L.wo0;
+            if constexpr (TN == 4)
+                *reinterpret_cast<float4 *>(dst) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+            else
+                *reinterpret_cast<float2 *>(dst) = make_float2(acc[m][0], acc[m][1]);
+        }
+    }
+}
+
+template <int S, int TM>
+__global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict__ gy,
+                                                         const float *__restrict__ x,
+                                                         const float *__restrict__ w, float *__restrict__ gx,
+                                                         int N, int Ci, int H, int W, int Co, int Ho, int Wo,
+                                                         int gpr, int groups) {
+    constexpr int TN = 4 / S;
+    const Lane1x1<S> L(blockIdx.x * 256 + threadIdx.x, groups, gpr, Ho);
+    const int ci0 = blockIdx.y * TM;
+    uniform_f32_ptr wc = as_uniform(w);
+    const size_t plane = (size_t)H * W;
+    const size_t xoff = (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
+    float xr[TM][TN], acc[TM][TN];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) {
+        const float4 v = *reinterpret_cast<const float4 *>(x + xoff + (size_t)min(ci0 + m, Ci - 1) * plane);
+        const float xs[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int t = 0; t < TN; ++t) { xr[m][t] = xs[t * S]; acc[m][t] = 0.f; }
+    }
+    const size_t gplane = (size_t)Ho * Wo;
+    const float *gp = gy + (size_t)L.n * Co * gplane + (size_t)L.ho * Wo + L.wo0;
+    for (int co = 0; co < Co; ++co) {
+        float g[TN];
+        if constexpr (TN == 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(gp + (size_t)co * gplane);
+            g[0] = v.x; g[1] = v.y; g[2] = v.z; g[3] = v.w;
+        } else {
+            const float2 v = *reinterpret_cast<const float2 *>(gp + (size_t)co * gplane);
+            g[0] = v.x; g[1] = v.y;
+        }
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const float wv = wc[co * Ci + min(ci0 + m, Ci - 1)];
+#pragma unroll
+            for (int t = 0; t < TN; ++t) acc[m][t] = fmaf(hardtanh(wv - xr[m][t]), g[t], acc[m][t]);
+        }
+    }
+    if (L.ok) {
+        const bool row2 = S == 2 && L.ho * 2 + 1 < H;  // the odd row below: never sampled by stride 2
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            if (ci0 + m >= Ci) continue;
+            float *dst = gx + xoff + (size_t)(ci0 + m) * plane;
+            if constexpr (S == 1) {
+                *reinterpret_cast<float4 *>(dst) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+            } else {
+                *reinterpret_cast<float4 *>(dst) = make_float4(acc[m][0], 0.f, acc[m][1], 0.f);
+                if (row2) *reinterpret_cast<float4 *>(dst + W) = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    }
+}
+
+// grad_w: a wave owns TM output channels x TC input channels; its lanes walk over position
+// groups, then the 64 lanes are folded through LDS (16 sums per round).
+template <int S, int TM, int TC>
+__global__ __launch_bounds__(256) void grad_w_1x1_kernel(const float *__restrict__ gy,
+                                                         const float *__restrict__ x, float *__restrict__ part,
+                                                         float *__restrict__ sgpart, int N, int Ci, int H,
+                                                         int W, int Co, int Ho, int Wo, int gpr, int groups) {
+    constexpr int TN = 4 / S, A = TM * TC;
+    const int co0 = blockIdx.y * TM, ci0 = blockIdx.z * TC;
+    const size_t plane = (size_t)H * W, gplane = (size_t)Ho * Wo;
+    float acc[TM][TC], sg[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) {
+        sg[m] = 0.f;
+#pragma unroll
+        for (int c = 0; c < TC; ++c) acc[m][c] = 0.f;
+    }
+    for (int g0 = blockIdx.x * 256 + threadIdx.x; g0 < groups; g0 += gridDim.x * 256) {
+        const Lane1x1<S> L(g0, groups, gpr, Ho);
+        const float *xp = x + (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
+        const float *gp = gy + (size_t)L.n * Co * gplane + (size_t)L.ho * Wo + L.wo0;
+        float xs[TC][TN], gs[TM][TN];
+#pragma unroll
+        for (int c = 0; c < TC; ++c) {
+            const float4 v = *reinterpret_cast<const float4 *>(xp + (size_t)min(ci0 + c, Ci - 1) * plane);
+            const float t4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int t = 0; t < TN; ++t) xs[c][t] = t4[t * S];
+        }
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const float *p = gp + (size_t)min(co0 + m, Co - 1) * gplane;
+            if constexpr (TN == 4) {
+                const float4 v = *reinterpret_cast<const float4 *>(p);
+                gs[m][0] = v.x; gs[m][1] = v.y; gs[m][2] = v.z; gs[m][3] = v.w;
+            } else {
+                const float2 v = *reinterpret_cast<const float2 *>(p);
+                gs[m][0] = v.x; gs[m][1] = v.y;
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                sg[m] += gs[m][t];
+#pragma unroll
+                for (int c = 0; c < TC; ++c) acc[m][c] = fmaf(gs[m][t], xs[c][t], acc[m][c]);
+            }
+        }
+    }
+    // fold lanes, then the 4 waves of the workgroup
+    __shared__ float red[4][64 * 17];
+    __shared__ float wsum[4][A + TM];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int TOT = A + TM;
+    float all[TOT];
+#pragma unroll
+    for (int a = 0; a < A; ++a) all[a] = acc[a / TC][a % TC];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) all[A + m] = sg[m];
+    constexpr int ROUNDS = ceil_div(TOT, 16);
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[wave][lane * 17 + e] = (r * 16 + e < TOT) ? all[(r * 16 + e) % TOT] : 0.f;
+        __syncthreads();
+        const int e = lane & 15, rg = lane >> 4;
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) s += red[wave][(rg * 16 + k) * 17 + e];
+        s += __shfl_xor(s, 16, 64);
+        s += __shfl_xor(s, 32, 64);
+        if (rg == 0 && r * 16 + e < TOT) wsum[wave][r * 16 + e] = s;
+        __syncthreads();
+    }
+    if (threadIdx.x < TOT) {
+        const int a = threadIdx.x;
+        const float s = (wsum[0][a] + wsum[1][a]) + (wsum[2][a] + wsum[3][a]);
+        if (a < A) {
+            const int co = co0 + a / TC, ci = ci0 + a % TC;
+            if (co < Co && ci < Ci) part[(size_t)blockIdx.x * Co * Ci + (size_t)co * Ci + ci] = s;
+        } else if (blockIdx.z == 0) {
+            const int co = co0 + a - A;
+            if (co < Co) sgpart[(size_t)blockIdx.x * Co + co] = s;
+        }
+    }
+}
+
+// ---- host side ------------------------------------------------------------------
+bool conv1x1_supported(const ConvDims &d, const void *a, const void *b) {
+    if (d.kh != 1 || d.kw != 1 || d.pad != 0 || (d.stride != 1 && d.stride != 2)) return false;
+    // one aligned float4 of the source row per lane, whole float4 / float2 groups of the output row
+    if (d.W % 4 != 0 || d.Wo % (4 / d.stride) != 0) return false;
+    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) return false;
+    return true;
+}
+
+static void lane_space(const ConvDims &d, int &gpr, int &groups) {
+    gpr = d.Wo / (4 / d.stride);
+    groups = d.N * d.Ho * gpr;
+}
+
+int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+    constexpr int TM = 8;
+    int gpr, groups;
+    lane_space(d, gpr, groups);
+    const dim3 grid(ceil_div(groups, 256), ceil_div(d.Co, TM));
+    if (d.stride == 1)
+        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM>), grid, dim3(256), 0, s, x, w, y, d.N, d.Ci, d.H, d.W, d.Co, d.Ho,
+                           d.Wo, gpr, groups);
+    else
+        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM>), grid, dim3(256), 0, s, x, w, y, d.N, d.Ci, d.H, d.W, d.Co, d.Ho,
+                           d.Wo, gpr, groups);
+    return check_launch();
+}
+
+int launch_grad_x_1x1(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
+                      hipStream_t s) {
+    constexpr int TM = 8;
+    int gpr, groups;
+    lane_space(d, gpr, groups);
+    const dim3 grid(ceil_div(groups, 256), ceil_div(d.Ci, TM));
+    if (d.stride == 1)
+        hipLaunchKernelGGL((grad_x_1x1_kernel<1, TM>), grid, dim3(256), 0, s, gy, x, w, gx, d.N, d.Ci, d.H, d.W,
+                           d.Co, d.Ho, d.Wo, gpr, groups);
+    else
+        hipLaunchKernelGGL((grad_x_1x1_kernel<2, TM>), grid, dim3(256), 0, s, gy, x, w, gx, d.N, d.Ci, d.H, d.W,
+                           d.Co, d.Ho, d.Wo, gpr, groups);
+    return check_launch();
+}
+
+static constexpr int kGw1x1TM = 8, kGw1x1TC = 8;
+
+int grad_w_1x1_slots(const ConvDims &d) {
+    int gpr, groups;
+    lane_space(d, gpr, groups);
+    const int blocks_yz = ceil_div(d.Co, kGw1x1TM) * ceil_div(d.Ci, kGw1x1TC);
+    int want = ceil_div(1024, blocks_yz);                 // ~4 workgroups per CU
+    const int cap = ceil_div(groups, 256 * 4);            // at least 4 position groups per lane
+    if (want > cap) want = cap;
+    return want < 1 ? 1 : want;
+}
+
+int launch_grad_w_1x1(const float *gy, const float *x, float *part, float *sgpart, int slots,
+                      const ConvDims &d, hipStream_t s) {
+    int gpr, groups;
+    lane_space(d, gpr, groups);
+    const dim3 grid(slots, ceil_div(d.Co, kGw1x1TM), ceil_div(d.Ci, kGw1x1TC));
+    if (d.stride == 1)
+        hipLaunchKernelGGL((grad_w_1x1_kernel<1, kGw1x1TM, kGw1x1TC>), grid, dim3(256), 0, s, gy, x, part, sgpart,
+                           d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, gpr, groups);
+    else
+        hipLaunchKernelGGL((grad_w_1x1_kernel<2, kGw1x1TM, kGw1x1TC>), grid, dim3(256), 0, s, gy, x, part, sgpart,
+                           d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, gpr, groups);
+    return check_launch();
+}
+
+}  // namespace adder

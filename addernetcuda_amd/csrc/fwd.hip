@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 }
 
 // ---------------------------------------------------------------------------
-// Tiled kernel for 3x3, stride 1, pad 1 (Ho = H, Wo = W).
+// Tiled kernel for 3x3, pad 1, stride S = 1 or 2.
 //
 // A workgroup owns NIMG images x a TH x TW patch of output positions and
 // TM*COW output channels.  TW = TN*SPR: each lane owns a strip of TN adjacent
@@ -77,16 +77,16 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 // output channels and sharing the LDS tile.
 //
 // LDS tile: [img][cc][TH+2][PITCH] floats, double buffered over chunks of CC
-// input channels.  Column 0 of a row is input column w0-1, so a lane's strip
-// starts at column strip*TN, which is 16-byte aligned for TN = 4.
+// input channels.  Column 0 of a row is input column w0*S-1, so a lane's strip
+// starts at column strip*TN*S, which is 16-byte aligned when TN*S is a multiple of 4.
 // ---------------------------------------------------------------------------
 template <class C>
-__global__ __launch_bounds__(C::NTHREADS) void fwd_3x3s1_kernel(const float *__restrict__ x,
+__global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__restrict__ x,
                                                                 const float *__restrict__ w,
                                                                 float *__restrict__ y, int N, int Ci,
-                                                                int H, int W, int Co, int tilesH,
-                                                                int tilesW) {
-    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ;
+                                                                int H, int W, int Co, int Ho, int Wo,
+                                                                int tilesH, int tilesW) {
+    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, S = C::S, STRIP = C::STRIP;
     extern __shared__ __align__(16) float smem[];
 
     int b = blockIdx.x;
@@ -119,66 +119,95 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3s1_kernel(const float *__r
 #pragma unroll
         for (int t = 0; t < TN; ++t) acc[m][t] = 0.f;
 
-    const int lane_off = img * C::CC * C::PLANE + row * C::PITCH + strip * TN;
+    const int lane_off = img * C::CC * C::PLANE + row * S * C::PITCH + strip * TN * S;
     const int nchunks = ceil_div(Ci, C::CC);
 
-    TileStage<C> st;
-    tile_fetch<C>(st, x, 0, Ci, n0, N, h0, w0, H, W);
-    tile_commit<C>(st, smem);
+    TileStage<typename C::Patch> st;
+    tile_fetch<typename C::Patch>(st, x, 0, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+    tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int ci0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<C>(st, x, ci0 + C::CC, Ci, n0, N, h0, w0, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Ci - ci0);
-#pragma unroll 1
-        for (int cc = 0; cc < ccnt; cc += CQ) {
-            float xr[CQ][3][TN + 2];
+        // Software pipeline over the input channels of the chunk: the strips of channel
+        // group cc+CQ and the weights of the next output channel are requested right after
+        // the first subtract of the current one, i.e. after the wait for the current
+        // operands and with the rest of the arithmetic still ahead to hide the latency.
+        float xr[2][CQ][3][STRIP];
+        float wv[2][CQ * 9];
 #pragma unroll
-            for (int q = 0; q < CQ; ++q)
+        for (int q = 0; q < CQ; ++q)
 #pragma unroll
-                for (int i = 0; i < 3; ++i)
-                    lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + (cc + q) * C::PLANE + i * C::PITCH, xr[q][i]);
+            for (int i = 0; i < 3; ++i)
+                lds_read_strip<STRIP, C::STRIP_ALIGN>(lbase + q * C::PLANE + i * C::PITCH, xr[0][q][i]);
+#pragma unroll
+        for (int e = 0; e < CQ * 9; ++e) wv[0][e] = wc[wrow[0] + ci0 * 9 + e];
+
+        auto half = [&](const int cc, const int cur) {
+            // cur = 0/1: which xr buffer holds channel group cc
             const int kofs = (ci0 + cc) * 9;
+            const bool more = cc + CQ < ccnt;
+            const int knext = more ? kofs + CQ * 9 : kofs;  // clamped: stays inside the weight row
 #pragma unroll
             for (int m = 0; m < TM; ++m) {
-                float wv[CQ * 9];
 #pragma unroll
-                for (int e = 0; e < CQ * 9; ++e) wv[e] = wc[wrow[m] + kofs + e];
+                for (int idx = 0; idx < CQ * 9 * TN; ++idx) {
+                    const int t = idx % TN, j = (idx / TN) % 3, i = (idx / TN / 3) % 3, q = idx / TN / 9;
+                    acc[m][t] -= fabsf(wv[m & 1][q * 9 + i * 3 + j] - xr[cur][q][i][t * S + j]);
+                    if (idx == 0) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (m + 1 < TM) {
 #pragma unroll
-                for (int q = 0; q < CQ; ++q)
+                            for (int e = 0; e < CQ * 9; ++e) wv[(m + 1) & 1][e] = wc[wrow[m + 1] + kofs + e];
+                        } else {
 #pragma unroll
-                    for (int i = 0; i < 3; ++i)
+                            for (int e = 0; e < CQ * 9; ++e) wv[(m + 1) & 1][e] = wc[wrow[0] + knext + e];
+                        }
+                        if (m == 0 && more) {
 #pragma unroll
-                        for (int j = 0; j < 3; ++j)
+                            for (int q2 = 0; q2 < CQ; ++q2)
 #pragma unroll
-                            for (int t = 0; t < TN; ++t)
-                                acc[m][t] -= fabsf(wv[q * 9 + i * 3 + j] - xr[q][i][t + j]);
+                                for (int i2 = 0; i2 < 3; ++i2)
+                                    lds_read_strip<STRIP, C::STRIP_ALIGN>(
+                                        lbase + (cc + CQ + q2) * C::PLANE + i2 * C::PITCH, xr[cur ^ 1][q2][i2]);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
             }
+        };
+        static_assert(TM % 2 == 0, "weight double buffer assumes an even number of channels per lane");
+#pragma unroll 1
+        for (int cc = 0; cc < ccnt; cc += 2 * CQ) {
+            half(cc, 0);
+            if (cc + CQ < ccnt) half(cc + CQ, 1);
         }
 
-        if (c + 1 < nchunks) tile_commit<C>(st, smem + ((c + 1) & 1) * C::BUF);
+        if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
         __syncthreads();
     }
 
     const int n = n0 + img, ho = h0 + row, wo = w0 + strip * TN;
-    if (lane_ok && n < N && ho < H) {
+    if (lane_ok && n < N && ho < Ho) {
+        const bool vec = TN % 4 == 0 && (Wo & 3) == 0 && wo + TN <= Wo;
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
             const int co = co_base + m;
             if (co < Co) {
-                float *dst = y + (((size_t)n * Co + co) * H + ho) * W + wo;
-                if (TN % 4 == 0 && wo + TN <= W) {
+                float *dst = y + (((size_t)n * Co + co) * Ho + ho) * Wo + wo;
+                if (vec) {
 #pragma unroll
-                    for (int t = 0; t < TN; t += 4)
+                    for (int t = 0; t + 3 < TN; t += 4)
                         *reinterpret_cast<float4 *>(dst + t) =
                             make_float4(acc[m][t], acc[m][t + 1], acc[m][t + 2], acc[m][t + 3]);
                 } else {
 #pragma unroll
                     for (int t = 0; t < TN; ++t)
-                        if (wo + t < W) dst[t] = acc[m][t];
+                        if (wo + t < Wo) dst[t] = acc[m][t];
                 }
             }
         }
@@ -186,36 +215,45 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3s1_kernel(const float *__r
 }
 
 template <class C>
-static int launch_fwd_3x3s1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
-    const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
+static int launch_fwd_3x3(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+    const int tilesH = ceil_div(d.Ho, C::TH), tilesW = ceil_div(d.Wo, C::TW);
     const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gy = ceil_div(d.Co, C::TM * C::COW);
     if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     static bool attr_set = false;
     if (!attr_set && C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3s1_kernel<C>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(fwd_3x3s1_kernel<C>, dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w,
-                       y, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW);
+    hipLaunchKernelGGL(fwd_3x3_kernel<C>, dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
+                       d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
     return check_launch();
 }
 
-//                      TN SPR TH NIMG TM COW CC CQ
-using FwdW32 = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1>;   // 32-wide maps, whole image per workgroup
-using FwdW16 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1>;   // 16-wide maps, one image per workgroup
-using FwdW8  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1>;    // 8-wide maps, one image x 32 channels per workgroup
+// Tile shapes, chosen per output width so that a ResNet-20 layer at batch 256 launches
+// 2048 waves (two per SIMD) and every workgroup reads each input element once.
+//                           TN SPR TH NIMG TM COW CC CQ S
+using FwdW32   = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1, 1>;   // outputs 32 wide: one image, 16 channels
+using FwdW16   = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1, 1>;   // outputs 16 wide: one image, 32 channels
+using FwdW8    = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1, 1>;    // outputs 8 wide: one image, 32 channels
+using FwdW16S2 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 4, 1, 2>;   // stride 2, outputs 16 wide
+using FwdW8S2  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1, 2>;    // stride 2, outputs 8 wide
 
 int launch_fwd(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
-    const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
-    if (k3s1p1 && d.W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-        (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
-        if (d.W > 16) return launch_fwd_3x3s1<FwdW32>(x, w, y, d, s);
-        if (d.W > 8) return launch_fwd_3x3s1<FwdW16>(x, w, y, d, s);
-        return launch_fwd_3x3s1<FwdW8>(x, w, y, d, s);
+    const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.W % 4 == 0 &&
+                      (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    if (k3p1 && d.stride == 1) {
+        if (d.Wo > 16) return launch_fwd_3x3<FwdW32>(x, w, y, d, s);
+        if (d.Wo > 8) return launch_fwd_3x3<FwdW16>(x, w, y, d, s);
+        return launch_fwd_3x3<FwdW8>(x, w, y, d, s);
     }
+    if (k3p1 && d.stride == 2) {
+        if (d.Wo > 8) return launch_fwd_3x3<FwdW16S2>(x, w, y, d, s);
+        return launch_fwd_3x3<FwdW8S2>(x, w, y, d, s);
+    }
+    if (conv1x1_supported(d, x, y)) return launch_fwd_1x1(x, w, y, d, s);
     constexpr int TM = 8;
     const long total = (long)d.N * d.Ho * d.Wo;
     hipLaunchKernelGGL(fwd_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Co, TM)),

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void grad_w_generic_kernel(const float *__rest
 }
 
 // ---------------------------------------------------------------------------
-// Tiled kernel for 3x3, stride 1, pad 1.
+// Tiled kernel for 3x3, pad 1, stride S = 1 or 2.
 //
 // Lanes own output positions (strip of TN in one row).  A wave owns a fixed
 // block of TM output channels x CQ input channels and keeps the TM*CQ*9
@@ -94,12 +94,12 @@ __global__ __launch_bounds__(256) void grad_w_generic_kernel(const float *__rest
 // LDS transpose and writes one partial (Co*K floats per grid.x slot) to the
 // workspace; grad_w_finalize_kernel sums the slots in fp64.
 // ---------------------------------------------------------------------------
-template <int TN_, int SPR_, int TH_, int NIMG_, int TM_, int CQ_, int NCOB_, int NCIB_>
+template <int TN_, int SPR_, int TH_, int NIMG_, int TM_, int CQ_, int NCOB_, int NCIB_, int S_ = 1>
 struct GradWCfg {
     static constexpr int TN = TN_, SPR = SPR_, TH = TH_, NIMG = NIMG_, TM = TM_, CQ = CQ_, NCOB = NCOB_,
-                         NCIB = NCIB_;
+                         NCIB = NCIB_, S = S_;
     static constexpr int COB = TM * NCOB, CIB = CQ * NCIB, NW = NCOB * NCIB;
-    using XT = Tile3x3Cfg<TN, SPR, TH, NIMG, TM, NW, CIB, CQ>;  // haloed x tile, staged by all NW waves
+    using XT = Tile3x3Cfg<TN, SPR, TH, NIMG, TM, NW, CIB, CQ, S>;  // haloed x tile, staged by all NW waves
     static constexpr int TW = XT::TW;
     static constexpr int NTHREADS = XT::NTHREADS;
     static constexpr int GPLANE = TH * TW;
@@ -124,7 +124,7 @@ struct GyStage {
 
 template <class G>
 __device__ __forceinline__ void gy_fetch(GyStage<G> &st, const float *__restrict__ gy, int co0, int Co,
-                                         int n0, int N, int h0, int w0, int H, int W) {
+                                         int n0, int N, int h0, int w0, int Ho, int Wo) {
 #pragma unroll
     for (int it = 0; it < G::GITER; ++it) {
         const int u = threadIdx.x + it * G::NTHREADS;
@@ -133,9 +133,9 @@ __device__ __forceinline__ void gy_fetch(GyStage<G> &st, const float *__restrict
         const int c = (u / (G::TW / 4) / G::TH) % G::COB;
         const int img = u / (G::TW / 4) / G::TH / G::COB;
         const int n = n0 + img, co = co0 + c, ho = h0 + r, wo = w0 + 4 * q;
-        const bool ok = (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) && n < N && co < Co && ho < H && wo < W;
+        const bool ok = (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) && n < N && co < Co && ho < Ho && wo < Wo;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok) val = *reinterpret_cast<const float4 *>(gy + (((size_t)n * Co + co) * H + ho) * W + wo);
+        if (ok) val = *reinterpret_cast<const float4 *>(gy + (((size_t)n * Co + co) * Ho + ho) * Wo + wo);
         st.v[it] = val;
     }
 }
@@ -153,14 +153,14 @@ __device__ __forceinline__ void gy_commit(const GyStage<G> &st, float *buf, floa
 }
 
 template <class G>
-__global__ __launch_bounds__(G::NTHREADS) void grad_w_3x3s1_kernel(const float *__restrict__ gy,
+__global__ __launch_bounds__(G::NTHREADS) void grad_w_3x3_kernel(const float *__restrict__ gy,
                                                                    const float *__restrict__ x,
                                                                    float *__restrict__ part,
                                                                    float *__restrict__ sgpart, int N, int Ci,
-                                                                   int H, int W, int Co, int tilesH,
-                                                                   int tilesW, int ntiles) {
+                                                                   int H, int W, int Co, int Ho, int Wo,
+                                                                   int tilesH, int tilesW, int ntiles) {
     using XT = typename G::XT;
-    constexpr int TN = G::TN, TM = G::TM, CQ = G::CQ;
+    constexpr int TN = G::TN, TM = G::TM, CQ = G::CQ, S = G::S, STRIP = XT::STRIP;
     extern __shared__ __align__(16) float smem[];
 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -181,10 +181,10 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_3x3s1_kernel(const float *
 #pragma unroll
     for (int it = 0; it < G::GITER; ++it) sg[it] = 0.f;
 
-    const int x_off = (img * G::CIB + cib * CQ) * XT::PLANE + row * XT::PITCH + strip * TN;
+    const int x_off = (img * G::CIB + cib * CQ) * XT::PLANE + row * S * XT::PITCH + strip * TN * S;
     const int g_off = XT::BUF + (img * G::COB + cob * TM) * G::GPLANE + row * G::TW + strip * TN;
 
-    TileStage<XT> xs;
+    TileStage<typename XT::Patch> xs;
     GyStage<G> gs;
     int tile = blockIdx.x;
     int n0 = 0, h0 = 0, w0 = 0;
@@ -195,9 +195,9 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_3x3s1_kernel(const float *
     };
     if (tile < ntiles) {
         decode(tile);
-        tile_fetch<XT>(xs, x, ci_blk, Ci, n0, N, h0, w0, H, W);
-        gy_fetch<G>(gs, gy, co_blk, Co, n0, N, h0, w0, H, W);
-        tile_commit<XT>(xs, smem);
+        tile_fetch<typename XT::Patch>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+        gy_fetch<G>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+        tile_commit<typename XT::Patch>(xs, smem);
         gy_commit<G>(gs, smem + XT::BUF, sg);
     }
     __syncthreads();
@@ -207,20 +207,20 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_3x3s1_kernel(const float *
         const int next = tile + gridDim.x;
         if (next < ntiles) {
             decode(next);
-            tile_fetch<XT>(xs, x, ci_blk, Ci, n0, N, h0, w0, H, W);
-            gy_fetch<G>(gs, gy, co_blk, Co, n0, N, h0, w0, H, W);
+            tile_fetch<typename XT::Patch>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+            gy_fetch<G>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         }
         const float *base = smem + cur * G::BUF;
-        float xr[CQ][3][TN + 2];
+        float xr[CQ][3][STRIP];
 #pragma unroll
         for (int q = 0; q < CQ; ++q)
 #pragma unroll
             for (int i = 0; i < 3; ++i)
-                lds_read_strip<TN + 2, XT::STRIP_ALIGN>(base + x_off + q * XT::PLANE + i * XT::PITCH, xr[q][i]);
+                lds_read_strip<STRIP, XT::STRIP_ALIGN>(base + x_off + q * XT::PLANE + i * XT::PITCH, xr[q][i]);
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
             float gr[TN];
-            lds_read_strip<TN, XT::STRIP_ALIGN>(base + g_off + m * G::GPLANE, gr);
+            lds_read_strip<TN, (TN % 4 == 0 ? 4 : (TN % 2 == 0 ? 2 : 1))>(base + g_off + m * G::GPLANE, gr);
 #pragma unroll
             for (int q = 0; q < CQ; ++q)
 #pragma unroll
@@ -229,10 +229,10 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_3x3s1_kernel(const float *
                     for (int j = 0; j < 3; ++j)
 #pragma unroll
                         for (int t = 0; t < TN; ++t)
-                            acc[m][q][i * 3 + j] = fmaf(gr[t], xr[q][i][t + j], acc[m][q][i * 3 + j]);
+                            acc[m][q][i * 3 + j] = fmaf(gr[t], xr[q][i][t * S + j], acc[m][q][i * 3 + j]);
         }
         if (next < ntiles) {
-            tile_commit<XT>(xs, smem + (cur ^ 1) * G::BUF);
+            tile_commit<typename XT::Patch>(xs, smem + (cur ^ 1) * G::BUF);
             gy_commit<G>(gs, smem + (cur ^ 1) * G::BUF + XT::BUF, sg);
         }
         __syncthreads();
@@ -366,20 +366,22 @@ int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStrea
 }
 
 // ---- dispatch -----------------------------------------------------------------
-//                     TN SPR TH NIMG TM CQ NCOB NCIB
-using GwW32 = GradWCfg<4, 8, 8, 1, 8, 2, 2, 4>;
-using GwW16 = GradWCfg<4, 4, 16, 1, 8, 2, 2, 4>;
-using GwW8  = GradWCfg<4, 2, 8, 4, 8, 2, 2, 4>;
+//                     TN SPR TH NIMG TM CQ NCOB NCIB S
+using GwW32   = GradWCfg<4, 8, 8, 1, 8, 2, 2, 4, 1>;
+using GwW16   = GradWCfg<4, 4, 16, 1, 8, 2, 2, 4, 1>;
+using GwW8    = GradWCfg<4, 2, 8, 4, 8, 2, 2, 4, 1>;
+using GwW16S2 = GradWCfg<4, 4, 16, 1, 8, 1, 2, 4, 2>;
+using GwW8S2  = GradWCfg<4, 2, 8, 4, 8, 1, 2, 4, 2>;
 
 struct GradWPlan {
-    int variant;  // 0 generic, 1 W32, 2 W16, 3 W8
+    int variant;  // 0 generic, 1 W32, 2 W16, 3 W8, 4 W16S2, 5 W8S2, 6 1x1
     int slots, gy, gz, tilesH, tilesW, ntiles;
 };
 
 template <class G>
 static void plan_tiled(const ConvDims &d, GradWPlan &p) {
-    p.tilesH = ceil_div(d.H, G::TH);
-    p.tilesW = ceil_div(d.W, G::TW);
+    p.tilesH = ceil_div(d.Ho, G::TH);
+    p.tilesW = ceil_div(d.Wo, G::TW);
     p.ntiles = ceil_div(d.N, G::NIMG) * p.tilesH * p.tilesW;
     p.gy = ceil_div(d.Co, G::COB);
     p.gz = ceil_div(d.Ci, G::CIB);
@@ -392,14 +394,21 @@ static void plan_tiled(const ConvDims &d, GradWPlan &p) {
 
 static GradWPlan plan_grad_w(const ConvDims &d) {
     GradWPlan p{};
-    const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
+    const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.W % 4 == 0 && d.Wo % 4 == 0;
     const long partial_cap = 1L << 28;  // keep the partial buffer below 1 GiB
-    if (k3s1p1 && d.W % 4 == 0) {
-        if (d.W > 16) { p.variant = 1; plan_tiled<GwW32>(d, p); }
-        else if (d.W > 8) { p.variant = 2; plan_tiled<GwW16>(d, p); }
+    if (k3p1 && d.stride == 1) {
+        if (d.Wo > 16) { p.variant = 1; plan_tiled<GwW32>(d, p); }
+        else if (d.Wo > 8) { p.variant = 2; plan_tiled<GwW16>(d, p); }
         else { p.variant = 3; plan_tiled<GwW8>(d, p); }
-        if ((long)p.slots * d.Co * d.K() > partial_cap) p.variant = 0;
+    } else if (k3p1 && d.stride == 2) {
+        if (d.Wo > 8) { p.variant = 4; plan_tiled<GwW16S2>(d, p); }
+        else { p.variant = 5; plan_tiled<GwW8S2>(d, p); }
     }
+    if (!p.variant && conv1x1_supported(d, nullptr, nullptr)) {
+        p.variant = 6;
+        p.slots = grad_w_1x1_slots(d);
+    }
+    if (p.variant && (long)p.slots * d.Co * d.K() > partial_cap) p.variant = 0;
     return p;
 }
 
@@ -415,13 +424,13 @@ static int launch_tiled(const float *gy, const float *x, float *part, float *sgp
                         const GradWPlan &p, hipStream_t s) {
     static bool attr_set = false;
     if (!attr_set && G::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_3x3s1_kernel<G>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_3x3_kernel<G>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(grad_w_3x3s1_kernel<G>, dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy,
-                       x, part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, p.tilesH, p.tilesW, p.ntiles);
+    hipLaunchKernelGGL(grad_w_3x3_kernel<G>, dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy,
+                       x, part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles);
     return check_launch();
 }
 
@@ -437,9 +446,14 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
         float *part = reinterpret_cast<float *>(ss + kNormBlocksMax);
         float *sgpart = part + (size_t)p.slots * d.Co * K;
         int rc;
-        if (p.variant == 1) rc = launch_tiled<GwW32>(gy, x, part, sgpart, d, p, s);
-        else if (p.variant == 2) rc = launch_tiled<GwW16>(gy, x, part, sgpart, d, p, s);
-        else rc = launch_tiled<GwW8>(gy, x, part, sgpart, d, p, s);
+        switch (p.variant) {
+            case 1: rc = launch_tiled<GwW32>(gy, x, part, sgpart, d, p, s); break;
+            case 2: rc = launch_tiled<GwW16>(gy, x, part, sgpart, d, p, s); break;
+            case 3: rc = launch_tiled<GwW8>(gy, x, part, sgpart, d, p, s); break;
+            case 4: rc = launch_tiled<GwW16S2>(gy, x, part, sgpart, d, p, s); break;
+            case 6: rc = launch_grad_w_1x1(gy, x, part, sgpart, p.slots, d, s); break;
+            default: rc = launch_tiled<GwW8S2>(gy, x, part, sgpart, d, p, s); break;
+        }
         if (rc) return rc;
         const int nb = (int)ceil_div_l(n, 256);
         const bool fused_norm = eta > 0.f && nb <= kNormBlocksMax;

@@ -128,14 +128,14 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     const int lane_off = img * C::CC * C::PLANE + row * C::PITCH + strip * TN;
     const int nchunks = ceil_div(Co, C::CC);
 
-    TileStage<C> st;
-    tile_fetch<C>(st, gy, 0, Co, n0, N, h0, w0, H, W);
-    tile_commit<C>(st, smem);
+    TileStage<typename C::Patch> st;
+    tile_fetch<typename C::Patch>(st, gy, 0, Co, n0, N, h0 - 1, w0, H, W);
+    tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int co0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<C>(st, gy, co0 + C::CC, Co, n0, N, h0, w0, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch>(st, gy, co0 + C::CC, Co, n0, N, h0 - 1, w0, H, W);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
             }
         }
 
-        if (c + 1 < nchunks) tile_commit<C>(st, smem + ((c + 1) & 1) * C::BUF);
+        if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
         __syncthreads();
     }
 
@@ -211,6 +211,165 @@ static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, 
     return check_launch();
 }
 
+// ---------------------------------------------------------------------------
+// Tiled kernel for 3x3, stride 2, pad 1.
+//
+// With stride 2 only taps of matching parity reach an input position:
+//   even row 2a   : i = 1 -> ho = a            odd row 2a+1 : i = 0 -> ho = a+1, i = 2 -> ho = a
+// and likewise for columns, so a 2 x 2 block of input positions sees the 9
+// taps exactly once between its four members.  A lane owns 2 rows x TNW
+// columns (TNW even) x TM input channels; the gy patch it needs is rows
+// a, a+1 and columns b .. b+TNW/2 of the output (halo on the bottom / right
+// only, zero beyond the output).
+// ---------------------------------------------------------------------------
+template <int TNW_, int BPR_, int TH_, int NIMG_, int TM_, int CIW_, int CC_>
+struct GradX3x3S2Cfg {
+    static constexpr int TNW = TNW_, BPR = BPR_, TH = TH_, NIMG = NIMG_, TM = TM_, CIW = CIW_, CC = CC_;
+    static constexpr int TW = TNW * BPR;
+    static constexpr int LANES = NIMG * (TH / 2) * BPR;
+    static constexpr int POSW = ceil_div(LANES, 64);
+    static constexpr int NTHREADS = 64 * POSW * CIW;
+    using Patch = PatchCfg<NIMG, CC, TH / 2 + 1, TW / 2, 0, 1, NTHREADS>;
+    static constexpr int PITCH = Patch::PITCH, PLANE = Patch::PLANE, BUF = Patch::BUF;
+    static constexpr int LDS_BYTES = 2 * BUF * 4;
+    static constexpr int GSTRIP = TNW / 2 + 1;
+    static_assert(TNW % 2 == 0 && TH % 2 == 0, "lanes own 2 x 2 parity blocks");
+};
+
+template <class C>
+__global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *__restrict__ gy,
+                                                                   const float *__restrict__ x,
+                                                                   const float *__restrict__ w,
+                                                                   float *__restrict__ gx, int N, int Ci,
+                                                                   int H, int W, int Co, int Ho, int Wo,
+                                                                   int tilesH, int tilesW) {
+    constexpr int TNW = C::TNW, TM = C::TM, GSTRIP = C::GSTRIP;
+    extern __shared__ __align__(16) float smem[];
+
+    int b = blockIdx.x;
+    const int tw = b % tilesW; b /= tilesW;
+    const int th = b % tilesH; b /= tilesH;
+    const int n0 = b * C::NIMG;
+    const int h0 = th * C::TH, w0 = tw * C::TW;  // both even
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int pw = wave % C::POSW, cw = wave / C::POSW;
+    int p = pw * 64 + lane;
+    const bool lane_ok = p < C::LANES;
+    if (!lane_ok) p = C::LANES - 1;
+    const int bcol = p % C::BPR;
+    const int brow = (p / C::BPR) % (C::TH / 2);
+    const int img = p / (C::BPR * (C::TH / 2));
+    const int ci_base = (blockIdx.y * C::CIW + cw) * TM;
+    const int K = Ci * 9;
+    uniform_f32_ptr wc = as_uniform(w);
+
+    const int n = n0 + img, hi0 = h0 + 2 * brow, wi0 = w0 + bcol * TNW;
+    const int nc = min(n, N - 1);
+
+    float xr[TM][2][TNW], acc[TM][2][TNW];
+    int wofs[TM];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) {
+        const int ci = min(ci_base + m, Ci - 1);
+        wofs[m] = __builtin_amdgcn_readfirstlane(ci * 9);
+#pragma unroll
+        for (int rp = 0; rp < 2; ++rp) {
+            const float *src = x + (((size_t)nc * Ci + ci) * H + min(hi0 + rp, H - 1)) * W;
+#pragma unroll
+            for (int t = 0; t < TNW; ++t) {
+                xr[m][rp][t] = src[min(wi0 + t, W - 1)];
+                acc[m][rp][t] = 0.f;
+            }
+        }
+    }
+
+    const int lane_off = img * C::CC * C::PLANE + brow * C::PITCH + bcol * (TNW / 2);
+    const int nchunks = ceil_div(Co, C::CC);
+    const int hb = h0 / 2, wb = w0 / 2;
+
+    TileStage<typename C::Patch> st;
+    tile_fetch<typename C::Patch>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
+    tile_commit<typename C::Patch>(st, smem);
+    __syncthreads();
+
+    for (int c = 0; c < nchunks; ++c) {
+        const int co0 = c * C::CC;
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch>(st, gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
+
+        const float *lbase = smem + (c & 1) * C::BUF + lane_off;
+        const int ccnt = min(C::CC, Co - co0);
+#pragma unroll 1
+        for (int cc = 0; cc < ccnt; ++cc) {
+            float gr[2][GSTRIP];
+#pragma unroll
+            for (int r = 0; r < 2; ++r) lds_read_strip<GSTRIP, 1>(lbase + cc * C::PLANE + r * C::PITCH, gr[r]);
+            const int kofs = (co0 + cc) * K;
+#pragma unroll
+            for (int m = 0; m < TM; ++m) {
+                float wv[9];
+#pragma unroll
+                for (int e = 0; e < 9; ++e) wv[e] = wc[kofs + wofs[m] + e];
+                // (row parity, tap row i, gy row) and (col parity, tap col j, gy col offset)
+                constexpr int RP[3] = {0, 1, 1}, RI[3] = {1, 0, 2}, RG[3] = {0, 1, 0};
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+#pragma unroll
+                    for (int bb = 0; bb < 3; ++bb)
+#pragma unroll
+                        for (int cp = 0; cp < TNW / 2; ++cp) {
+                            const int t = 2 * cp + RP[bb];
+                            acc[m][RP[a]][t] = fmaf(hardtanh(wv[RI[a] * 3 + RI[bb]] - xr[m][RP[a]][t]),
+                                                    gr[RG[a]][cp + RG[bb]], acc[m][RP[a]][t]);
+                        }
+            }
+        }
+
+        if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
+        __syncthreads();
+    }
+
+    if (lane_ok && n < N) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const int ci = ci_base + m;
+            if (ci >= Ci) continue;
+#pragma unroll
+            for (int rp = 0; rp < 2; ++rp) {
+                const int hi = hi0 + rp;
+                if (hi >= H) continue;
+                float *dst = gx + (((size_t)n * Ci + ci) * H + hi) * W + wi0;
+                if ((W & 1) == 0 && wi0 + TNW <= W) {
+#pragma unroll
+                    for (int t = 0; t < TNW; t += 2)
+                        *reinterpret_cast<float2 *>(dst + t) = make_float2(acc[m][rp][t], acc[m][rp][t + 1]);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < TNW; ++t)
+                        if (wi0 + t < W) dst[t] = acc[m][rp][t];
+                }
+            }
+        }
+    }
+}
+
+template <class C>
+static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, float *gx,
+                               const ConvDims &d, hipStream_t s) {
+    const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
+    const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
+    const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
+    if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
+    static_assert(C::LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
+    hipLaunchKernelGGL(grad_x_3x3s2_kernel<C>, dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
+                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
+    return check_launch();
+}
+
+//                              TNW BPR TH NIMG TM CIW CC
+using GxS2W32 = GradX3x3S2Cfg<2, 16, 32, 1, 8, 2, 8>;   // inputs 32 wide
+using GxS2W16 = GradX3x3S2Cfg<2, 8, 16, 1, 8, 4, 8>;    // inputs 16 wide
+
 //                        TN SPR TH NIMG TM COW CC CQ
 using GxW32 = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1>;
 using GxW16 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1>;
@@ -225,6 +384,13 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s);
     }
+    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.Wo % 4 == 0 && d.W % 2 == 0 &&
+        (reinterpret_cast<uintptr_t>(gy) & 15) == 0 && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
+        if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);
+        return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s);
+    }
+    if (conv1x1_supported(d, gy, gx) && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
+        return launch_grad_x_1x1(gy, x, w, gx, d, s);
     constexpr int TM = 8;
     const long total = (long)d.N * d.H * d.W;
     hipLaunchKernelGGL(grad_x_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Ci, TM)),

@@ -1,100 +1,126 @@
-// Tile geometry and global->LDS staging shared by the 3x3 / stride-1 / pad-1
-// forward and input-gradient kernels.  Both stage a haloed (TH+2) x (TW+2)
-// patch of some NCHW tensor per channel, zero-filled outside the image (the
-// forward's padding taps are x = 0; the input gradient's out-of-range output
-// positions contribute nothing).
+// Tile geometry and global->LDS staging shared by the tiled 3x3 / pad-1 kernels
+// (stride 1 or 2).  A workgroup covers NIMG images x TH x TW positions of the
+// "lane space" (output positions for the forward and weight-gradient kernels,
+// input positions for the stride-1 input gradient) and stages, per channel, the
+// haloed patch of the source tensor those positions touch:
+//   rows  h0*S-1 .. h0*S-1 + (TH-1)*S+2,   columns  w0*S-1 .. w0*S-1 + (TW-1)*S+2,
+// zero-filled outside the tensor.  (For the forward the zeros are the padding
+// taps, x = 0; for the input gradient they are output positions that do not
+// exist and must contribute nothing.)
 #pragma once
 #include "common.hpp"
 
 namespace adder {
 
-template <int TN_, int SPR_, int TH_, int NIMG_, int TM_, int COW_, int CC_, int CQ_>
-struct Tile3x3Cfg {
-    static constexpr int TN = TN_, SPR = SPR_, TH = TH_, NIMG = NIMG_, TM = TM_, COW = COW_,
-                         CC = CC_, CQ = CQ_;
-    static constexpr int TW = TN * SPR;
-    static constexpr int LANES = NIMG * TH * SPR;
-    static constexpr int POSW = ceil_div(LANES, 64);
-    static constexpr int NTHREADS = 64 * POSW * COW;
-    static constexpr int PITCH = round_up(TW + 2, 4);
-    static constexpr int ROWS = TH + 2;
+// A rectangular patch of an NCHW tensor staged per channel into LDS as
+// [img][cc][ROWS][PITCH]: ICOLS float4-aligned interior columns starting at LDS
+// column LHALO, plus an optional single halo column on either side.
+template <int NIMG_, int CC_, int ROWS_, int ICOLS_, int LHALO_, int RHALO_, int NTHREADS_>
+struct PatchCfg {
+    static constexpr int NIMG = NIMG_, CC = CC_, ROWS = ROWS_, ICOLS = ICOLS_, LHALO = LHALO_, RHALO = RHALO_,
+                         NTHREADS = NTHREADS_;
+    static constexpr int PITCH = round_up(LHALO + ICOLS + RHALO, 4);
     static constexpr int PLANE = ROWS * PITCH;
     static constexpr int BUF = NIMG * CC * PLANE;  // floats per buffer
-    static constexpr int LDS_BYTES = 2 * BUF * 4;
-    static constexpr int STRIP_ALIGN = (TN % 4 == 0) ? 4 : (TN % 2 == 0 ? 2 : 1);
-    // global -> LDS staging: interior as float4 units, halo columns as scalars
-    static constexpr int NUV = NIMG * CC * ROWS * (TW / 4);
+    static constexpr int NUV = NIMG * CC * ROWS * (ICOLS / 4);
     static constexpr int VITER = ceil_div(NUV, NTHREADS);
-    static constexpr int NUH = NIMG * CC * ROWS * 2;
-    static constexpr int HITER = ceil_div(NUH, NTHREADS);
-    static_assert(TW % 4 == 0, "tile width must be a multiple of 4");
-    static_assert(CC % CQ == 0, "CC must be a multiple of CQ");
+    static constexpr int NSIDES = LHALO + RHALO;
+    static constexpr int NUH = NIMG * CC * ROWS * NSIDES;
+    static constexpr int HITER = NSIDES ? ceil_div(NUH, NTHREADS) : 0;
+    static_assert(ICOLS % 4 == 0, "interior must cover whole float4 groups of the source");
+    static_assert(LHALO == 0 || LHALO == 1, "at most one halo column per side");
+    static_assert(RHALO == 0 || RHALO == 1, "at most one halo column per side");
 };
 
-template <class C>
+template <class P>
 struct TileStage {
-    float4 v[C::VITER];
-    float h[C::HITER];
+    float4 v[P::VITER];
+    float h[P::HITER > 0 ? P::HITER : 1];
 };
 
-// Issue the global loads of one channel chunk into registers.
-template <class C>
-__device__ __forceinline__ void tile_fetch(TileStage<C> &st, const float *__restrict__ src,
-                                           int chan0, int nchan, int n0, int nimg_total, int h0,
-                                           int w0, int H, int W) {
-    // src is (nimg_total, nchan, H, W); the tile covers rows h0-1.., cols w0-1..
+// Issue the global loads of one channel chunk into registers.  src is
+// (nimg_total, nchan, H, W); (hb, wb) is the source position of the first
+// interior element of the patch.  Everything outside the tensor reads as zero.
+template <class P>
+__device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__restrict__ src,
+                                           int chan0, int nchan, int n0, int nimg_total, int hb,
+                                           int wb, int H, int W) {
     const int tid = threadIdx.x;
 #pragma unroll
-    for (int it = 0; it < C::VITER; ++it) {
-        const int u = tid + it * C::NTHREADS;
-        const int q = u % (C::TW / 4);
-        const int r = (u / (C::TW / 4)) % C::ROWS;
-        const int cc = (u / (C::TW / 4) / C::ROWS) % C::CC;
-        const int img = u / (C::TW / 4) / C::ROWS / C::CC;
-        const int n = n0 + img, ch = chan0 + cc, hi = h0 - 1 + r, wi = w0 + 4 * q;
-        const bool ok = (C::NUV % C::NTHREADS == 0 || u < C::NUV) && n < nimg_total && ch < nchan &&
+    for (int it = 0; it < P::VITER; ++it) {
+        const int u = tid + it * P::NTHREADS;
+        const int q = u % (P::ICOLS / 4);
+        const int r = (u / (P::ICOLS / 4)) % P::ROWS;
+        const int cc = (u / (P::ICOLS / 4) / P::ROWS) % P::CC;
+        const int img = u / (P::ICOLS / 4) / P::ROWS / P::CC;
+        const int n = n0 + img, ch = chan0 + cc, hi = hb + r, wi = wb + 4 * q;
+        const bool ok = (P::NUV % P::NTHREADS == 0 || u < P::NUV) && n < nimg_total && ch < nchan &&
                         hi >= 0 && hi < H && wi < W;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok) val = *reinterpret_cast<const float4 *>(src + (((size_t)n * nchan + ch) * H + hi) * W + wi);
         st.v[it] = val;
     }
 #pragma unroll
-    for (int it = 0; it < C::HITER; ++it) {
-        const int u = tid + it * C::NTHREADS;
-        const int side = u & 1;
-        const int r = (u >> 1) % C::ROWS;
-        const int cc = (u >> 1) / C::ROWS % C::CC;
-        const int img = (u >> 1) / C::ROWS / C::CC;
-        const int n = n0 + img, ch = chan0 + cc, hi = h0 - 1 + r, wi = side ? w0 + C::TW : w0 - 1;
-        const bool ok = (C::NUH % C::NTHREADS == 0 || u < C::NUH) && n < nimg_total && ch < nchan &&
+    for (int it = 0; it < P::HITER; ++it) {
+        const int u = tid + it * P::NTHREADS;
+        const int side = P::LHALO ? u % P::NSIDES : 1;  // 0 = left, 1 = right
+        const int rest = u / P::NSIDES;
+        const int r = rest % P::ROWS;
+        const int cc = rest / P::ROWS % P::CC;
+        const int img = rest / P::ROWS / P::CC;
+        const int n = n0 + img, ch = chan0 + cc, hi = hb + r, wi = side ? wb + P::ICOLS : wb - 1;
+        const bool ok = (P::NUH % P::NTHREADS == 0 || u < P::NUH) && n < nimg_total && ch < nchan &&
                         hi >= 0 && hi < H && wi >= 0 && wi < W;
         st.h[it] = ok ? src[(((size_t)n * nchan + ch) * H + hi) * W + wi] : 0.f;
     }
 }
 
 // Write the staged chunk into one LDS buffer.
-template <class C>
-__device__ __forceinline__ void tile_commit(const TileStage<C> &st, float *buf) {
+template <class P>
+__device__ __forceinline__ void tile_commit(const TileStage<P> &st, float *buf) {
     const int tid = threadIdx.x;
 #pragma unroll
-    for (int it = 0; it < C::VITER; ++it) {
-        const int u = tid + it * C::NTHREADS;
-        if (C::NUV % C::NTHREADS == 0 || u < C::NUV) {
-            const int q = u % (C::TW / 4);
-            const int rest = u / (C::TW / 4);  // = (img*CC + cc)*ROWS + r
-            float *dst = buf + rest * C::PITCH + 1 + 4 * q;
-            dst[0] = st.v[it].x; dst[1] = st.v[it].y; dst[2] = st.v[it].z; dst[3] = st.v[it].w;
+    for (int it = 0; it < P::VITER; ++it) {
+        const int u = tid + it * P::NTHREADS;
+        if (P::NUV % P::NTHREADS == 0 || u < P::NUV) {
+            const int q = u % (P::ICOLS / 4);
+            const int rest = u / (P::ICOLS / 4);  // = (img*CC + cc)*ROWS + r
+            float *dst = buf + rest * P::PITCH + P::LHALO + 4 * q;
+            if (P::LHALO == 0) {
+                *reinterpret_cast<float4 *>(dst) = st.v[it];
+            } else {
+                dst[0] = st.v[it].x; dst[1] = st.v[it].y; dst[2] = st.v[it].z; dst[3] = st.v[it].w;
+            }
         }
     }
 #pragma unroll
-    for (int it = 0; it < C::HITER; ++it) {
-        const int u = tid + it * C::NTHREADS;
-        if (C::NUH % C::NTHREADS == 0 || u < C::NUH) {
-            const int side = u & 1;
-            const int rest = u >> 1;
-            buf[rest * C::PITCH + (side ? C::TW + 1 : 0)] = st.h[it];
+    for (int it = 0; it < P::HITER; ++it) {
+        const int u = tid + it * P::NTHREADS;
+        if (P::NUH % P::NTHREADS == 0 || u < P::NUH) {
+            const int side = P::LHALO ? u % P::NSIDES : 1;
+            const int rest = u / P::NSIDES;
+            buf[rest * P::PITCH + (side ? P::LHALO + P::ICOLS : 0)] = st.h[it];
         }
     }
 }
+
+// Geometry of the tiled 3x3 / pad-1 kernels (see the header comment).
+template <int TN_, int SPR_, int TH_, int NIMG_, int TM_, int COW_, int CC_, int CQ_, int S_ = 1>
+struct Tile3x3Cfg {
+    static constexpr int TN = TN_, SPR = SPR_, TH = TH_, NIMG = NIMG_, TM = TM_, COW = COW_,
+                         CC = CC_, CQ = CQ_, S = S_;
+    static constexpr int TW = TN * SPR;
+    static constexpr int LANES = NIMG * TH * SPR;
+    static constexpr int POSW = ceil_div(LANES, 64);
+    static constexpr int NTHREADS = 64 * POSW * COW;
+    // stride 2 never reads past the interior on the right
+    using Patch = PatchCfg<NIMG, CC, (TH - 1) * S + 3, TW * S, 1, (S == 1) ? 1 : 0, NTHREADS>;
+    static constexpr int PITCH = Patch::PITCH, PLANE = Patch::PLANE, BUF = Patch::BUF;
+    static constexpr int LDS_BYTES = 2 * BUF * 4;
+    static constexpr int STRIP = (TN - 1) * S + 3;  // floats a lane reads per tile row
+    static constexpr int STRIP_ALIGN = ((TN * S) % 4 == 0) ? 4 : ((TN * S) % 2 == 0 ? 2 : 1);
+    static_assert(S == 1 || S == 2, "stride 1 or 2");
+    static_assert(CC % CQ == 0, "CC must be a multiple of CQ");
+};
 
 }  // namespace adder

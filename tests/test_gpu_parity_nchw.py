@@ -21,11 +21,20 @@ TILED = [
     (1, 3, 9, 40, 4, 3, 1, 1),      # two tiles along W
     (2, 12, 8, 8, 12, 3, 1, 1),     # DenseNet-style 12 channels
     (1, 24, 4, 4, 48, 3, 1, 1),     # map smaller than a tile
+    (2, 16, 32, 32, 32, 3, 2, 1),   # ResNet-20 strided 3x3, 32 -> 16
+    (3, 32, 16, 16, 64, 3, 2, 1),   # ResNet-20 strided 3x3, 16 -> 8
+    (2, 6, 14, 24, 10, 3, 2, 1),    # strided, channel tails, partial tiles (Ho = 7, Wo = 12)
+    (2, 5, 12, 20, 7, 3, 2, 1),     # strided, Wo = 10 (forward tiled, gradients generic)
+    (2, 16, 32, 32, 32, 1, 2, 0),   # ResNet-20 1x1 stride-2 downsample
+    (2, 32, 16, 16, 64, 1, 2, 0),   # second downsample
+    (2, 8, 8, 8, 16, 1, 1, 0),      # 1x1 stride 1
+    (3, 13, 12, 12, 9, 1, 2, 0),    # 1x1 stride 2 with channel tails
+    (2, 9, 6, 12, 20, 1, 1, 0),     # 1x1 stride 1 with channel tails
 ]
 GENERIC = [
-    (2, 16, 32, 32, 32, 3, 2, 1),   # ResNet-20 strided 3x3
-    (2, 16, 32, 32, 32, 1, 2, 0),   # ResNet-20 1x1 stride-2 downsample
-    (2, 8, 7, 7, 16, 1, 1, 0),      # 1x1
+    (2, 8, 7, 7, 16, 1, 1, 0),      # 1x1, W % 4 != 0
+    (2, 4, 9, 9, 6, 3, 2, 1),       # strided 3x3, odd size
+    (2, 4, 9, 9, 6, 1, 2, 0),       # strided 1x1, odd size
     (2, 3, 7, 7, 5, 3, 1, 1),       # W % 4 != 0
     (1, 4, 11, 9, 6, 5, 1, 2),      # 5x5
     (2, 3, 11, 9, 4, 3, 3, 2),      # stride 3, floor output size
