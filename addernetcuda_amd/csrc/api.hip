@@ -3,6 +3,7 @@
 // exercised on a machine without a GPU.
 #include "common.hpp"
 
+#include <cstdlib>
 #include <string>
 
 namespace adder {
@@ -17,6 +18,12 @@ int record_hip_error(hipError_t e) {
 int check_launch() {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? ADDER_OK : record_hip_error(e);
+}
+
+int tune_knob(const char *name, int dflt) {
+    const std::string key = std::string("ADDERNET_") + name;
+    const char *v = std::getenv(key.c_str());
+    return v ? std::atoi(v) : dflt;
 }
 
 static const long kMaxElems = 0x7fffffffL;

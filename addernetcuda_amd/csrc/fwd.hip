@@ -232,26 +232,37 @@ static int launch_fwd_3x3(const float *x, const float *w, float *y, const ConvDi
     return check_launch();
 }
 
-// Tile shapes, chosen per output width so that a ResNet-20 layer at batch 256 launches
-// 2048 waves (two per SIMD) and every workgroup reads each input element once.
+// Tile shapes per output width.  They are chosen so that (i) a ResNet-20 layer at batch 256
+// launches >= 2048 waves, (ii) one pipeline unit (one output channel x CQ input channels) has
+// enough vector instructions (18*CQ*TN) to cover a scalar-cache miss, and (iii) the two weight
+// buffers (18*CQ SGPRs) stay far from the 102-SGPR limit: spilled SGPRs come back as
+// v_readlane, i.e. as vector instructions inside the hot loop.
 //                           TN SPR TH NIMG TM COW CC CQ S
-using FwdW32   = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1, 1>;   // outputs 32 wide: one image, 16 channels
-using FwdW16   = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1, 1>;   // outputs 16 wide: one image, 32 channels
-using FwdW8    = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1, 1>;    // outputs 8 wide: one image, 32 channels
-using FwdW16S2 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 4, 1, 2>;   // stride 2, outputs 16 wide
-using FwdW8S2  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1, 2>;    // stride 2, outputs 8 wide
+using FwdW32   = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 2, 1>;    // outputs 32 wide: one image x 16 channels
+using FwdW16   = Tile3x3Cfg<2, 8, 16, 1, 4, 8, 16, 2, 1>;   // outputs 16 wide: one image x 32 channels
+using FwdW8    = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 2, 1>;    // outputs 8 wide: two images x 32 channels
+using FwdW16S2 = Tile3x3Cfg<2, 8, 16, 1, 4, 8, 8, 2, 2>;    // stride 2, outputs 16 wide
+using FwdW8S2  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 2, 2>;    // stride 2, outputs 8 wide
+// same tiles with one input channel per unit, for odd channel counts
+using FwdW32o   = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1, 1>;
+using FwdW16o   = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 16, 1, 1>;
+using FwdW8o    = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1, 1>;
+using FwdW16S2o = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1, 2>;
+using FwdW8S2o  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1, 2>;
 
 int launch_fwd(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
     const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.W % 4 == 0 &&
                       (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const bool even = d.Ci % 2 == 0;
     if (k3p1 && d.stride == 1) {
-        if (d.Wo > 16) return launch_fwd_3x3<FwdW32>(x, w, y, d, s);
-        if (d.Wo > 8) return launch_fwd_3x3<FwdW16>(x, w, y, d, s);
-        return launch_fwd_3x3<FwdW8>(x, w, y, d, s);
+        if (d.Wo > 16) return even ? launch_fwd_3x3<FwdW32>(x, w, y, d, s) : launch_fwd_3x3<FwdW32o>(x, w, y, d, s);
+        if (d.Wo > 8) return even ? launch_fwd_3x3<FwdW16>(x, w, y, d, s) : launch_fwd_3x3<FwdW16o>(x, w, y, d, s);
+        return even ? launch_fwd_3x3<FwdW8>(x, w, y, d, s) : launch_fwd_3x3<FwdW8o>(x, w, y, d, s);
     }
     if (k3p1 && d.stride == 2) {
-        if (d.Wo > 8) return launch_fwd_3x3<FwdW16S2>(x, w, y, d, s);
-        return launch_fwd_3x3<FwdW8S2>(x, w, y, d, s);
+        if (d.Wo > 8)
+            return even ? launch_fwd_3x3<FwdW16S2>(x, w, y, d, s) : launch_fwd_3x3<FwdW16S2o>(x, w, y, d, s);
+        return even ? launch_fwd_3x3<FwdW8S2>(x, w, y, d, s) : launch_fwd_3x3<FwdW8S2o>(x, w, y, d, s);
     }
     if (conv1x1_supported(d, x, y)) return launch_fwd_1x1(x, w, y, d, s);
     constexpr int TM = 8;

@@ -14,7 +14,7 @@
 
 namespace adder {
 
-static constexpr int kNormBlocksMax = 1024;  // sum-of-squares partials kept at the head of the workspace
+static constexpr int kNormBlocksMax = 4096;  // sum-of-squares partials kept at the head of the workspace
 
 // ---------------------------------------------------------------------------
 // Generic kernel: one workgroup per (co, ci) [KH x KW taps in registers] or,
@@ -287,30 +287,43 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_3x3_kernel(const float *__
 }
 
 // gw = sum_slots part - w * sum_slots sgpart ; per-block sum of squares for the norm when ss != NULL.
+// A workgroup finishes 16 outputs: thread (sl, o) adds slots sl, sl+16, ... of output o in fp64, so the
+// dependent chain is slots/16 long and every 16-lane group reads 64 contiguous bytes.
+static constexpr int kFinOut = 16;
 __global__ __launch_bounds__(256) void grad_w_finalize_kernel(const float *__restrict__ part,
                                                               const float *__restrict__ sgpart,
                                                               const float *__restrict__ w,
                                                               float *__restrict__ gw, double *__restrict__ ss,
                                                               int slots, int Co, int K) {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
+    const int o = threadIdx.x & 15, sl = threadIdx.x >> 4;
     const int total = Co * K;
-    double v = 0.0;
-    if (idx < total) {
-        const int co = idx / K;
-        double a = 0.0, sgs = 0.0;
-        for (int p = 0; p < slots; ++p) {
-            a += (double)part[(size_t)p * total + idx];
-            sgs += (double)sgpart[(size_t)p * Co + co];
-        }
-        const float r = (float)(a - (double)w[idx] * sgs);
-        gw[idx] = r;
-        v = (double)r * (double)r;
+    const int idx = blockIdx.x * kFinOut + o;
+    const int idc = idx < total ? idx : total - 1;
+    const int co = idc / K;
+    double a = 0.0, sgs = 0.0;
+    for (int p = sl; p < slots; p += 16) {
+        a += (double)part[(size_t)p * total + idc];
+        sgs += (double)sgpart[(size_t)p * Co + co];
     }
-    __shared__ double red[4];
-    v = wave_sum(v);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __shared__ double ra[16][kFinOut + 1], rs[16][kFinOut + 1];
+    ra[sl][o] = a;
+    rs[sl][o] = sgs;
     __syncthreads();
-    if (threadIdx.x == 0 && ss) ss[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+    if (threadIdx.x < kFinOut) {
+        double ta = 0.0, ts = 0.0;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) { ta += ra[k][o]; ts += rs[k][o]; }
+        double v = 0.0;
+        if (idx < total) {
+            const float r = (float)(ta - (double)w[idx] * ts);
+            gw[idx] = r;
+            v = (double)r * (double)r;
+        }
+        // lanes 0..15 of wave 0 hold the squares
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+        if (threadIdx.x == 0 && ss) ss[blockIdx.x] = v;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -455,12 +468,13 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
             default: rc = launch_tiled<GwW8S2>(gy, x, part, sgpart, d, p, s); break;
         }
         if (rc) return rc;
-        const int nb = (int)ceil_div_l(n, 256);
+        const int nb = (int)ceil_div_l(n, kFinOut);
         const bool fused_norm = eta > 0.f && nb <= kNormBlocksMax;
         hipLaunchKernelGGL(grad_w_finalize_kernel, dim3(nb), dim3(256), 0, s, part, sgpart, w, gw,
                            fused_norm ? ss : nullptr, p.slots, d.Co, K);
         if (fused_norm)
-            hipLaunchKernelGGL(norm_scale_kernel, dim3(nb), dim3(256), 0, s, gw, n, ss, nb, eta, 1e-12f);
+            hipLaunchKernelGGL(norm_scale_kernel, dim3(norm_blocks(n)), dim3(256), 0, s, gw, n, ss, nb, eta,
+                               1e-12f);
         rc = check_launch();
         if (rc || fused_norm || !(eta > 0.f)) return rc;
         return launch_norm_scale(gw, n, eta, 1e-12f, ws, s);

@@ -102,9 +102,13 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     const int strip = p % C::SPR;
     const int row = (p / C::SPR) % C::TH;
     const int img = p / (C::SPR * C::TH);
-    const int ci_base = (blockIdx.y * C::COW + cw) * TM;
+    // The last channel group is shifted down to end at Ci (Ci >= TM is a launch precondition) so
+    // that the TM channels of a wave are always valid and their weights contiguous; channels
+    // below ci_first belong to the previous group and are not stored.
+    const int ci_first = (blockIdx.y * C::COW + cw) * TM;
+    const int ci_base = __builtin_amdgcn_readfirstlane(min(ci_first, Ci - TM));
     const int K = Ci * 9;
-    uniform_f32_ptr wc = as_uniform(w);
+    uniform_f32_ptr wc = as_uniform(w) + ci_base * 9;
 
     const int n = n0 + img, hi = h0 + row, wi0 = w0 + strip * TN;
     const bool pos_ok = lane_ok && n < N && hi < H;
@@ -112,11 +116,9 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
 
     // own x values and accumulators live in registers for the whole kernel
     float xr[TM][TN], acc[TM][TN];
-    int wofs[TM];
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
-        const int ci = min(ci_base + m, Ci - 1);
-        wofs[m] = __builtin_amdgcn_readfirstlane(ci * 9);
+        const int ci = ci_base + m;
         const float *src = x + (((size_t)nc * Ci + ci) * H + hc) * W;
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
@@ -139,32 +141,58 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
-#pragma unroll 1
-        for (int cc = 0; cc < ccnt; cc += CQ) {
-            float gr[CQ][3][TN + 2];
+        // Software pipeline over the output channels of the chunk, in units of HM input channels
+        // (9*HM contiguous weights): right after the first instruction of a unit, i.e. after the
+        // wait for its operands, the weights of the next unit and (once per output channel) the
+        // gy strips of the next channel are requested.
+        static_assert(CQ == 1, "pipeline is written for one output channel per step");
+        // input channels per unit: keeps ~100 vector instructions per unit and both weight
+        // buffers (2 * 9 * HM SGPRs) well inside the scalar register file
+        constexpr int HM = TN >= 4 ? 1 : 2, NU = TM / HM, HW = HM * 9;
+        static_assert(TM % HM == 0 && NU % 2 == 0, "even number of units per output channel");
+        float gr[2][3][TN + 2];
+        float wv[2][HW];
 #pragma unroll
-            for (int q = 0; q < CQ; ++q)
+        for (int i = 0; i < 3; ++i) lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + i * C::PITCH, gr[0][i]);
 #pragma unroll
-                for (int i = 0; i < 3; ++i)
-                    lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + (cc + q) * C::PLANE + i * C::PITCH, gr[q][i]);
+        for (int e = 0; e < HW; ++e) wv[0][e] = wc[co0 * K + e];
+
+        auto one_channel = [&](const int cc, const int cur) {
+            const int kofs = (co0 + cc) * K;
+            const bool more = cc + 1 < ccnt;
+            const int knext = more ? kofs + K : kofs;
 #pragma unroll
-            for (int q = 0; q < CQ; ++q) {
-                const int kofs = (co0 + cc + q) * K;
+            for (int h = 0; h < NU; ++h) {
 #pragma unroll
-                for (int m = 0; m < TM; ++m) {
-                    float wv[9];
+                for (int idx = 0; idx < HM * 9 * TN; ++idx) {
+                    const int t = idx % TN, j = (idx / TN) % 3, i = (idx / TN / 3) % 3, mm = idx / TN / 9;
+                    const int m = h * HM + mm;
+                    acc[m][t] = fmaf(hardtanh(wv[h & 1][mm * 9 + i * 3 + j] - xr[m][t]), gr[cur][2 - i][t + 2 - j],
+                                     acc[m][t]);
+                    if (idx == 0) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (h + 1 < NU) {
 #pragma unroll
-                    for (int e = 0; e < 9; ++e) wv[e] = wc[kofs + wofs[m] + e];
+                            for (int e = 0; e < HW; ++e) wv[(h + 1) & 1][e] = wc[kofs + (h + 1) * HW + e];
+                        } else {
 #pragma unroll
-                    for (int i = 0; i < 3; ++i)
+                            for (int e = 0; e < HW; ++e) wv[0][e] = wc[knext + e];
+                        }
+                        if (h == 0 && more) {
 #pragma unroll
-                        for (int j = 0; j < 3; ++j)
-#pragma unroll
-                            for (int t = 0; t < TN; ++t)
-                                acc[m][t] = fmaf(hardtanh(wv[i * 3 + j] - xr[m][t]), gr[q][2 - i][t + 2 - j],
-                                                 acc[m][t]);
+                            for (int i2 = 0; i2 < 3; ++i2)
+                                lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + (cc + 1) * C::PLANE + i2 * C::PITCH,
+                                                                       gr[cur ^ 1][i2]);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             }
+        };
+#pragma unroll 1
+        for (int cc = 0; cc < ccnt; cc += 2) {
+            one_channel(cc, 0);
+            if (cc + 1 < ccnt) one_channel(cc + 1, 1);
         }
 
         if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
@@ -175,7 +203,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
             const int ci = ci_base + m;
-            if (ci < Ci) {
+            if (ci >= ci_first) {
                 float *dst = gx + (((size_t)n * Ci + ci) * H + hi) * W + wi0;
                 if (TN % 4 == 0 && wi0 + TN <= W) {
 #pragma unroll
@@ -367,18 +395,18 @@ static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, 
 }
 
 //                              TNW BPR TH NIMG TM CIW CC
-using GxS2W32 = GradX3x3S2Cfg<2, 16, 32, 1, 8, 2, 8>;   // inputs 32 wide
-using GxS2W16 = GradX3x3S2Cfg<2, 8, 16, 1, 8, 4, 8>;    // inputs 16 wide
+using GxS2W32 = GradX3x3S2Cfg<2, 16, 32, 1, 8, 2, 16>;   // inputs 32 wide
+using GxS2W16 = GradX3x3S2Cfg<2, 8, 16, 1, 8, 4, 16>;    // inputs 16 wide
 
 //                        TN SPR TH NIMG TM COW CC CQ
 using GxW32 = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1>;
-using GxW16 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1>;
-using GxW8  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 8, 1>;
+using GxW16 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 16, 1>;
+using GxW8  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1>;
 
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s) {
     const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
-    if (k3s1p1 && d.W % 4 == 0 && (reinterpret_cast<uintptr_t>(gy) & 15) == 0 &&
+    if (k3s1p1 && d.W % 4 == 0 && d.Ci >= 8 && (reinterpret_cast<uintptr_t>(gy) & 15) == 0 &&
         (reinterpret_cast<uintptr_t>(gx) & 15) == 0) {
         if (d.W > 16) return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s);
         if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s);

@@ -1,0 +1,81 @@
+"""CIFAR ResNet-20 AdderNet: the harness model for the adder-conv kernels.
+
+Same architecture and state_dict keys as the reference's resnet20.py:7-97:
+regular 3x3 stem conv (resnet20.py:49), three stages of three BasicBlocks at
+16/32/64 channels whose convs are adder2d 3x3 pad 1 (resnet20.py:7-9,16-20),
+adder2d 1x1 stride-2 + BatchNorm downsample on the first block of stages 2
+and 3 (resnet20.py:66-70), 8x8 average pool, a regular 1x1 conv classifier
+followed by BatchNorm (resnet20.py:55-57,89-93), BatchNorm weights 1 / biases 0
+(resnet20.py:59-62).
+
+``adder2d_cls`` lets a caller build the same network around another
+implementation of the layer (the tests do this with their CPU reference).
+"""
+import torch.nn as nn
+
+from . import adder as _adder
+
+
+class BasicBlock(nn.Module):
+    expansion = 1
+
+    def __init__(self, inplanes, planes, stride=1, downsample=None, adder2d_cls=None, **adder_kw):
+        super().__init__()
+        make = adder2d_cls or _adder.adder2d
+        self.conv1 = make(inplanes, planes, kernel_size=3, stride=stride, padding=1, bias=False, **adder_kw)
+        self.bn1 = nn.BatchNorm2d(planes)
+        self.relu = nn.ReLU(inplace=True)
+        self.conv2 = make(planes, planes, kernel_size=3, stride=1, padding=1, bias=False, **adder_kw)
+        self.bn2 = nn.BatchNorm2d(planes)
+        self.downsample = downsample
+        self.stride = stride
+
+    def forward(self, x):
+        out = self.relu(self.bn1(self.conv1(x)))
+        out = self.bn2(self.conv2(out))
+        shortcut = x if self.downsample is None else self.downsample(x)
+        return self.relu(out + shortcut)
+
+
+class ResNet(nn.Module):
+    def __init__(self, block, layers, num_classes=10, adder2d_cls=None, **adder_kw):
+        super().__init__()
+        self._make = adder2d_cls or _adder.adder2d
+        self._adder_kw = adder_kw
+        self.inplanes = 16
+        self.conv1 = nn.Conv2d(3, 16, kernel_size=3, stride=1, padding=1, bias=False)
+        self.bn1 = nn.BatchNorm2d(16)
+        self.relu = nn.ReLU(inplace=True)
+        self.layer1 = self._make_layer(block, 16, layers[0])
+        self.layer2 = self._make_layer(block, 32, layers[1], stride=2)
+        self.layer3 = self._make_layer(block, 64, layers[2], stride=2)
+        self.avgpool = nn.AvgPool2d(8, stride=1)
+        self.fc = nn.Conv2d(64 * block.expansion, num_classes, 1, bias=False)
+        self.bn2 = nn.BatchNorm2d(num_classes)
+        for m in self.modules():
+            if isinstance(m, nn.BatchNorm2d):
+                nn.init.ones_(m.weight)
+                nn.init.zeros_(m.bias)
+
+    def _make_layer(self, block, planes, blocks, stride=1):
+        downsample = None
+        if stride != 1 or self.inplanes != planes * block.expansion:
+            downsample = nn.Sequential(
+                self._make(self.inplanes, planes * block.expansion, kernel_size=1, stride=stride, bias=False,
+                           **self._adder_kw),
+                nn.BatchNorm2d(planes * block.expansion))
+        stage = [block(self.inplanes, planes, stride, downsample, adder2d_cls=self._make, **self._adder_kw)]
+        self.inplanes = planes * block.expansion
+        stage += [block(self.inplanes, planes, adder2d_cls=self._make, **self._adder_kw) for _ in range(1, blocks)]
+        return nn.Sequential(*stage)
+
+    def forward(self, x):
+        x = self.relu(self.bn1(self.conv1(x)))
+        x = self.layer3(self.layer2(self.layer1(x)))
+        x = self.bn2(self.fc(self.avgpool(x)))
+        return x.view(x.size(0), -1)
+
+
+def resnet20(**kwargs):
+    """resnet20.py:96-97."""
+    return ResNet(BasicBlock, [3, 3, 3], **kwargs)

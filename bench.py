@@ -1,0 +1,279 @@
+#!/usr/bin/env python3
+"""ResNet-20 AdderNet training-step benchmark on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu] [--layers]
+
+Prints ONE JSON line.  `value` is milliseconds per training step (forward +
+backward + SGD) of the ResNet-20 AdderNet at batch 256, 3x32x32 fp32 synthetic
+input resident in HBM; `layers` carries, per adder-layer shape of the network,
+the time, TFLOP/s and fraction of the fp32 vector peak of each of the three
+kernels; `roofline` is the dominant kernel; `cpu_baseline` is the CPU oracle's
+training step (batch 8, scaled to 256) timed on this box's host cores.
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_TFLOPS = 157.3           # MI355X vendor fp32 vector peak (256 CU x 64 lanes x 2 (packed) x 2 (FMA) x 2.4 GHz)
+PEAK_VALU_ISSUE = 256 * 64 * 2.4e9  # lane-instructions per second (one fp32 VALU op per lane per clock)
+BATCH = 256
+ETA = 0.1
+
+# distinct adder-layer shapes of ResNet-20 at 32x32 input: (count, Ci, H, W, Co, k, stride, pad)
+RESNET20_LAYERS = [
+    (6, 16, 32, 32, 16, 3, 1, 1),
+    (1, 16, 32, 32, 32, 1, 2, 0),
+    (1, 16, 32, 32, 32, 3, 2, 1),
+    (5, 32, 16, 16, 32, 3, 1, 1),
+    (1, 32, 16, 16, 64, 1, 2, 0),
+    (1, 32, 16, 16, 64, 3, 2, 1),
+    (5, 64, 8, 8, 64, 3, 1, 1),
+]
+# flops per (co, k, position) term and the fewest fp32 VALU instructions that implement it
+OPS = {"fwd": (2, 2), "grad_x": (4, 3), "grad_w": (3, 1)}
+
+
+def event_time(fn, warmup, iters):
+    """Average seconds per call, HIP events on the stream the kernels are launched on (torch's current one)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e-3 / iters
+
+
+def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
+    """The three C-ABI calls of one layer shape on synthetic tensors; returns (E, {op: callable})."""
+    from addernetcuda_amd._lib import lib, ptr, stream_ptr, conv_dims, check
+    g = torch.Generator(device=dev).manual_seed(1000 + Ci + Co + k + stride)
+    x = torch.randn(N, Ci, H, W, device=dev, generator=g)
+    w = torch.randn(Co, Ci, k, k, device=dev, generator=g) * math.sqrt(2.0 / (Ci * k * k))
+    dims, Ho, Wo = conv_dims(x.shape, w.shape, stride, pad)
+    y = torch.empty(N, Co, Ho, Wo, device=dev)
+    gy = torch.randn(N, Co, Ho, Wo, device=dev, generator=g)
+    gx, gw = torch.empty_like(x), torch.empty_like(w)
+    need = ctypes.c_size_t()
+    check(lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)), "workspace")
+    ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=dev)
+    st = stream_ptr(dev)
+    E = Co * Ci * k * k * N * Ho * Wo
+    keep = (x, w, y, gy, gx, gw, ws)
+    ops = {
+        "fwd": lambda: check(lib.adder_conv2d_fwd_f32(ptr(x), ptr(w), ptr(y), *dims, st), "fwd"),
+        "grad_x": lambda: check(lib.adder_conv2d_bwd_f32(ptr(gy), ptr(x), ptr(w), ptr(gx), None, 0.0, None, 0,
+                                                         *dims, st), "grad_x"),
+        "grad_w": lambda: check(lib.adder_conv2d_bwd_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gw), ETA, ptr(ws),
+                                                         need.value, *dims, st), "grad_w"),
+    }
+    return E, ops, keep
+
+
+def bench_layers(dev, warmup=5, iters=20):
+    rows = []
+    for cnt, Ci, H, W, Co, k, s, p in RESNET20_LAYERS:
+        E, ops, keep = layer_ops(BATCH, Ci, H, W, Co, k, s, p, dev)
+        for name, fn in ops.items():
+            t = event_time(fn, warmup, iters)
+            flop, slots = OPS[name]
+            rows.append({
+                "layer": f"{Ci}->{Co} k{k} s{s} p{p} @{H}x{W}", "count": cnt, "op": name, "us": round(t * 1e6, 2),
+                "tflops": round(flop * E / t / 1e12, 2),
+                "frac_fp32_peak": round(flop * E / t / 1e12 / PEAK_FP32_TFLOPS, 4),
+                "valu_issue_util": round(slots * E / t / PEAK_VALU_ISSUE, 4),
+            })
+        del keep
+    return rows
+
+
+def dominant_kernel(dev, steps):
+    """grad_x of the 16->16 3x3 @32x32 layer: the kernel with the largest share of a training step."""
+    cnt, Ci, H, W, Co, k, s, p = RESNET20_LAYERS[0]
+    E, ops, keep = layer_ops(BATCH, Ci, H, W, Co, k, s, p, dev)
+    t = event_time(ops["grad_x"], 5, max(20, steps))
+    flop = OPS["grad_x"][0] * E
+    achieved = flop / t / 1e12
+    return {
+        "bound": "valu", "kernel": "adder::grad_x_3x3s1_kernel (16->16, 3x3 s1 p1, 32x32, batch 256)",
+        "achieved": round(achieved, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_FP32_TFLOPS, 4), "traffic": None,
+        "avg_launch_us": round(t * 1e6, 2), "flop_per_launch": flop,
+        "valu_issue_util": round(OPS["grad_x"][1] * E / t / PEAK_VALU_ISSUE, 4),
+        "note": "fp32 VALU-bound (|a-b| accumulation has no FMA/MFMA form); peak is the packed-FMA vector "
+                "figure, the 3-instruction-per-4-flop inner op caps this kernel at 1/3 of it",
+    }
+
+
+def make_step(model, opt, x, y):
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.cross_entropy(model(x), y)
+        loss.backward()
+        opt.step()
+        return loss
+    return step
+
+
+def build_training(dev, seed=0):
+    from addernetcuda_amd.resnet20 import resnet20
+    torch.manual_seed(seed)
+    model = resnet20(eta=ETA).to(dev)
+    opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4)
+    g = torch.Generator(device=dev).manual_seed(seed + 1)
+    x = torch.randn(BATCH, 3, 32, 32, device=dev, generator=g)
+    y = torch.randint(0, 10, (BATCH,), device=dev, generator=g)
+    return model, opt, x, y
+
+
+def capture_step(model, opt, x, y):
+    """Whole training step as one HIP graph (the eager step is launch-bound on the host)."""
+    step = make_step(model, opt, x, y)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    opt.zero_grad(set_to_none=True)
+    with torch.cuda.graph(graph):
+        loss = torch.nn.functional.cross_entropy(model(x), y)
+        loss.backward()
+        opt.step()
+    return graph, loss
+
+
+def graph_matches_eager(dev, replays=4):
+    """Replay the captured step from a saved state and run the eager step from the same state, several times.
+
+    Torch's own kernels are not run-to-run deterministic, so trajectories cannot be compared over many steps;
+    one step from identical weights, momentum and BatchNorm statistics can.
+    """
+    import copy
+    model, opt, x, y = build_training(dev)
+    graph, loss = capture_step(model, opt, x, y)
+    eager = make_step(model, opt, x, y)
+    worst = 0.0
+    losses = []
+    for _ in range(replays):
+        saved = ({k: v.clone() for k, v in model.state_dict().items()}, copy.deepcopy(opt.state_dict()))
+        graph.replay()
+        torch.cuda.synchronize()
+        lg = loss.item()
+        pg = {k: v.clone() for k, v in model.state_dict().items()}
+        model.load_state_dict(saved[0])
+        opt.load_state_dict(saved[1])
+        le = eager().item()
+        torch.cuda.synchronize()
+        pe = model.state_dict()
+        worst = max(worst, max((pg[k].float() - pe[k].float()).abs().max().item() for k in pg))
+        losses.append((lg, le))
+    ok = worst <= 1e-4 and all(abs(a - b) <= 1e-4 * max(1.0, abs(b)) for a, b in losses)
+    return ok, worst, losses
+
+
+def cpu_baseline(repeats=5):
+    """The CPU oracle's ResNet-20 training step at batch 8 (seeded), median of `repeats`, scaled to batch 256."""
+    from addernetcuda_amd.resnet20 import resnet20
+    from oracle import adder_oracle
+    torch.manual_seed(0)
+    model = resnet20(adder2d_cls=adder_oracle.adder2d, eta=ETA)
+    opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4)
+    bs = 8
+    x = torch.randn(bs, 3, 32, 32)
+    y = torch.randint(0, 10, (bs,))
+    step = make_step(model, opt, x, y)
+    step()
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {
+        "value": round(med * 1e3 * (BATCH / bs), 1), "unit": "ms/batch (batch 256)", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"ResNet-20 AdderNet fwd+bwd+SGD at batch {bs} through the pure-PyTorch unfold oracle, median of "
+                  f"{repeats} steps = {med * 1e3:.0f} ms, scaled x{BATCH // bs} to batch 256",
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-graph", action="store_true", help="time the eager step instead of the captured HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (every box here has a single MI355X)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    mode = "eager"
+    graph_check = None
+    model, opt, x, y = build_training(dev)
+    if not args.no_graph:
+        ok, worst, losses = graph_matches_eager(dev)
+        graph_check = {"ok": ok, "max_param_diff_vs_eager_step": worst,
+                       "loss_graph_vs_eager": [[round(a, 6), round(b, 6)] for a, b in losses]}
+        if ok:
+            mode = "hipgraph"
+    if mode == "hipgraph":
+        graph, loss = capture_step(model, opt, x, y)
+        run = graph.replay
+    else:
+        run = make_step(model, opt, x, y)
+
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    out = {
+        "metric": "ResNet-20 AdderNet train ms/batch (bs256)", "value": round(ms, 3), "unit": "ms/batch",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "ResNet-20 AdderNet, batch 256, 3x32x32, 10 classes, SGD momentum 0.9 lr 0.1 wd 5e-4, "
+                               "adaptive eta 0.1, fwd+bwd+optimizer", "step_mode": mode},
+        "images_per_s": round(BATCH / ms * 1e3, 1),
+        "roofline": dominant_kernel(dev, args.steps),
+    }
+    if graph_check is not None:
+        out["graph_check"] = graph_check
+    if not args.no_layers:
+        rows = bench_layers(dev)
+        out["layers"] = rows
+        out["adder_kernel_ms_per_step"] = round(sum(r["us"] * r["count"] for r in rows) / 1e3, 3)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -20,6 +20,7 @@ TILED = [
     (2, 5, 12, 20, 7, 3, 1, 1),     # channel tails, H != W, partial tiles
     (1, 3, 9, 40, 4, 3, 1, 1),      # two tiles along W
     (2, 12, 8, 8, 12, 3, 1, 1),     # DenseNet-style 12 channels
+    (2, 20, 12, 20, 12, 3, 1, 1),   # channel tails on the tiled path (Ci, Co not multiples of 8)
     (1, 24, 4, 4, 48, 3, 1, 1),     # map smaller than a tile
     (2, 16, 32, 32, 32, 3, 2, 1),   # ResNet-20 strided 3x3, 32 -> 16
     (3, 32, 16, 16, 64, 3, 2, 1),   # ResNet-20 strided 3x3, 16 -> 8
