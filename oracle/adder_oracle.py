@@ -53,7 +53,7 @@ def col_forward(X_col, W_col):
     """
     Co, K = W_col.shape
     NL = X_col.shape[1]
-    out = torch.empty((Co, NL), dtype=X_col.dtype)
+    out = torch.empty((Co, NL), dtype=X_col.dtype, device=X_col.device)
     step = _chunk_len(Co, K)
     for a, b in _chunks(NL, step):
         out[:, a:b] = -(W_col.unsqueeze(2) - X_col[:, a:b].unsqueeze(0)).abs().sum(1)
@@ -64,7 +64,7 @@ def col_grad_w(X_col, W_col, grad_output):
     """grad_W[co,k] = sum_nl (X[k,nl] - W[co,k]) * g[co,nl]  (test_cuda.py:35-41, adder.py:70)."""
     Co, K = W_col.shape
     NL = X_col.shape[1]
-    acc = torch.zeros((Co, K), dtype=X_col.dtype)
+    acc = torch.zeros((Co, K), dtype=X_col.dtype, device=X_col.device)
     step = _chunk_len(Co, K)
     for a, b in _chunks(NL, step):
         acc += ((X_col[:, a:b].unsqueeze(0) - W_col.unsqueeze(2))
@@ -79,7 +79,7 @@ def col_grad_x(X_col, W_col, grad_output):
     """
     Co, K = W_col.shape
     NL = X_col.shape[1]
-    out = torch.empty((K, NL), dtype=X_col.dtype)
+    out = torch.empty((K, NL), dtype=X_col.dtype, device=X_col.device)
     step = _chunk_len(Co, K)
     for a, b in _chunks(NL, step):
         out[:, a:b] = (-(X_col[:, a:b].unsqueeze(0) - W_col.unsqueeze(2)).clamp(-1, 1)

@@ -1,0 +1,112 @@
+"""The C-ABI library loads, exports every symbol the header declares, and rejects bad
+arguments before touching the GPU (so all of this runs on a machine without one)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "addernet_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return sorted(set(re.findall(r"ADDER_API\s+(?:const\s+)?\w+\s*\*?\s*(adder_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for must in ("adder_conv2d_fwd_f32", "adder_conv2d_bwd_f32", "adder_conv2d_bwd_workspace_bytes",
+                 "adder_col_fwd_f32", "adder_col_bwd_f32", "adder_col_gradw_f32", "adder_col_gradx_f32",
+                 "adder_grad_norm_scale_f32", "adder_strerror"):
+        assert must in names
+    assert len(names) >= 14
+
+
+def test_library_exports_every_declared_symbol():
+    from addernetcuda_amd import _lib
+    assert os.path.exists(_lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(_lib.lib, name), f"{name} is declared in the header but not exported"
+        assert name in _lib.EXPORTED, f"{name} has no ctypes signature in _lib.py"
+
+
+def test_status_strings_and_version():
+    from addernetcuda_amd._lib import lib
+    assert lib.adder_abi_version() == 1
+    assert lib.adder_strerror(0) == b"ok"
+    seen = {lib.adder_strerror(c) for c in range(-6, 1)}
+    assert len(seen) == 7 and b"unknown status" not in seen
+    assert lib.adder_strerror(-99) == b"unknown status"
+
+
+@pytest.mark.parametrize("h,k,p,s,want", [(32, 3, 1, 1, 32), (32, 3, 1, 2, 16), (32, 1, 0, 2, 16), (7, 3, 1, 2, 4),
+                                           (11, 5, 2, 3, 4), (5, 3, 0, 1, 3), (2, 3, 0, 1, 0), (0, 3, 1, 1, 0)])
+def test_out_dim_follows_the_reference_formula(h, k, p, s, want):
+    from addernetcuda_amd._lib import lib
+    assert lib.adder_out_dim(h, k, p, s) == want
+    if want > 0:
+        assert want == int((h - k + 2 * p) / s + 1)      # adder.py:26-31
+
+
+def test_forward_rejects_bad_arguments_without_a_gpu():
+    from addernetcuda_amd._lib import lib
+    P = ctypes.c_void_p
+    ok = (P(4096), P(8192), P(1 << 20))
+    assert lib.adder_conv2d_fwd_f32(None, ok[1], ok[2], 1, 1, 4, 4, 1, 3, 3, 1, 1, None) == -1
+    assert lib.adder_conv2d_fwd_f32(ok[0], ok[1], None, 1, 1, 4, 4, 1, 3, 3, 1, 1, None) == -1
+    assert lib.adder_conv2d_fwd_f32(*ok, 0, 1, 4, 4, 1, 3, 3, 1, 1, None) == -2      # N = 0
+    assert lib.adder_conv2d_fwd_f32(*ok, 1, 1, 4, 4, 1, 3, 3, 0, 1, None) == -2      # stride 0
+    assert lib.adder_conv2d_fwd_f32(*ok, 1, 1, 4, 4, 1, 3, 3, 1, -1, None) == -2     # negative padding
+    assert lib.adder_conv2d_fwd_f32(*ok, 1, 1, 2, 2, 1, 5, 5, 1, 0, None) == -2      # kernel larger than input
+    assert lib.adder_conv2d_fwd_f32(*ok, 1 << 20, 64, 64, 64, 1, 3, 3, 1, 1, None) == -3   # > 2^31-1 elements
+    assert lib.adder_conv2d_fwd_f32(P(4096), P(8192), P(4100), 1, 1, 4, 4, 1, 3, 3, 1, 1, None) == -6  # y overlaps x
+
+
+def test_backward_rejects_bad_arguments_without_a_gpu():
+    from addernetcuda_amd._lib import lib
+    P = ctypes.c_void_p
+    dims = (2, 4, 8, 8, 4, 3, 3, 1, 1)
+    need = ctypes.c_size_t()
+    assert lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)) == 0 and need.value >= 256
+    assert lib.adder_conv2d_bwd_workspace_bytes(*dims, None) == -1
+    gy, x, w, gx, gw, ws = (P(a << 20) for a in range(1, 7))
+    call = lib.adder_conv2d_bwd_f32
+    assert call(None, x, w, gx, gw, 0.2, ws, need.value, *dims, None) == -1
+    assert call(gy, x, w, None, None, 0.2, ws, need.value, *dims, None) == -1        # nothing to compute
+    assert call(gy, x, w, gx, gw, -1.0, ws, need.value, *dims, None) == -2           # negative eta
+    assert call(gy, x, w, gx, gw, float("nan"), ws, need.value, *dims, None) == -2
+    assert call(gy, x, w, gx, gw, 0.2, None, 0, *dims, None) == -4                   # grad_w needs scratch
+    assert call(gy, x, w, gx, gw, 0.2, ws, need.value - 1, *dims, None) == -4
+    assert call(gy, x, w, gx, gw, 0.2, P((6 << 20) + 8), need.value, *dims, None) == -4   # misaligned scratch
+    assert call(gy, x, w, x, gw, 0.2, ws, need.value, *dims, None) == -6             # gx aliases x
+    assert call(gy, x, w, gx, gw, 0.2, gw, need.value, *dims, None) == -6            # scratch aliases gw
+
+
+def test_column_entry_points_reject_bad_arguments_without_a_gpu():
+    from addernetcuda_amd._lib import lib
+    P = ctypes.c_void_p
+    a, b, c, d, e = (P(k << 24) for k in range(1, 6))
+    assert lib.adder_col_fwd_f32(a, b, None, 9, 16, 4, None) == -1
+    assert lib.adder_col_fwd_f32(a, b, c, 0, 16, 4, None) == -2
+    assert lib.adder_col_fwd_f32(a, b, c, 9, 1 << 40, 4, None) == -3
+    assert lib.adder_col_fwd_f32(a, b, a, 9, 16, 4, None) == -6
+    assert lib.adder_col_bwd_f32(a, b, c, d, None, 9, 16, 4, None, 0, None) == -1
+    assert lib.adder_col_gradw_f32(a, b, c, c, 9, 16, 4, None, 0, None) == -6
+    assert lib.adder_col_gradx_f32(a, b, c, b, 9, 16, 4, None) == -6
+    n = ctypes.c_size_t(123)
+    assert lib.adder_col_bwd_workspace_bytes(9, 16, 4, ctypes.byref(n)) == 0
+    assert lib.adder_grad_norm_scale_f32(None, 10, 0.2, 1e-12, a, 1 << 20, None) == -1
+    assert lib.adder_grad_norm_scale_f32(a, 0, 0.2, 1e-12, b, 1 << 20, None) == -2
+    assert lib.adder_grad_norm_scale_f32(a, 10, 0.2, 0.0, b, 1 << 20, None) == -2    # eps must be positive
+    assert lib.adder_grad_norm_scale_f32(a, 10, 0.2, 1e-12, None, 0, None) == -4
+
+
+def test_workspace_is_large_enough_for_the_partials_of_big_layers():
+    from addernetcuda_amd._lib import lib
+    need = ctypes.c_size_t()
+    for dims in [(256, 16, 32, 32, 16, 3, 3, 1, 1), (256, 64, 8, 8, 64, 3, 3, 1, 1), (128, 512, 8, 8, 512, 3, 3, 1, 1),
+                 (64, 256, 56, 56, 64, 1, 1, 1, 0)]:
+        assert lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)) == 0
+        assert need.value % 256 == 0 and need.value < (2 << 30)

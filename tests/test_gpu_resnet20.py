@@ -1,0 +1,106 @@
+"""ResNet-20 AdderNet training on the HIP layer: against the same network built on the oracle layer,
+and the captured HIP graph against the eager step."""
+import copy
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(gpu, batch, eta=0.1, seed=0):
+    from addernetcuda_amd.resnet20 import resnet20
+    from oracle import adder_oracle
+    torch.manual_seed(seed)
+    hip = resnet20(eta=eta).to(gpu)
+    ref = resnet20(adder2d_cls=adder_oracle.adder2d, eta=eta).to(gpu)   # pure-torch unfold formulas, run on the GPU
+    ref.load_state_dict(hip.state_dict())
+    g = torch.Generator(device=gpu).manual_seed(seed + 1)
+    x = torch.randn(batch, 3, 32, 32, device=gpu, generator=g)
+    y = torch.randint(0, 10, (batch,), device=gpu, generator=g)
+    return hip, ref, x, y
+
+
+def test_one_step_matches_the_unfold_reference_path(gpu):
+    """Same weights, same batch: logits, loss and every gradient agree with the reference formulation.
+
+    Gradients are compared to 2% of each tensor's largest entry: behind 19 BatchNorm + ReLU stages a
+    1e-6 difference in an activation can flip a ReLU gate, which moves single entries of the deepest
+    layers' gradients by parts in a thousand; the per-layer kernels themselves are held to
+    rtol 1e-5 / atol 1e-4 elsewhere."""
+    hip, ref, x, y = _pair(gpu, 16)
+    outs = []
+    for m in (hip, ref):
+        logits = m(x)
+        loss = torch.nn.functional.cross_entropy(logits, y)
+        loss.backward()
+        outs.append((logits.detach(), loss.item()))
+    assert torch.allclose(outs[0][0], outs[1][0], rtol=1e-3, atol=1e-3)
+    assert outs[0][1] == pytest.approx(outs[1][1], rel=1e-4)
+    ph, pr = dict(hip.named_parameters()), dict(ref.named_parameters())
+    for name in ph:
+        a, b = ph[name].grad, pr[name].grad
+        scale = b.abs().max().item() + 1e-12
+        assert (a - b).abs().max().item() <= 2e-2 * scale, name
+
+
+def test_loss_curves_track_the_reference_path(gpu):
+    """50 SGD steps (momentum 0.9, lr 0.1, wd 5e-4, eta 0.1) on one synthetic batch of 64.
+
+    The first two losses must agree tightly (same weights, one update).  After that fp32 training of this
+    network is chaotic: two runs of the *same* code already differ by up to ~0.2 in loss around step 20-30
+    because torch's BatchNorm / reduction kernels are not run-to-run reproducible and the eta-normalised
+    updates amplify a flipped ReLU gate.  So from step 2 on the curves are required to stay within 0.35 of
+    each other, and both must fit the batch (loss down to a quarter of its start)."""
+    hip, ref, x, y = _pair(gpu, 64)
+    curves = []
+    for m in (hip, ref):
+        opt = torch.optim.SGD(m.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4)
+        losses = []
+        for _ in range(50):
+            opt.zero_grad(set_to_none=True)
+            loss = torch.nn.functional.cross_entropy(m(x), y)
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+        curves.append(losses)
+    a, b = curves
+    for i in range(2):
+        assert abs(a[i] - b[i]) <= 1e-3 * max(1.0, abs(b[i])), (i, a[i], b[i])
+    for i in range(2, 50):
+        assert abs(a[i] - b[i]) <= 0.35, (i, a[i], b[i])
+    assert a[-1] < 0.25 * a[0] and b[-1] < 0.25 * b[0]
+
+
+def test_captured_graph_replays_match_the_eager_step(gpu):
+    """The whole training step as one HIP graph: every replay, with eager work and synchronisation in
+    between, must land on the same weights as the eager step from the same state."""
+    import bench
+    model, opt, x, y = bench.build_training(gpu)
+    graph, loss = bench.capture_step(model, opt, x, y)
+    eager = bench.make_step(model, opt, x, y)
+    for _ in range(4):
+        saved = ({k: v.clone() for k, v in model.state_dict().items()}, copy.deepcopy(opt.state_dict()))
+        graph.replay()
+        torch.cuda.synchronize()
+        lg = loss.item()
+        got = {k: v.clone() for k, v in model.state_dict().items()}
+        model.load_state_dict(saved[0])
+        opt.load_state_dict(saved[1])
+        le = eager().item()
+        torch.cuda.synchronize()
+        want = model.state_dict()
+        assert lg == pytest.approx(le, rel=1e-5)
+        for k in got:
+            assert torch.allclose(got[k].float(), want[k].float(), rtol=1e-4, atol=1e-5), k
+
+
+def test_state_dict_round_trip_and_eval_forward(gpu):
+    from addernetcuda_amd.resnet20 import resnet20
+    torch.manual_seed(3)
+    a, b = resnet20().to(gpu), resnet20().to(gpu)
+    b.load_state_dict(a.state_dict())
+    a.eval(), b.eval()
+    x = torch.randn(8, 3, 32, 32, device=gpu)
+    with torch.no_grad():
+        assert torch.equal(a(x), b(x))
