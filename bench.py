@@ -29,6 +29,9 @@ PEAK_FP32_TFLOPS = 157.3           # MI355X vendor fp32 vector peak (256 CU x 64
 PEAK_VALU_ISSUE = 256 * 64 * 2.4e9  # lane-instructions per second (one fp32 VALU op per lane per clock)
 BATCH = 256
 ETA = 0.1
+# HBM bytes per launch of the dominant kernel, from the rocprofv3 counter passes kept under profiles/
+# (34.0 MB fetched + 16.8 MB written; cannot be read without the profiler attached)
+DOMINANT_TRAFFIC_BYTES = 50.8e6
 
 # distinct adder-layer shapes of ResNet-20 at 32x32 input: (count, Ci, H, W, Co, k, stride, pad)
 RESNET20_LAYERS = [
@@ -111,7 +114,10 @@ def dominant_kernel(dev, steps):
     return {
         "bound": "valu", "kernel": "adder::grad_x_3x3s1_kernel (16->16, 3x3 s1 p1, 32x32, batch 256)",
         "achieved": round(achieved, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved / PEAK_FP32_TFLOPS, 4), "traffic": None,
+        "frac": round(achieved / PEAK_FP32_TFLOPS, 4), "traffic": DOMINANT_TRAFFIC_BYTES,
+        "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy: "
+                          "profiles/grad_x_3x3s1_resnet20_16to16_32x32_bs256.md",
+        "algorithmic_bytes": 4 * (2 * BATCH * Ci * H * W + BATCH * Co * H * W + Co * Ci * k * k),
         "avg_launch_us": round(t * 1e6, 2), "flop_per_launch": flop,
         "valu_issue_util": round(OPS["grad_x"][1] * E / t / PEAK_VALU_ISSUE, 4),
         "note": "fp32 VALU-bound (|a-b| accumulation has no FMA/MFMA form); peak is the packed-FMA vector "
@@ -223,6 +229,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time the eager step instead of the captured HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="launch only the dominant kernel (and one 256 MiB device copy as a counter yardstick); "
+                         "meant to run under rocprofv3 --pmc / --kernel-trace")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (every box here has a single MI355X)")
@@ -230,6 +239,15 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.roofline_only:
+        src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)            # 256 MiB read + 256 MiB written per launch
+        torch.cuda.synchronize()
+        print(json.dumps({"roofline": dominant_kernel(dev, args.steps), "copy_bytes_each_way": src.numel() * 4}))
+        return
 
     mode = "eager"
     graph_check = None
