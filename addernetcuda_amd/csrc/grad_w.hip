@@ -135,7 +135,7 @@ __device__ __forceinline__ void gy_fetch(GyStage<G> &st, const float *__restrict
         const int n = n0 + img, co = co0 + c, ho = h0 + r, wo = w0 + 4 * q;
         const bool ok = (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) && n < N && co < Co && ho < Ho && wo < Wo;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok) val = *reinterpret_cast<const float4 *>(gy + (((size_t)n * Co + co) * Ho + ho) * Wo + wo);
+        if (ok) val = *reinterpret_cast<const float4 *>(gy + (((n * Co + co) * Ho + ho) * Wo + wo));
         st.v[it] = val;
     }
 }
@@ -379,15 +379,22 @@ int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStrea
 }
 
 // ---- dispatch -----------------------------------------------------------------
-//                     TN SPR TH NIMG TM CQ NCOB NCIB S
-using GwW32   = GradWCfg<4, 8, 8, 1, 8, 2, 2, 4, 1>;
-using GwW16   = GradWCfg<4, 4, 16, 1, 8, 2, 2, 4, 1>;
-using GwW8    = GradWCfg<4, 2, 8, 4, 8, 2, 2, 4, 1>;
-using GwW16S2 = GradWCfg<4, 4, 16, 1, 8, 1, 2, 4, 2>;
-using GwW8S2  = GradWCfg<4, 2, 8, 4, 8, 1, 2, 4, 2>;
+// Channel blocking of a workgroup: TM x CQ (co, ci) pairs per wave, NCOB x NCIB waves.
+struct GwChan0 { static constexpr int TM = 8, CQ = 2, NCOB = 2, NCIB = 4; };   // 144 sums per lane, 8 waves
+struct GwChan1 { static constexpr int TM = 8, CQ = 1, NCOB = 2, NCIB = 4; };   // 72 sums per lane, 8 waves
+struct GwChan2 { static constexpr int TM = 4, CQ = 2, NCOB = 4, NCIB = 2; };   // 72 sums per lane, 8 waves
+struct GwChan3 { static constexpr int TM = 8, CQ = 1, NCOB = 2, NCIB = 8; };   // 72 sums per lane, 16 waves
+struct GwChan4 { static constexpr int TM = 4, CQ = 2, NCOB = 4, NCIB = 4; };   // 72 sums per lane, 16 waves
+//                                     TN SPR TH NIMG
+template <class Ch> using GwW32   = GradWCfg<4, 8, 8, 1, Ch::TM, Ch::CQ, Ch::NCOB, Ch::NCIB, 1>;
+template <class Ch> using GwW16   = GradWCfg<4, 4, 16, 1, Ch::TM, Ch::CQ, Ch::NCOB, Ch::NCIB, 1>;
+template <class Ch> using GwW8    = GradWCfg<4, 2, 8, 4, Ch::TM, Ch::CQ, Ch::NCOB, Ch::NCIB, 1>;
+template <class Ch> using GwW16S2 = GradWCfg<4, 4, 16, 1, Ch::TM, Ch::CQ, Ch::NCOB, Ch::NCIB, 2>;
+template <class Ch> using GwW8S2  = GradWCfg<4, 2, 8, 4, Ch::TM, Ch::CQ, Ch::NCOB, Ch::NCIB, 2>;
 
 struct GradWPlan {
     int variant;  // 0 generic, 1 W32, 2 W16, 3 W8, 4 W16S2, 5 W8S2, 6 1x1
+    int chan;     // channel blocking (GwChan<chan>) of the tiled variants
     int slots, gy, gz, tilesH, tilesW, ntiles;
 };
 
@@ -398,24 +405,42 @@ static void plan_tiled(const ConvDims &d, GradWPlan &p) {
     p.ntiles = ceil_div(d.N, G::NIMG) * p.tilesH * p.tilesW;
     p.gy = ceil_div(d.Co, G::COB);
     p.gz = ceil_div(d.Ci, G::CIB);
-    // about one 8-wave workgroup per CU, but at least ~4 tiles each so the fold is amortised
-    int want = ceil_div(256, p.gy * p.gz);
+    // enough workgroups to fill the chip, but at least ~4 tiles each so the fold is amortised
+    static const int wgs = tune_knob("GW_WGS", 256);
+    int want = ceil_div(wgs, p.gy * p.gz);
     int cap = p.ntiles / 4 > 0 ? p.ntiles / 4 : 1;
     p.slots = want < cap ? want : cap;
     if (p.slots > p.ntiles) p.slots = p.ntiles;
+}
+
+template <class Ch>
+static void plan_shape(const ConvDims &d, GradWPlan &p) {
+    switch (p.variant) {
+        case 1: plan_tiled<GwW32<Ch>>(d, p); break;
+        case 2: plan_tiled<GwW16<Ch>>(d, p); break;
+        case 3: plan_tiled<GwW8<Ch>>(d, p); break;
+        case 4: plan_tiled<GwW16S2<Ch>>(d, p); break;
+        case 5: plan_tiled<GwW8S2<Ch>>(d, p); break;
+    }
 }
 
 static GradWPlan plan_grad_w(const ConvDims &d) {
     GradWPlan p{};
     const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.W % 4 == 0 && d.Wo % 4 == 0;
     const long partial_cap = 1L << 28;  // keep the partial buffer below 1 GiB
-    if (k3p1 && d.stride == 1) {
-        if (d.Wo > 16) { p.variant = 1; plan_tiled<GwW32>(d, p); }
-        else if (d.Wo > 8) { p.variant = 2; plan_tiled<GwW16>(d, p); }
-        else { p.variant = 3; plan_tiled<GwW8>(d, p); }
-    } else if (k3p1 && d.stride == 2) {
-        if (d.Wo > 8) { p.variant = 4; plan_tiled<GwW16S2>(d, p); }
-        else { p.variant = 5; plan_tiled<GwW8S2>(d, p); }
+    if (k3p1 && d.stride == 1) p.variant = d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
+    else if (k3p1 && d.stride == 2) p.variant = d.Wo > 8 ? 4 : 5;
+    if (p.variant) {
+        static const int chan_s1 = tune_knob("GW_CHAN", 0), chan_s2 = tune_knob("GW_CHAN_S2", 1);
+        p.chan = d.stride == 1 ? chan_s1 : chan_s2;
+        if (d.stride == 2 && (p.chan == 0)) p.chan = 1;   // 144 sums + stride-2 strips do not fit the register file
+        switch (p.chan) {
+            case 0: plan_shape<GwChan0>(d, p); break;
+            case 1: plan_shape<GwChan1>(d, p); break;
+            case 2: plan_shape<GwChan2>(d, p); break;
+            case 3: plan_shape<GwChan3>(d, p); break;
+            default: p.chan = 4; plan_shape<GwChan4>(d, p); break;
+        }
     }
     if (!p.variant && conv1x1_supported(d, nullptr, nullptr)) {
         p.variant = 6;
@@ -447,6 +472,19 @@ static int launch_tiled(const float *gy, const float *x, float *part, float *sgp
     return check_launch();
 }
 
+template <class Ch>
+static int launch_shape(const float *gy, const float *x, float *part, float *sgpart, const ConvDims &d,
+                        const GradWPlan &p, hipStream_t s) {
+    switch (p.variant) {
+        case 1: return launch_tiled<GwW32<Ch>>(gy, x, part, sgpart, d, p, s);
+        case 2: return launch_tiled<GwW16<Ch>>(gy, x, part, sgpart, d, p, s);
+        case 3: return launch_tiled<GwW8<Ch>>(gy, x, part, sgpart, d, p, s);
+        case 4: if constexpr (Ch::TM * Ch::CQ <= 8) return launch_tiled<GwW16S2<Ch>>(gy, x, part, sgpart, d, p, s);
+        default: if constexpr (Ch::TM * Ch::CQ <= 8) return launch_tiled<GwW8S2<Ch>>(gy, x, part, sgpart, d, p, s);
+    }
+    return ADDER_ERR_BAD_SHAPE;
+}
+
 int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
                   size_t ws_bytes, const ConvDims &d, hipStream_t s) {
     if (ws_bytes < grad_w_workspace_bytes(d)) return ADDER_ERR_WORKSPACE;
@@ -459,13 +497,16 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
         float *part = reinterpret_cast<float *>(ss + kNormBlocksMax);
         float *sgpart = part + (size_t)p.slots * d.Co * K;
         int rc;
-        switch (p.variant) {
-            case 1: rc = launch_tiled<GwW32>(gy, x, part, sgpart, d, p, s); break;
-            case 2: rc = launch_tiled<GwW16>(gy, x, part, sgpart, d, p, s); break;
-            case 3: rc = launch_tiled<GwW8>(gy, x, part, sgpart, d, p, s); break;
-            case 4: rc = launch_tiled<GwW16S2>(gy, x, part, sgpart, d, p, s); break;
-            case 6: rc = launch_grad_w_1x1(gy, x, part, sgpart, p.slots, d, s); break;
-            default: rc = launch_tiled<GwW8S2>(gy, x, part, sgpart, d, p, s); break;
+        if (p.variant == 6) {
+            rc = launch_grad_w_1x1(gy, x, part, sgpart, p.slots, d, s);
+        } else {
+            switch (p.chan) {
+                case 0: rc = launch_shape<GwChan0>(gy, x, part, sgpart, d, p, s); break;
+                case 1: rc = launch_shape<GwChan1>(gy, x, part, sgpart, d, p, s); break;
+                case 2: rc = launch_shape<GwChan2>(gy, x, part, sgpart, d, p, s); break;
+                case 3: rc = launch_shape<GwChan3>(gy, x, part, sgpart, d, p, s); break;
+                default: rc = launch_shape<GwChan4>(gy, x, part, sgpart, d, p, s); break;
+            }
         }
         if (rc) return rc;
         const int nb = (int)ceil_div_l(n, kFinOut);

@@ -288,19 +288,19 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     const int bcol = p % C::BPR;
     const int brow = (p / C::BPR) % (C::TH / 2);
     const int img = p / (C::BPR * (C::TH / 2));
-    const int ci_base = (blockIdx.y * C::CIW + cw) * TM;
+    // as in the stride-1 kernel: the last channel group is shifted down so all TM channels are valid
+    const int ci_first = (blockIdx.y * C::CIW + cw) * TM;
+    const int ci_base = __builtin_amdgcn_readfirstlane(min(ci_first, Ci - TM));
     const int K = Ci * 9;
-    uniform_f32_ptr wc = as_uniform(w);
+    uniform_f32_ptr wc = as_uniform(w) + ci_base * 9;
 
     const int n = n0 + img, hi0 = h0 + 2 * brow, wi0 = w0 + bcol * TNW;
     const int nc = min(n, N - 1);
 
     float xr[TM][2][TNW], acc[TM][2][TNW];
-    int wofs[TM];
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
-        const int ci = min(ci_base + m, Ci - 1);
-        wofs[m] = __builtin_amdgcn_readfirstlane(ci * 9);
+        const int ci = ci_base + m;
 #pragma unroll
         for (int rp = 0; rp < 2; ++rp) {
             const float *src = x + (((size_t)nc * Ci + ci) * H + min(hi0 + rp, H - 1)) * W;
@@ -327,30 +327,55 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
-#pragma unroll 1
-        for (int cc = 0; cc < ccnt; ++cc) {
-            float gr[2][GSTRIP];
+        // same software pipeline as the stride-1 kernel: units of HM input channels, next unit's
+        // weights and next channel's gy strips requested right after a unit's first instruction
+        constexpr int HM = 2, NU = TM / HM, HW = HM * 9, TERMS = 9 * (TNW / 2);
+        static_assert(TM % HM == 0 && NU % 2 == 0, "even number of units per output channel");
+        // (row parity, tap row i, gy row) and (col parity, tap col j, gy col offset)
+        constexpr int RP[3] = {0, 1, 1}, RI[3] = {1, 0, 2}, RG[3] = {0, 1, 0};
+        float gr[2][2][GSTRIP];
+        float wv[2][HW];
 #pragma unroll
-            for (int r = 0; r < 2; ++r) lds_read_strip<GSTRIP, 1>(lbase + cc * C::PLANE + r * C::PITCH, gr[r]);
+        for (int r = 0; r < 2; ++r) lds_read_strip<GSTRIP, 1>(lbase + r * C::PITCH, gr[0][r]);
+#pragma unroll
+        for (int e = 0; e < HW; ++e) wv[0][e] = wc[co0 * K + e];
+
+        auto one_channel = [&](const int cc, const int cur) {
             const int kofs = (co0 + cc) * K;
+            const bool more = cc + 1 < ccnt;
+            const int knext = more ? kofs + K : kofs;
 #pragma unroll
-            for (int m = 0; m < TM; ++m) {
-                float wv[9];
+            for (int h = 0; h < NU; ++h) {
 #pragma unroll
-                for (int e = 0; e < 9; ++e) wv[e] = wc[kofs + wofs[m] + e];
-                // (row parity, tap row i, gy row) and (col parity, tap col j, gy col offset)
-                constexpr int RP[3] = {0, 1, 1}, RI[3] = {1, 0, 2}, RG[3] = {0, 1, 0};
+                for (int idx = 0; idx < HM * TERMS; ++idx) {
+                    const int cp = idx % (TNW / 2), bb = (idx / (TNW / 2)) % 3, a = (idx / (TNW / 2) / 3) % 3,
+                              mm = idx / TERMS;
+                    const int m = h * HM + mm, t = 2 * cp + RP[bb];
+                    acc[m][RP[a]][t] = fmaf(hardtanh(wv[h & 1][mm * 9 + RI[a] * 3 + RI[bb]] - xr[m][RP[a]][t]),
+                                            gr[cur][RG[a]][cp + RG[bb]], acc[m][RP[a]][t]);
+                    if (idx == 0) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (h + 1 < NU) {
 #pragma unroll
-                for (int a = 0; a < 3; ++a)
+                            for (int e = 0; e < HW; ++e) wv[(h + 1) & 1][e] = wc[kofs + (h + 1) * HW + e];
+                        } else {
 #pragma unroll
-                    for (int bb = 0; bb < 3; ++bb)
-#pragma unroll
-                        for (int cp = 0; cp < TNW / 2; ++cp) {
-                            const int t = 2 * cp + RP[bb];
-                            acc[m][RP[a]][t] = fmaf(hardtanh(wv[RI[a] * 3 + RI[bb]] - xr[m][RP[a]][t]),
-                                                    gr[RG[a]][cp + RG[bb]], acc[m][RP[a]][t]);
+                            for (int e = 0; e < HW; ++e) wv[0][e] = wc[knext + e];
                         }
+                        if (h == 0 && more) {
+#pragma unroll
+                            for (int r = 0; r < 2; ++r)
+                                lds_read_strip<GSTRIP, 1>(lbase + (cc + 1) * C::PLANE + r * C::PITCH, gr[cur ^ 1][r]);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
             }
+        };
+#pragma unroll 1
+        for (int cc = 0; cc < ccnt; cc += 2) {
+            one_channel(cc, 0);
+            if (cc + 1 < ccnt) one_channel(cc + 1, 1);
         }
 
         if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
@@ -361,7 +386,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
             const int ci = ci_base + m;
-            if (ci >= Ci) continue;
+            if (ci < ci_first) continue;
 #pragma unroll
             for (int rp = 0; rp < 2; ++rp) {
                 const int hi = hi0 + rp;
@@ -395,8 +420,8 @@ static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, 
 }
 
 //                              TNW BPR TH NIMG TM CIW CC
-using GxS2W32 = GradX3x3S2Cfg<2, 16, 32, 1, 8, 2, 16>;   // inputs 32 wide
-using GxS2W16 = GradX3x3S2Cfg<2, 8, 16, 1, 8, 4, 16>;    // inputs 16 wide
+using GxS2W32 = GradX3x3S2Cfg<2, 16, 32, 1, 4, 4, 16>;   // inputs 32 wide: one image x 16 channels, 16 waves
+using GxS2W16 = GradX3x3S2Cfg<2, 8, 16, 1, 4, 8, 16>;    // inputs 16 wide: one image x 32 channels, 8 waves
 
 //                        TN SPR TH NIMG TM COW CC CQ
 using GxW32 = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1>;
@@ -412,7 +437,7 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s);
     }
-    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.Wo % 4 == 0 && d.W % 2 == 0 &&
+    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.Wo % 4 == 0 && d.W % 2 == 0 && d.Ci >= 8 &&
         (reinterpret_cast<uintptr_t>(gy) & 15) == 0 && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
         if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s);

@@ -40,7 +40,8 @@ struct TileStage {
 
 // Issue the global loads of one channel chunk into registers.  src is
 // (nimg_total, nchan, H, W); (hb, wb) is the source position of the first
-// interior element of the patch.  Everything outside the tensor reads as zero.
+// interior element of the patch.  Everything outside the tensor reads as zero.  Index arithmetic is
+// 32-bit: the C ABI refuses tensors of 2^31 elements or more.
 template <class P>
 __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__restrict__ src,
                                            int chan0, int nchan, int n0, int nimg_total, int hb,
@@ -57,7 +58,7 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
         const bool ok = (P::NUV % P::NTHREADS == 0 || u < P::NUV) && n < nimg_total && ch < nchan &&
                         hi >= 0 && hi < H && wi < W;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok) val = *reinterpret_cast<const float4 *>(src + (((size_t)n * nchan + ch) * H + hi) * W + wi);
+        if (ok) val = *reinterpret_cast<const float4 *>(src + (((n * nchan + ch) * H + hi) * W + wi));
         st.v[it] = val;
     }
 #pragma unroll
@@ -71,7 +72,7 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
         const int n = n0 + img, ch = chan0 + cc, hi = hb + r, wi = side ? wb + P::ICOLS : wb - 1;
         const bool ok = (P::NUH % P::NTHREADS == 0 || u < P::NUH) && n < nimg_total && ch < nchan &&
                         hi >= 0 && hi < H && wi >= 0 && wi < W;
-        st.h[it] = ok ? src[(((size_t)n * nchan + ch) * H + hi) * W + wi] : 0.f;
+        st.h[it] = ok ? src[((n * nchan + ch) * H + hi) * W + wi] : 0.f;
     }
 }
 
