@@ -24,12 +24,16 @@ __global__ __launch_bounds__(256) void col_fwd_kernel(const float *__restrict__ 
     int wrow[TM];
 #pragma unroll
     for (int m = 0; m < TM; ++m) wrow[m] = min(co0 + m, Co - 1) * K;
-    float acc[TM];
+    float acc[TM], tot[TM];   // two-level sum: acc holds at most 64 rows of X
 #pragma unroll
-    for (int m = 0; m < TM; ++m) acc[m] = 0.f;
+    for (int m = 0; m < TM; ++m) acc[m] = tot[m] = 0.f;
     const float *xp = X + nl;
     int k = 0;
     for (; k + 4 <= K; k += 4) {
+        if ((k & 63) == 0) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m) { tot[m] += acc[m]; acc[m] = 0.f; }
+        }
         float xv[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) xv[e] = xp[(size_t)(k + e) * NL];
@@ -46,7 +50,7 @@ __global__ __launch_bounds__(256) void col_fwd_kernel(const float *__restrict__ 
     if (active) {
 #pragma unroll
         for (int m = 0; m < TM; ++m)
-            if (co0 + m < Co) out[(size_t)(co0 + m) * NL + nl] = acc[m];
+            if (co0 + m < Co) out[(size_t)(co0 + m) * NL + nl] = tot[m] + acc[m];
     }
 }
 
@@ -61,23 +65,27 @@ __global__ __launch_bounds__(256) void col_grad_x_kernel(const float *__restrict
     if (!active) nl = NL - 1;
     const int k0 = blockIdx.y * TK;
     uniform_f32_ptr wc = as_uniform(Wm);
-    float xv[TK], acc[TK];
+    float xv[TK], acc[TK], tot[TK];   // two-level sum: acc holds at most 64 rows of W
     int kk[TK];
 #pragma unroll
     for (int t = 0; t < TK; ++t) {
         kk[t] = min(k0 + t, K - 1);
         xv[t] = X[(size_t)kk[t] * NL + nl];
-        acc[t] = 0.f;
+        acc[t] = tot[t] = 0.f;
     }
     for (int co = 0; co < Co; ++co) {
         const float g = gy[(size_t)co * NL + nl];
 #pragma unroll
         for (int t = 0; t < TK; ++t) acc[t] = fmaf(hardtanh(wc[co * K + kk[t]] - xv[t]), g, acc[t]);
+        if ((co & 63) == 63) {
+#pragma unroll
+            for (int t = 0; t < TK; ++t) { tot[t] += acc[t]; acc[t] = 0.f; }
+        }
     }
     if (active) {
 #pragma unroll
         for (int t = 0; t < TK; ++t)
-            if (k0 + t < K) gX[(size_t)(k0 + t) * NL + nl] += acc[t];
+            if (k0 + t < K) gX[(size_t)(k0 + t) * NL + nl] += tot[t] + acc[t];
     }
 }
 

@@ -40,16 +40,22 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
     int wrow[TM];
 #pragma unroll
     for (int m = 0; m < TM; ++m) wrow[m] = min(co0 + m, Co - 1) * Ci;
-    float acc[TM][TN];
+    float acc[TM][TN], tot[TM][TN];   // two-level sum: acc holds at most 64 channels
 #pragma unroll
     for (int m = 0; m < TM; ++m)
 #pragma unroll
-        for (int t = 0; t < TN; ++t) acc[m][t] = 0.f;
+        for (int t = 0; t < TN; ++t) acc[m][t] = tot[m][t] = 0.f;
 
     const size_t plane = (size_t)H * W;
     const float *xp = x + (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
     int ci = 0;
     for (; ci + 4 <= Ci; ci += 4) {
+        if ((ci & 63) == 0) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m)
+#pragma unroll
+                for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+        }
         float4 xv[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) xv[e] = *reinterpret_cast<const float4 *>(xp + (size_t)(ci + e) * plane);
@@ -73,15 +79,19 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
             for (int t = 0; t < TN; ++t) acc[m][t] -= fabsf(wv - xs[t * S]);
         }
     }
+#pragma unroll
+    for (int m = 0; m < TM; ++m)
+#pragma unroll
+        for (int t = 0; t < TN; ++t) tot[m][t] += acc[m][t];
     if (L.ok) {
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
             if (co0 + m >= Co) continue;
             float *dst = y + (((size_t)L.n * Co + co0 + m) * Ho + L.ho) * Wo + L.wo0;
             if constexpr (TN == 4)
-                *reinterpret_cast<float4 *>(dst) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+                *reinterpret_cast<float4 *>(dst) = make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]);
             else
-                *reinterpret_cast<float2 *>(dst) = make_float2(acc[m][0], acc[m][1]);
+                *reinterpret_cast<float2 *>(dst) = make_float2(tot[m][0], tot[m][1]);
         }
     }
 }
@@ -98,13 +108,13 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
     uniform_f32_ptr wc = as_uniform(w);
     const size_t plane = (size_t)H * W;
     const size_t xoff = (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
-    float xr[TM][TN], acc[TM][TN];
+    float xr[TM][TN], acc[TM][TN], tot[TM][TN];   // two-level sum: acc holds at most 64 output channels
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const float4 v = *reinterpret_cast<const float4 *>(x + xoff + (size_t)min(ci0 + m, Ci - 1) * plane);
         const float xs[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int t = 0; t < TN; ++t) { xr[m][t] = xs[t * S]; acc[m][t] = 0.f; }
+        for (int t = 0; t < TN; ++t) { xr[m][t] = xs[t * S]; acc[m][t] = tot[m][t] = 0.f; }
     }
     const size_t gplane = (size_t)Ho * Wo;
     const float *gp = gy + (size_t)L.n * Co * gplane + (size_t)L.ho * Wo + L.wo0;
@@ -123,6 +133,12 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
 #pragma unroll
             for (int t = 0; t < TN; ++t) acc[m][t] = fmaf(hardtanh(wv - xr[m][t]), g[t], acc[m][t]);
         }
+        if ((co & 63) == 63 || co + 1 == Co) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m)
+#pragma unroll
+                for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+        }
     }
     if (L.ok) {
         const bool row2 = S == 2 && L.ho * 2 + 1 < H;  // the odd row below: never sampled by stride 2
@@ -131,9 +147,9 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
             if (ci0 + m >= Ci) continue;
             float *dst = gx + xoff + (size_t)(ci0 + m) * plane;
             if constexpr (S == 1) {
-                *reinterpret_cast<float4 *>(dst) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+                *reinterpret_cast<float4 *>(dst) = make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]);
             } else {
-                *reinterpret_cast<float4 *>(dst) = make_float4(acc[m][0], 0.f, acc[m][1], 0.f);
+                *reinterpret_cast<float4 *>(dst) = make_float4(tot[m][0], 0.f, tot[m][1], 0.f);
                 if (row2) *reinterpret_cast<float4 *>(dst + W) = make_float4(0.f, 0.f, 0.f, 0.f);
             }
         }

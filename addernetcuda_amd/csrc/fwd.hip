@@ -37,9 +37,9 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
     const int K = d.K();
     uniform_f32_ptr wc = as_uniform(w);
 
-    float acc[TM];
+    float acc[TM], tot[TM];   // acc: at most 16 channels' taps, tot: the rest (keeps fp32 error small for large K)
 #pragma unroll
-    for (int m = 0; m < TM; ++m) acc[m] = 0.f;
+    for (int m = 0; m < TM; ++m) acc[m] = tot[m] = 0.f;
 
     int wrow[TM];
 #pragma unroll
@@ -59,11 +59,15 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
                 for (int m = 0; m < TM; ++m) acc[m] -= fabsf(wc[wrow[m] + k] - xv);
             }
         }
+        if ((ci & 15) == 15 || ci + 1 == d.Ci) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m) { tot[m] += acc[m]; acc[m] = 0.f; }
+        }
     }
     if (active) {
 #pragma unroll
         for (int m = 0; m < TM; ++m)
-            if (co0 + m < d.Co) y[(((size_t)n * d.Co + co0 + m) * d.Ho + ho) * d.Wo + wo] = acc[m];
+            if (co0 + m < d.Co) y[(((size_t)n * d.Co + co0 + m) * d.Ho + ho) * d.Wo + wo] = tot[m];
     }
 }
 
@@ -113,11 +117,13 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     for (int m = 0; m < TM; ++m)
         wrow[m] = __builtin_amdgcn_readfirstlane(min(co_base + m, Co - 1) * K);
 
-    float acc[TM][TN];
+    // two-level sum: `acc` collects one channel chunk (<= 9*CC terms), `tot` the chunks, so the
+    // rounding error grows with the square roots of the two lengths instead of with K
+    float acc[TM][TN], tot[TM][TN];
 #pragma unroll
     for (int m = 0; m < TM; ++m)
 #pragma unroll
-        for (int t = 0; t < TN; ++t) acc[m][t] = 0.f;
+        for (int t = 0; t < TN; ++t) acc[m][t] = tot[m][t] = 0.f;
 
     const int lane_off = img * C::CC * C::PLANE + row * S * C::PITCH + strip * TN * S;
     const int nchunks = ceil_div(Ci, C::CC);
@@ -187,6 +193,11 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
             if (cc + CQ < ccnt) half(cc + CQ, 1);
         }
 
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+#pragma unroll
+            for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+
         if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
         __syncthreads();
     }
@@ -203,11 +214,11 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
 #pragma unroll
                     for (int t = 0; t + 3 < TN; t += 4)
                         *reinterpret_cast<float4 *>(dst + t) =
-                            make_float4(acc[m][t], acc[m][t + 1], acc[m][t + 2], acc[m][t + 3]);
+                            make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]);
                 } else {
 #pragma unroll
                     for (int t = 0; t < TN; ++t)
-                        if (wo + t < Wo) dst[t] = acc[m][t];
+                        if (wo + t < Wo) dst[t] = tot[m][t];
                 }
             }
         }

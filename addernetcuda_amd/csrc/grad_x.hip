@@ -36,13 +36,13 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
     const int K = d.Ci * KK;
     uniform_f32_ptr wc = as_uniform(w);
 
-    float xr[TM], acc[TM];
+    float xr[TM], acc[TM], tot[TM];   // two-level sum: acc holds at most 16 output channels' taps
     int wofs[TM];
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = min(ci0 + m, d.Ci - 1);
         xr[m] = x[(((size_t)n * d.Ci + ci) * d.H + hi) * d.W + wi];
-        acc[m] = 0.f;
+        acc[m] = tot[m] = 0.f;
         wofs[m] = ci * KK;
     }
     const float *gn = gy + (size_t)n * d.Co * d.Ho * d.Wo;
@@ -62,11 +62,15 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
                     acc[m] = fmaf(hardtanh(wc[kofs + wofs[m]] - xr[m]), g, acc[m]);
             }
         }
+        if ((co & 15) == 15 || co + 1 == d.Co) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m) { tot[m] += acc[m]; acc[m] = 0.f; }
+        }
     }
     if (active) {
 #pragma unroll
         for (int m = 0; m < TM; ++m)
-            if (ci0 + m < d.Ci) gx[(((size_t)n * d.Ci + ci0 + m) * d.H + hi) * d.W + wi] = acc[m];
+            if (ci0 + m < d.Ci) gx[(((size_t)n * d.Ci + ci0 + m) * d.H + hi) * d.W + wi] = tot[m];
     }
 }
 
@@ -115,7 +119,8 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     const int nc = min(n, N - 1), hc = min(hi, H - 1);
 
     // own x values and accumulators live in registers for the whole kernel
-    float xr[TM][TN], acc[TM][TN];
+    // (two-level sum: acc collects one chunk of output channels, tot the chunks)
+    float xr[TM][TN], acc[TM][TN], tot[TM][TN];
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
@@ -123,7 +128,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
             xr[m][t] = src[min(wi0 + t, W - 1)];
-            acc[m][t] = 0.f;
+            acc[m][t] = tot[m][t] = 0.f;
         }
     }
 
@@ -195,6 +200,11 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
             if (cc + 1 < ccnt) one_channel(cc + 1, 1);
         }
 
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+#pragma unroll
+            for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+
         if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
         __syncthreads();
     }
@@ -209,11 +219,11 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
 #pragma unroll
                     for (int t = 0; t < TN; t += 4)
                         *reinterpret_cast<float4 *>(dst + t) =
-                            make_float4(acc[m][t], acc[m][t + 1], acc[m][t + 2], acc[m][t + 3]);
+                            make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]);
                 } else {
 #pragma unroll
                     for (int t = 0; t < TN; ++t)
-                        if (wi0 + t < W) dst[t] = acc[m][t];
+                        if (wi0 + t < W) dst[t] = tot[m][t];
                 }
             }
         }
@@ -297,7 +307,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     const int n = n0 + img, hi0 = h0 + 2 * brow, wi0 = w0 + bcol * TNW;
     const int nc = min(n, N - 1);
 
-    float xr[TM][2][TNW], acc[TM][2][TNW];
+    float xr[TM][2][TNW], acc[TM][2][TNW], tot[TM][2][TNW];
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
@@ -307,7 +317,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 #pragma unroll
             for (int t = 0; t < TNW; ++t) {
                 xr[m][rp][t] = src[min(wi0 + t, W - 1)];
-                acc[m][rp][t] = 0.f;
+                acc[m][rp][t] = tot[m][rp][t] = 0.f;
             }
         }
     }
@@ -378,6 +388,13 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
             if (cc + 1 < ccnt) one_channel(cc + 1, 1);
         }
 
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+#pragma unroll
+            for (int rp = 0; rp < 2; ++rp)
+#pragma unroll
+                for (int t = 0; t < TNW; ++t) { tot[m][rp][t] += acc[m][rp][t]; acc[m][rp][t] = 0.f; }
+
         if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
         __syncthreads();
     }
@@ -395,11 +412,11 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
                 if ((W & 1) == 0 && wi0 + TNW <= W) {
 #pragma unroll
                     for (int t = 0; t < TNW; t += 2)
-                        *reinterpret_cast<float2 *>(dst + t) = make_float2(acc[m][rp][t], acc[m][rp][t + 1]);
+                        *reinterpret_cast<float2 *>(dst + t) = make_float2(tot[m][rp][t], tot[m][rp][t + 1]);
                 } else {
 #pragma unroll
                     for (int t = 0; t < TNW; ++t)
-                        if (wi0 + t < W) dst[t] = acc[m][rp][t];
+                        if (wi0 + t < W) dst[t] = tot[m][rp][t];
                 }
             }
         }

@@ -1,0 +1,42 @@
+"""Layer shapes of the other reference models (VGG-small-style stack, ResNet-50 bottlenecks, DenseNet-BC)
+at reduced batch against the float64 C oracle: large K (up to 4608), 1x1 and strided layers on
+56/28/14/7-wide maps, 12-channel growth, the 3-channel VGG stem."""
+import pytest
+import torch
+
+from tests.util import make_case, assert_close
+
+pytestmark = pytest.mark.gpu
+
+# (N, Ci, H, W, Co, k, stride, pad)
+SHAPES = [
+    (2, 128, 32, 32, 128, 3, 1, 1),    # VGG-small 128->128 @32, K = 1152
+    (2, 256, 16, 16, 256, 3, 1, 1),    # K = 2304
+    (2, 512, 8, 8, 512, 3, 1, 1),      # K = 4608
+    (2, 3, 32, 32, 64, 3, 1, 1),       # vgg.py:60-66: the 3-channel stem is an adder layer too
+    (1, 64, 56, 56, 64, 3, 1, 1),      # ResNet-50 3x3 @56
+    (1, 64, 56, 56, 256, 1, 1, 0),     # 1x1 expand @56
+    (1, 256, 56, 56, 512, 1, 2, 0),    # 1x1 stride-2 downsample 56 -> 28
+    (1, 128, 56, 56, 128, 3, 2, 1),    # strided 3x3 56 -> 28
+    (2, 256, 14, 14, 256, 3, 1, 1),    # 14-wide maps (W % 4 != 0)
+    (2, 1024, 14, 14, 256, 1, 1, 0),   # 1x1 reduce @14, K = 1024
+    (2, 512, 7, 7, 512, 3, 1, 1),      # 7-wide maps
+    (2, 2048, 7, 7, 512, 1, 1, 0),     # K = 2048
+    (3, 24, 32, 32, 48, 1, 1, 0),      # DenseNet-BC bottleneck 1x1 (densenet.py:12-14)
+    (3, 48, 32, 32, 12, 3, 1, 1),      # DenseNet-BC growth conv, Co = 12
+]
+
+
+@pytest.mark.parametrize("case", SHAPES, ids=str)
+def test_layer_matches_oracle(case, gpu):
+    from addernetcuda_amd import adder
+    from oracle import c_oracle
+    s, p = case[6], case[7]
+    x, w, gy = make_case(*case, w_init="normal")          # adder2d's own N(0,1) init (adder.py:97)
+    xg, wg = x.to(gpu).requires_grad_(True), w.to(gpu).requires_grad_(True)
+    y = adder.adder2d_function(xg, wg, s, p, eta=0.0)
+    y.backward(gy.to(gpu))
+    torch.cuda.synchronize()
+    assert_close(y, c_oracle.conv2d_fwd(x, w, s, p), f"forward {case}")
+    assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p), f"grad_X {case}")
+    assert_close(wg.grad, c_oracle.conv2d_grad_w(gy, x, w, s, p), f"grad_W {case}")
