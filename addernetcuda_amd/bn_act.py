@@ -1,0 +1,88 @@
+"""BatchNorm2d fused with the residual add and ReLU that follow every adder layer.
+
+``BatchNormAct2d`` is an ``nn.BatchNorm2d`` (same parameters, buffers and state_dict keys) whose
+training-mode forward on the GPU runs as two HIP passes, statistics then
+``relu(gamma * (x - mean) * rstd + beta [+ residual])``, and whose backward is two more; see
+csrc/bn_act.hip.  It replaces the separate bn / += residual / relu ops of resnet20.py:28-39.
+Anything the fused kernels do not cover (eval mode, CPU tensors, non-fp32) goes through the
+ordinary torch ops with identical semantics.
+"""
+import ctypes
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.autograd import Function
+
+from ._lib import lib, check, ptr, stream_ptr
+
+
+def _workspace(N, C, HW, device):
+    need = ctypes.c_size_t(0)
+    check(lib.adder_bn_act_workspace_bytes(N, C, HW, ctypes.byref(need)), "adder_bn_act_workspace_bytes")
+    return torch.empty(max(need.value, 256), dtype=torch.uint8, device=device), need.value
+
+
+class _bn_act(Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, residual, running_mean, running_var, momentum, eps, relu):
+        x = x.contiguous()
+        if residual is not None:
+            residual = residual.contiguous()
+        N, C = x.shape[0], x.shape[1]
+        HW = x.numel() // (N * C)
+        dev = x.device
+        y = torch.empty_like(x)
+        mean = torch.empty(C, dtype=torch.float32, device=dev)
+        rstd = torch.empty(C, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            ws, nbytes = _workspace(N, C, HW, dev)
+            check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mean), ptr(rstd),
+                                           ptr(running_mean), ptr(running_var), float(momentum), float(eps), int(relu),
+                                           N, C, HW, ptr(ws), nbytes, stream_ptr(dev)), "adder_bn_act_fwd_f32")
+        ctx.save_for_backward(x, y if relu else None, weight, mean, rstd)
+        ctx.relu, ctx.has_res, ctx.dims = relu, residual is not None, (N, C, HW)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, y, weight, mean, rstd = ctx.saved_tensors
+        dy = dy.contiguous()
+        N, C, HW = ctx.dims
+        dev = x.device
+        dx = torch.empty_like(x)
+        dres = torch.empty_like(x) if ctx.has_res else None
+        dgamma, dbeta = torch.empty_like(weight), torch.empty_like(weight)
+        with torch.cuda.device(dev):
+            ws, nbytes = _workspace(N, C, HW, dev)
+            check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
+                                           ptr(dres), ptr(dgamma), ptr(dbeta), int(ctx.relu), N, C, HW, ptr(ws), nbytes,
+                                           stream_ptr(dev)), "adder_bn_act_bwd_f32")
+        return dx, dgamma, dbeta, dres, None, None, None, None, None
+
+
+class BatchNormAct2d(nn.BatchNorm2d):
+    """``y = act(batch_norm(x) [+ residual])`` with ``act`` = ReLU when ``relu`` is set."""
+
+    def __init__(self, num_features, relu=True, **kwargs):
+        super().__init__(num_features, **kwargs)
+        self.relu = relu
+
+    def _fusable(self, x):
+        return (self.training and x.is_cuda and x.dtype == torch.float32 and self.affine and x.dim() == 4
+                and self.weight.dtype == torch.float32)
+
+    def forward(self, x, residual=None):
+        if not self._fusable(x):
+            out = super().forward(x)
+            if residual is not None:
+                out = out + residual
+            return F.relu(out) if self.relu else out
+        momentum = self.momentum
+        if self.track_running_stats:
+            self.num_batches_tracked.add_(1)
+            if momentum is None:  # cumulative moving average, as nn.BatchNorm2d defines it
+                momentum = 1.0 / float(self.num_batches_tracked)
+        rm = self.running_mean if self.track_running_stats else None
+        rv = self.running_var if self.track_running_stats else None
+        return _bn_act.apply(x, self.weight, self.bias, residual, rm, rv, momentum, self.eps, self.relu)

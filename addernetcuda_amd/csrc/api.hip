@@ -199,4 +199,43 @@ int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps, void *ws, 
     return launch_norm_scale(g, n, eta, eps, ws, static_cast<hipStream_t>(stream));
 }
 
+static int check_bn(int N, int C, int HW) {
+    if (N <= 0 || C <= 0 || HW <= 0) return ADDER_ERR_BAD_SHAPE;
+    if ((long)N * C * HW > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    return ADDER_OK;
+}
+
+int adder_bn_act_workspace_bytes(int N, int C, int HW, size_t *bytes) {
+    if (!bytes) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_bn(N, C, HW)) return rc;
+    *bytes = bn_workspace_bytes(N, C, HW);
+    return ADDER_OK;
+}
+
+int adder_bn_act_fwd_f32(const float *x, const float *residual, const float *gamma, const float *beta, float *y,
+                         float *save_mean, float *save_rstd, float *running_mean, float *running_var,
+                         float momentum, float eps, int relu, int N, int C, int HW, void *ws, size_t ws_bytes,
+                         void *stream) {
+    if (!x || !gamma || !beta || !y || !save_mean || !save_rstd) return ADDER_ERR_NULL_POINTER;
+    if ((running_mean == nullptr) != (running_var == nullptr)) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_bn(N, C, HW)) return rc;
+    if (!(eps > 0.f) || !(momentum >= 0.f && momentum <= 1.f)) return ADDER_ERR_BAD_SHAPE;
+    if (!ws || ws_bytes < bn_workspace_bytes(N, C, HW) || (reinterpret_cast<uintptr_t>(ws) & 255))
+        return ADDER_ERR_WORKSPACE;
+    return launch_bn_act_fwd(x, residual, gamma, beta, y, save_mean, save_rstd, running_mean, running_var, momentum,
+                             eps, relu != 0, N, C, HW, ws, static_cast<hipStream_t>(stream));
+}
+
+int adder_bn_act_bwd_f32(const float *dy, const float *y, const float *x, const float *gamma, const float *save_mean,
+                         const float *save_rstd, float *dx, float *dresidual, float *dgamma, float *dbeta, int relu,
+                         int N, int C, int HW, void *ws, size_t ws_bytes, void *stream) {
+    if (!dy || !x || !gamma || !save_mean || !save_rstd || !dx || !dgamma || !dbeta) return ADDER_ERR_NULL_POINTER;
+    if (relu && !y) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_bn(N, C, HW)) return rc;
+    if (!ws || ws_bytes < bn_workspace_bytes(N, C, HW) || (reinterpret_cast<uintptr_t>(ws) & 255))
+        return ADDER_ERR_WORKSPACE;
+    return launch_bn_act_bwd(dy, y, x, gamma, save_mean, save_rstd, dx, dresidual, dgamma, dbeta, relu != 0, N, C, HW,
+                             ws, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

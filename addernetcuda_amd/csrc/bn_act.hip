@@ -1,0 +1,250 @@
+// Training-mode BatchNorm2d fused with the residual add and ReLU that follow every adder layer
+// (resnet20.py:28-39: out = relu(bn(conv(x)) [+ residual])).  After the adder kernels these
+// element-wise neighbours dominate a training step; they are HBM-bound, so the point of the fusion
+// is to touch each activation as few times as possible:
+//   forward   pass 1  per-channel sum / sum of squares (fp64)            reads x
+//             pass 2  y = relu(gamma * (x - mean) * rstd + beta + res)    reads x (+ res), writes y
+//   backward  pass 1  per-channel sum(dz), sum(dz * xhat), dz = dy * [y > 0]      reads dy, y, x
+//             pass 2  dx = gamma * rstd * (dz - mean(dz) - xhat * mean(dz * xhat)),
+//                     dres = dz                                           reads dy, y, x, writes dx (+ dres)
+// Statistics follow torch.nn.BatchNorm2d: biased variance for normalisation, unbiased for running_var.
+#include "common.hpp"
+
+namespace adder {
+
+static constexpr int kBnThreads = 256;
+
+// V consecutive floats (V = 4 when HW is a multiple of 4, else 1)
+template <int V> struct Pack { float v[V]; };
+template <int V> __device__ __forceinline__ Pack<V> ld(const float *p, size_t i) {
+    Pack<V> r;
+    if constexpr (V == 4) {
+        const float4 t = reinterpret_cast<const float4 *>(p)[i];
+        r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+    } else {
+        r.v[0] = p[i];
+    }
+    return r;
+}
+template <int V> __device__ __forceinline__ void st(float *p, size_t i, const Pack<V> &r) {
+    if constexpr (V == 4) reinterpret_cast<float4 *>(p)[i] = make_float4(r.v[0], r.v[1], r.v[2], r.v[3]);
+    else p[i] = r.v[0];
+}
+
+// Per-channel partial sums.  grid = (S, C); block (s, c) walks over the float4 groups
+// i = s*256 + tid, s*256 + tid + S*256, ... of channel c (i = n * HW/4 + q).
+template <bool BWD, int V>
+__global__ __launch_bounds__(kBnThreads) void bn_partial_kernel(const float *__restrict__ x,
+                                                                const float *__restrict__ dy,
+                                                                const float *__restrict__ y,
+                                                                const float *__restrict__ mean,
+                                                                const float *__restrict__ rstd, int relu,
+                                                                int N, int C, int HW4 /* HW / V */,
+                                                                double *__restrict__ part) {
+    const int c = blockIdx.y, S = gridDim.x;
+    const int total = N * HW4;
+    float mu = 0.f, rs = 0.f;
+    if (BWD) { mu = mean[c]; rs = rstd[c]; }
+    double a = 0.0, b = 0.0;
+    for (int i0 = blockIdx.x * kBnThreads; i0 < total; i0 += S * kBnThreads) {
+        const int i = i0 + threadIdx.x;
+        float s1 = 0.f, s2 = 0.f;
+        if (i < total) {
+            const int n = i / HW4, q = i - n * HW4;
+            const size_t off = ((size_t)n * C + c) * HW4 + q;
+            const Pack<V> xv = ld<V>(x, off);
+            if (!BWD) {
+#pragma unroll
+                for (int e = 0; e < V; ++e) { s1 += xv.v[e]; s2 = fmaf(xv.v[e], xv.v[e], s2); }
+            } else {
+                Pack<V> g = ld<V>(dy, off);
+                if (relu) {
+                    const Pack<V> yv = ld<V>(y, off);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) g.v[e] = yv.v[e] > 0.f ? g.v[e] : 0.f;
+                }
+#pragma unroll
+                for (int e = 0; e < V; ++e) { s1 += g.v[e]; s2 = fmaf(g.v[e], (xv.v[e] - mu) * rs, s2); }
+            }
+        }
+        a += (double)s1;   // at most four elements per fp32 partial, everything above in fp64
+        b += (double)s2;
+    }
+    __shared__ double ra[kBnThreads / 64], rb[kBnThreads / 64];
+    a = wave_sum(a);
+    b = wave_sum(b);
+    if ((threadIdx.x & 63) == 0) { ra[threadIdx.x >> 6] = a; rb[threadIdx.x >> 6] = b; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        part[((size_t)c * S + blockIdx.x) * 2 + 0] = (ra[0] + ra[1]) + (ra[2] + ra[3]);
+        part[((size_t)c * S + blockIdx.x) * 2 + 1] = (rb[0] + rb[1]) + (rb[2] + rb[3]);
+    }
+}
+
+// One thread per channel: mean, rstd, running statistics.
+__global__ void bn_fwd_finalize_kernel(const double *__restrict__ part, int S, int C, double count, float eps,
+                                       float momentum, float *__restrict__ mean, float *__restrict__ rstd,
+                                       float *__restrict__ running_mean, float *__restrict__ running_var) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    double s1 = 0.0, s2 = 0.0;
+    for (int s = 0; s < S; ++s) { s1 += part[((size_t)c * S + s) * 2]; s2 += part[((size_t)c * S + s) * 2 + 1]; }
+    const double mu = s1 / count;
+    double var = s2 / count - mu * mu;
+    if (var < 0.0) var = 0.0;
+    mean[c] = (float)mu;
+    rstd[c] = (float)(1.0 / sqrt(var + (double)eps));
+    if (running_mean) {
+        const double unbiased = count > 1.0 ? var * count / (count - 1.0) : var;
+        running_mean[c] = (float)((1.0 - momentum) * (double)running_mean[c] + momentum * mu);
+        running_var[c] = (float)((1.0 - momentum) * (double)running_var[c] + momentum * unbiased);
+    }
+}
+
+// One thread per channel: dgamma, dbeta and the two per-channel means the dx pass needs.
+__global__ void bn_bwd_finalize_kernel(const double *__restrict__ part, int S, int C, double count,
+                                       float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                       float *__restrict__ coef /* [C][2]: mean(dz), mean(dz*xhat) */) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    double s1 = 0.0, s2 = 0.0;
+    for (int s = 0; s < S; ++s) { s1 += part[((size_t)c * S + s) * 2]; s2 += part[((size_t)c * S + s) * 2 + 1]; }
+    dbeta[c] = (float)s1;
+    dgamma[c] = (float)s2;
+    coef[2 * c] = (float)(s1 / count);
+    coef[2 * c + 1] = (float)(s2 / count);
+}
+
+template <int V>
+__global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const float *__restrict__ x,
+                                                              const float *__restrict__ res,
+                                                              const float *__restrict__ mean,
+                                                              const float *__restrict__ rstd,
+                                                              const float *__restrict__ gamma,
+                                                              const float *__restrict__ beta, float *__restrict__ y,
+                                                              int relu, int C, int HW4, long total4) {
+    for (long i = (long)blockIdx.x * kBnThreads + threadIdx.x; i < total4; i += (long)gridDim.x * kBnThreads) {
+        const int c = (int)((i / HW4) % C);
+        const float sc = gamma[c] * rstd[c], mu = mean[c], sh = beta[c];
+        const Pack<V> v = ld<V>(x, i);
+        Pack<V> o;
+#pragma unroll
+        for (int e = 0; e < V; ++e) o.v[e] = fmaf(v.v[e] - mu, sc, sh);   // subtract first: |x| >> |x - mean| here
+        if (res) {
+            const Pack<V> r = ld<V>(res, i);
+#pragma unroll
+            for (int e = 0; e < V; ++e) o.v[e] += r.v[e];
+        }
+        if (relu) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) o.v[e] = fmaxf(o.v[e], 0.f);
+        }
+        st<V>(y, i, o);
+    }
+}
+
+template <int V>
+__global__ __launch_bounds__(kBnThreads) void bn_bwd_apply_kernel(const float *__restrict__ dy,
+                                                                  const float *__restrict__ y,
+                                                                  const float *__restrict__ x,
+                                                                  const float *__restrict__ mean,
+                                                                  const float *__restrict__ rstd,
+                                                                  const float *__restrict__ gamma,
+                                                                  const float *__restrict__ coef,
+                                                                  float *__restrict__ dx, float *__restrict__ dres,
+                                                                  int relu, int C, int HW4, long total4) {
+    for (long i = (long)blockIdx.x * kBnThreads + threadIdx.x; i < total4; i += (long)gridDim.x * kBnThreads) {
+        const int c = (int)((i / HW4) % C);
+        const float mu = mean[c], rs = rstd[c], k = gamma[c] * rs, m1 = coef[2 * c], m2 = coef[2 * c + 1];
+        Pack<V> g = ld<V>(dy, i);
+        if (relu) {
+            const Pack<V> yv = ld<V>(y, i);
+#pragma unroll
+            for (int e = 0; e < V; ++e) g.v[e] = yv.v[e] > 0.f ? g.v[e] : 0.f;
+        }
+        if (dres) st<V>(dres, i, g);
+        const Pack<V> v = ld<V>(x, i);
+        Pack<V> o;
+#pragma unroll
+        for (int e = 0; e < V; ++e) o.v[e] = k * (g.v[e] - m1 - (v.v[e] - mu) * rs * m2);
+        st<V>(dx, i, o);
+    }
+}
+
+static int bn_splits(int N, int C, int HW4) {
+    const long per_channel = (long)N * HW4;
+    long s = 2048 / C;                                   // ~2048 workgroups over the chip
+    const long cap = ceil_div_l(per_channel, 4L * kBnThreads);  // at least ~4 float4 per thread
+    if (s > cap) s = cap;
+    return (int)(s < 1 ? 1 : s);
+}
+
+static bool bn_vec4(int HW, const void *a, const void *b, const void *c, const void *d, const void *e) {
+    const uintptr_t m = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c) |
+                        reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(e);
+    return HW % 4 == 0 && (m & 15) == 0;
+}
+
+size_t bn_workspace_bytes(int N, int C, int HW) {
+    // sized for the scalar layout (the larger of the two) so the choice can depend on pointer alignment
+    return (((size_t)C * bn_splits(N, C, HW) * 2 * sizeof(double) + (size_t)C * 2 * sizeof(float)) + 255) &
+           ~(size_t)255;
+}
+
+static int apply_blocks(long total4) {
+    long b = ceil_div_l(total4, kBnThreads);
+    return (int)(b > 16384 ? 16384 : (b < 1 ? 1 : b));
+}
+
+template <int V>
+static int bn_fwd_v(const float *x, const float *res, const float *gamma, const float *beta, float *y, float *mean,
+                    float *rstd, float *running_mean, float *running_var, float momentum, float eps, int relu,
+                    int N, int C, int HW, void *ws, hipStream_t s) {
+    const int HWV = HW / V, S = bn_splits(N, C, HWV);
+    double *part = reinterpret_cast<double *>(ws);
+    hipLaunchKernelGGL((bn_partial_kernel<false, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, nullptr, nullptr, nullptr,
+                       nullptr, 0, N, C, HWV, part);
+    hipLaunchKernelGGL(bn_fwd_finalize_kernel, dim3(ceil_div(C, 64)), dim3(64), 0, s, part, S, C, (double)N * HW, eps,
+                       momentum, mean, rstd, running_mean, running_var);
+    const long total = (long)N * C * HWV;
+    hipLaunchKernelGGL(bn_apply_kernel<V>, dim3(apply_blocks(total)), dim3(kBnThreads), 0, s, x, res, mean, rstd, gamma,
+                       beta, y, relu, C, HWV, total);
+    return check_launch();
+}
+
+int launch_bn_act_fwd(const float *x, const float *res, const float *gamma, const float *beta, float *y,
+                      float *mean, float *rstd, float *running_mean, float *running_var, float momentum,
+                      float eps, int relu, int N, int C, int HW, void *ws, hipStream_t s) {
+    if (bn_vec4(HW, x, res, y, nullptr, nullptr))
+        return bn_fwd_v<4>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, momentum, eps, relu, N, C,
+                           HW, ws, s);
+    return bn_fwd_v<1>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, momentum, eps, relu, N, C, HW,
+                       ws, s);
+}
+
+template <int V>
+static int bn_bwd_v(const float *dy, const float *y, const float *x, const float *gamma, const float *mean,
+                    const float *rstd, float *dx, float *dres, float *dgamma, float *dbeta, int relu, int N, int C,
+                    int HW, void *ws, hipStream_t s) {
+    const int HWV = HW / V, S = bn_splits(N, C, HWV);
+    double *part = reinterpret_cast<double *>(ws);
+    float *coef = reinterpret_cast<float *>(part + (size_t)C * S * 2);
+    hipLaunchKernelGGL((bn_partial_kernel<true, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, dy, y, mean, rstd, relu, N,
+                       C, HWV, part);
+    hipLaunchKernelGGL(bn_bwd_finalize_kernel, dim3(ceil_div(C, 64)), dim3(64), 0, s, part, S, C, (double)N * HW,
+                       dgamma, dbeta, coef);
+    const long total = (long)N * C * HWV;
+    hipLaunchKernelGGL(bn_bwd_apply_kernel<V>, dim3(apply_blocks(total)), dim3(kBnThreads), 0, s, dy, y, x, mean, rstd,
+                       gamma, coef, dx, dres, relu, C, HWV, total);
+    return check_launch();
+}
+
+int launch_bn_act_bwd(const float *dy, const float *y, const float *x, const float *gamma, const float *mean,
+                      const float *rstd, float *dx, float *dres, float *dgamma, float *dbeta, int relu, int N,
+                      int C, int HW, void *ws, hipStream_t s) {
+    if (bn_vec4(HW, dy, y, x, dx, dres))
+        return bn_bwd_v<4>(dy, y, x, gamma, mean, rstd, dx, dres, dgamma, dbeta, relu, N, C, HW, ws, s);
+    return bn_bwd_v<1>(dy, y, x, gamma, mean, rstd, dx, dres, dgamma, dbeta, relu, N, C, HW, ws, s);
+}
+
+}  // namespace adder

@@ -10,10 +10,15 @@ followed by BatchNorm (resnet20.py:55-57,89-93), BatchNorm weights 1 / biases 0
 
 ``adder2d_cls`` lets a caller build the same network around another
 implementation of the layer (the tests do this with their CPU reference).
+
+The BatchNorm layers are ``BatchNormAct2d``: the same module as nn.BatchNorm2d
+(parameters, buffers, state_dict keys) with the ReLU, and in the second half
+of a block the residual add, folded into its GPU kernels.
 """
 import torch.nn as nn
 
 from . import adder as _adder
+from .bn_act import BatchNormAct2d
 
 
 class BasicBlock(nn.Module):
@@ -23,18 +28,17 @@ class BasicBlock(nn.Module):
         super().__init__()
         make = adder2d_cls or _adder.adder2d
         self.conv1 = make(inplanes, planes, kernel_size=3, stride=stride, padding=1, bias=False, **adder_kw)
-        self.bn1 = nn.BatchNorm2d(planes)
-        self.relu = nn.ReLU(inplace=True)
+        self.bn1 = BatchNormAct2d(planes, relu=True)
+        self.relu = nn.ReLU(inplace=True)    # kept for the reference's module layout; the ReLUs run inside bn1 / bn2
         self.conv2 = make(planes, planes, kernel_size=3, stride=1, padding=1, bias=False, **adder_kw)
-        self.bn2 = nn.BatchNorm2d(planes)
+        self.bn2 = BatchNormAct2d(planes, relu=True)
         self.downsample = downsample
         self.stride = stride
 
     def forward(self, x):
-        out = self.relu(self.bn1(self.conv1(x)))
-        out = self.bn2(self.conv2(out))
+        out = self.bn1(self.conv1(x))                                   # bn + relu
         shortcut = x if self.downsample is None else self.downsample(x)
-        return self.relu(out + shortcut)
+        return self.bn2(self.conv2(out), residual=shortcut)             # bn + residual + relu
 
 
 class ResNet(nn.Module):
@@ -44,7 +48,7 @@ class ResNet(nn.Module):
         self._adder_kw = adder_kw
         self.inplanes = 16
         self.conv1 = nn.Conv2d(3, 16, kernel_size=3, stride=1, padding=1, bias=False)
-        self.bn1 = nn.BatchNorm2d(16)
+        self.bn1 = BatchNormAct2d(16, relu=True)
         self.relu = nn.ReLU(inplace=True)
         self.layer1 = self._make_layer(block, 16, layers[0])
         self.layer2 = self._make_layer(block, 32, layers[1], stride=2)
@@ -63,14 +67,14 @@ class ResNet(nn.Module):
             downsample = nn.Sequential(
                 self._make(self.inplanes, planes * block.expansion, kernel_size=1, stride=stride, bias=False,
                            **self._adder_kw),
-                nn.BatchNorm2d(planes * block.expansion))
+                BatchNormAct2d(planes * block.expansion, relu=False))
         stage = [block(self.inplanes, planes, stride, downsample, adder2d_cls=self._make, **self._adder_kw)]
         self.inplanes = planes * block.expansion
         stage += [block(self.inplanes, planes, adder2d_cls=self._make, **self._adder_kw) for _ in range(1, blocks)]
         return nn.Sequential(*stage)
 
     def forward(self, x):
-        x = self.relu(self.bn1(self.conv1(x)))
+        x = self.bn1(self.conv1(x))
         x = self.layer3(self.layer2(self.layer1(x)))
         x = self.bn2(self.fc(self.avgpool(x)))
         return x.view(x.size(0), -1)

@@ -119,6 +119,27 @@ ADDER_API int adder_norm_scale_workspace_bytes(long n, size_t *bytes);
 ADDER_API int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps,
                               void *ws, size_t ws_bytes, void *stream);
 
+/* ------------------------------------------------------------------------
+ * The element-wise neighbours of every adder layer: training-mode BatchNorm2d fused with the
+ * residual add and ReLU that follow it.  The reference runs these as separate PyTorch ops
+ * (resnet20.py:28-39: bn -> relu, bn -> += residual -> relu); here each direction is one
+ * statistics pass and one apply pass.  x, y, residual, dy, dx, dresidual are (N, C, H*W).
+ *   forward : y = act(gamma * (x - mean) * rstd + beta [+ residual]),  act = ReLU if relu != 0
+ *             save_mean / save_rstd (C) are written for the backward; running_mean / running_var
+ *             (nullable, both or neither) are updated with `momentum` (unbiased variance).
+ *   backward: dx, dgamma, dbeta; dresidual (nullable) receives the gradient of the residual input.
+ *             y (the forward output) is needed only when relu != 0.
+ * ---------------------------------------------------------------------- */
+ADDER_API int adder_bn_act_workspace_bytes(int N, int C, int HW, size_t *bytes);
+ADDER_API int adder_bn_act_fwd_f32(const float *x, const float *residual, const float *gamma, const float *beta,
+                                   float *y, float *save_mean, float *save_rstd,
+                                   float *running_mean, float *running_var, float momentum, float eps, int relu,
+                                   int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);
+ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const float *x, const float *gamma,
+                                   const float *save_mean, const float *save_rstd,
+                                   float *dx, float *dresidual, float *dgamma, float *dbeta, int relu,
+                                   int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
