@@ -25,7 +25,7 @@ def _workspace(N, C, HW, device):
 
 class _bn_act(Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, residual, running_mean, running_var, momentum, eps, relu):
+    def forward(ctx, x, weight, bias, residual, running_mean, running_var, num_batches, momentum, eps, relu):
         x = x.contiguous()
         if residual is not None:
             residual = residual.contiguous()
@@ -38,7 +38,8 @@ class _bn_act(Function):
         with torch.cuda.device(dev):
             ws, nbytes = _workspace(N, C, HW, dev)
             check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mean), ptr(rstd),
-                                           ptr(running_mean), ptr(running_var), float(momentum), float(eps), int(relu),
+                                           ptr(running_mean), ptr(running_var), ptr(num_batches), float(momentum), float(eps),
+                                           int(relu),
                                            N, C, HW, ptr(ws), nbytes, stream_ptr(dev)), "adder_bn_act_fwd_f32")
         ctx.save_for_backward(x, y if relu else None, weight, mean, rstd)
         ctx.relu, ctx.has_res, ctx.dims = relu, residual is not None, (N, C, HW)
@@ -58,7 +59,7 @@ class _bn_act(Function):
             check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
                                            ptr(dres), ptr(dgamma), ptr(dbeta), int(ctx.relu), N, C, HW, ptr(ws), nbytes,
                                            stream_ptr(dev)), "adder_bn_act_bwd_f32")
-        return dx, dgamma, dbeta, dres, None, None, None, None, None
+        return dx, dgamma, dbeta, dres, None, None, None, None, None, None
 
 
 class BatchNormAct2d(nn.BatchNorm2d):
@@ -69,8 +70,9 @@ class BatchNormAct2d(nn.BatchNorm2d):
         self.relu = relu
 
     def _fusable(self, x):
+        # momentum=None (cumulative average) needs the batch count on the host: left to torch
         return (self.training and x.is_cuda and x.dtype == torch.float32 and self.affine and x.dim() == 4
-                and self.weight.dtype == torch.float32)
+                and self.weight.dtype == torch.float32 and self.momentum is not None)
 
     def forward(self, x, residual=None):
         if not self._fusable(x):
@@ -78,11 +80,7 @@ class BatchNormAct2d(nn.BatchNorm2d):
             if residual is not None:
                 out = out + residual
             return F.relu(out) if self.relu else out
-        momentum = self.momentum
-        if self.track_running_stats:
-            self.num_batches_tracked.add_(1)
-            if momentum is None:  # cumulative moving average, as nn.BatchNorm2d defines it
-                momentum = 1.0 / float(self.num_batches_tracked)
         rm = self.running_mean if self.track_running_stats else None
         rv = self.running_var if self.track_running_stats else None
-        return _bn_act.apply(x, self.weight, self.bias, residual, rm, rv, momentum, self.eps, self.relu)
+        nb = self.num_batches_tracked if self.track_running_stats else None   # advanced inside the kernel
+        return _bn_act.apply(x, self.weight, self.bias, residual, rm, rv, nb, self.momentum, self.eps, self.relu)

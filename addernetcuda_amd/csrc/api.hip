@@ -214,16 +214,17 @@ int adder_bn_act_workspace_bytes(int N, int C, int HW, size_t *bytes) {
 
 int adder_bn_act_fwd_f32(const float *x, const float *residual, const float *gamma, const float *beta, float *y,
                          float *save_mean, float *save_rstd, float *running_mean, float *running_var,
-                         float momentum, float eps, int relu, int N, int C, int HW, void *ws, size_t ws_bytes,
-                         void *stream) {
+                         long long *num_batches_tracked, float momentum, float eps, int relu, int N, int C, int HW,
+                         void *ws, size_t ws_bytes, void *stream) {
     if (!x || !gamma || !beta || !y || !save_mean || !save_rstd) return ADDER_ERR_NULL_POINTER;
     if ((running_mean == nullptr) != (running_var == nullptr)) return ADDER_ERR_NULL_POINTER;
     if (int rc = check_bn(N, C, HW)) return rc;
     if (!(eps > 0.f) || !(momentum >= 0.f && momentum <= 1.f)) return ADDER_ERR_BAD_SHAPE;
     if (!ws || ws_bytes < bn_workspace_bytes(N, C, HW) || (reinterpret_cast<uintptr_t>(ws) & 255))
         return ADDER_ERR_WORKSPACE;
-    return launch_bn_act_fwd(x, residual, gamma, beta, y, save_mean, save_rstd, running_mean, running_var, momentum,
-                             eps, relu != 0, N, C, HW, ws, static_cast<hipStream_t>(stream));
+    return launch_bn_act_fwd(x, residual, gamma, beta, y, save_mean, save_rstd, running_mean, running_var,
+                             num_batches_tracked, momentum, eps, relu != 0, N, C, HW, ws,
+                             static_cast<hipStream_t>(stream));
 }
 
 int adder_bn_act_bwd_f32(const float *dy, const float *y, const float *x, const float *gamma, const float *save_mean,

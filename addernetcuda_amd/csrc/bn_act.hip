@@ -81,14 +81,23 @@ __global__ __launch_bounds__(kBnThreads) void bn_partial_kernel(const float *__r
     }
 }
 
-// One thread per channel: mean, rstd, running statistics.
-__global__ void bn_fwd_finalize_kernel(const double *__restrict__ part, int S, int C, double count, float eps,
-                                       float momentum, float *__restrict__ mean, float *__restrict__ rstd,
-                                       float *__restrict__ running_mean, float *__restrict__ running_var) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
+// One wave per channel: add the S partials, then mean, rstd and the running statistics.
+// Block 0 also advances num_batches_tracked (nullable), saving PyTorch a launch of its own.
+__global__ __launch_bounds__(64) void bn_fwd_finalize_kernel(const double *__restrict__ part, int S, double count,
+                                                             float eps, float momentum, float *__restrict__ mean,
+                                                             float *__restrict__ rstd,
+                                                             float *__restrict__ running_mean,
+                                                             float *__restrict__ running_var,
+                                                             long long *__restrict__ num_batches) {
+    const int c = blockIdx.x;
     double s1 = 0.0, s2 = 0.0;
-    for (int s = 0; s < S; ++s) { s1 += part[((size_t)c * S + s) * 2]; s2 += part[((size_t)c * S + s) * 2 + 1]; }
+    for (int s = threadIdx.x; s < S; s += 64) {
+        s1 += part[((size_t)c * S + s) * 2];
+        s2 += part[((size_t)c * S + s) * 2 + 1];
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (threadIdx.x != 0) return;
     const double mu = s1 / count;
     double var = s2 / count - mu * mu;
     if (var < 0.0) var = 0.0;
@@ -99,20 +108,26 @@ __global__ void bn_fwd_finalize_kernel(const double *__restrict__ part, int S, i
         running_mean[c] = (float)((1.0 - momentum) * (double)running_mean[c] + momentum * mu);
         running_var[c] = (float)((1.0 - momentum) * (double)running_var[c] + momentum * unbiased);
     }
+    if (c == 0 && num_batches) *num_batches += 1;
 }
 
-// One thread per channel: dgamma, dbeta and the two per-channel means the dx pass needs.
-__global__ void bn_bwd_finalize_kernel(const double *__restrict__ part, int S, int C, double count,
-                                       float *__restrict__ dgamma, float *__restrict__ dbeta,
-                                       float *__restrict__ coef /* [C][2]: mean(dz), mean(dz*xhat) */) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
+// One wave per channel: dgamma, dbeta and the two per-channel means the dx pass needs.
+__global__ __launch_bounds__(64) void bn_bwd_finalize_kernel(const double *__restrict__ part, int S, double count,
+                                                             float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                                             float *__restrict__ coef /* [C][2] */) {
+    const int c = blockIdx.x;
     double s1 = 0.0, s2 = 0.0;
-    for (int s = 0; s < S; ++s) { s1 += part[((size_t)c * S + s) * 2]; s2 += part[((size_t)c * S + s) * 2 + 1]; }
+    for (int s = threadIdx.x; s < S; s += 64) {
+        s1 += part[((size_t)c * S + s) * 2];
+        s2 += part[((size_t)c * S + s) * 2 + 1];
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (threadIdx.x != 0) return;
     dbeta[c] = (float)s1;
     dgamma[c] = (float)s2;
-    coef[2 * c] = (float)(s1 / count);
-    coef[2 * c + 1] = (float)(s2 / count);
+    coef[2 * c] = (float)(s1 / count);       // mean(dz)
+    coef[2 * c + 1] = (float)(s2 / count);   // mean(dz * xhat)
 }
 
 template <int V>
@@ -198,14 +213,14 @@ static int apply_blocks(long total4) {
 
 template <int V>
 static int bn_fwd_v(const float *x, const float *res, const float *gamma, const float *beta, float *y, float *mean,
-                    float *rstd, float *running_mean, float *running_var, float momentum, float eps, int relu,
-                    int N, int C, int HW, void *ws, hipStream_t s) {
+                    float *rstd, float *running_mean, float *running_var, long long *num_batches, float momentum,
+                    float eps, int relu, int N, int C, int HW, void *ws, hipStream_t s) {
     const int HWV = HW / V, S = bn_splits(N, C, HWV);
     double *part = reinterpret_cast<double *>(ws);
     hipLaunchKernelGGL((bn_partial_kernel<false, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, nullptr, nullptr, nullptr,
                        nullptr, 0, N, C, HWV, part);
-    hipLaunchKernelGGL(bn_fwd_finalize_kernel, dim3(ceil_div(C, 64)), dim3(64), 0, s, part, S, C, (double)N * HW, eps,
-                       momentum, mean, rstd, running_mean, running_var);
+    hipLaunchKernelGGL(bn_fwd_finalize_kernel, dim3(C), dim3(64), 0, s, part, S, (double)N * HW, eps, momentum, mean,
+                       rstd, running_mean, running_var, num_batches);
     const long total = (long)N * C * HWV;
     hipLaunchKernelGGL(bn_apply_kernel<V>, dim3(apply_blocks(total)), dim3(kBnThreads), 0, s, x, res, mean, rstd, gamma,
                        beta, y, relu, C, HWV, total);
@@ -213,13 +228,13 @@ static int bn_fwd_v(const float *x, const float *res, const float *gamma, const 
 }
 
 int launch_bn_act_fwd(const float *x, const float *res, const float *gamma, const float *beta, float *y,
-                      float *mean, float *rstd, float *running_mean, float *running_var, float momentum,
-                      float eps, int relu, int N, int C, int HW, void *ws, hipStream_t s) {
+                      float *mean, float *rstd, float *running_mean, float *running_var, long long *num_batches,
+                      float momentum, float eps, int relu, int N, int C, int HW, void *ws, hipStream_t s) {
     if (bn_vec4(HW, x, res, y, nullptr, nullptr))
-        return bn_fwd_v<4>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, momentum, eps, relu, N, C,
-                           HW, ws, s);
-    return bn_fwd_v<1>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, momentum, eps, relu, N, C, HW,
-                       ws, s);
+        return bn_fwd_v<4>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, num_batches, momentum, eps,
+                           relu, N, C, HW, ws, s);
+    return bn_fwd_v<1>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, num_batches, momentum, eps, relu,
+                       N, C, HW, ws, s);
 }
 
 template <int V>
@@ -231,8 +246,7 @@ static int bn_bwd_v(const float *dy, const float *y, const float *x, const float
     float *coef = reinterpret_cast<float *>(part + (size_t)C * S * 2);
     hipLaunchKernelGGL((bn_partial_kernel<true, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, dy, y, mean, rstd, relu, N,
                        C, HWV, part);
-    hipLaunchKernelGGL(bn_bwd_finalize_kernel, dim3(ceil_div(C, 64)), dim3(64), 0, s, part, S, C, (double)N * HW,
-                       dgamma, dbeta, coef);
+    hipLaunchKernelGGL(bn_bwd_finalize_kernel, dim3(C), dim3(64), 0, s, part, S, (double)N * HW, dgamma, dbeta, coef);
     const long total = (long)N * C * HWV;
     hipLaunchKernelGGL(bn_bwd_apply_kernel<V>, dim3(apply_blocks(total)), dim3(kBnThreads), 0, s, dy, y, x, mean, rstd,
                        gamma, coef, dx, dres, relu, C, HWV, total);

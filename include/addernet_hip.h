@@ -126,14 +126,16 @@ ADDER_API int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps,
  * statistics pass and one apply pass.  x, y, residual, dy, dx, dresidual are (N, C, H*W).
  *   forward : y = act(gamma * (x - mean) * rstd + beta [+ residual]),  act = ReLU if relu != 0
  *             save_mean / save_rstd (C) are written for the backward; running_mean / running_var
- *             (nullable, both or neither) are updated with `momentum` (unbiased variance).
+ *             (nullable, both or neither) are updated with `momentum` (unbiased variance);
+ *             num_batches_tracked (nullable, one int64 on the device) is incremented by one.
  *   backward: dx, dgamma, dbeta; dresidual (nullable) receives the gradient of the residual input.
  *             y (the forward output) is needed only when relu != 0.
  * ---------------------------------------------------------------------- */
 ADDER_API int adder_bn_act_workspace_bytes(int N, int C, int HW, size_t *bytes);
 ADDER_API int adder_bn_act_fwd_f32(const float *x, const float *residual, const float *gamma, const float *beta,
                                    float *y, float *save_mean, float *save_rstd,
-                                   float *running_mean, float *running_var, float momentum, float eps, int relu,
+                                   float *running_mean, float *running_var, long long *num_batches_tracked,
+                                   float momentum, float eps, int relu,
                                    int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);
 ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const float *x, const float *gamma,
                                    const float *save_mean, const float *save_rstd,
