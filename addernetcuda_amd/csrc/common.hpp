@@ -82,6 +82,12 @@ size_t grad_w_workspace_bytes(const ConvDims &d);
 int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta,
                   void *ws, size_t ws_bytes, const ConvDims &d, hipStream_t s);
 
+// matrix-core weight gradient of the 3x3 / pad-1 layers (grad_w_mfma.hip); variant 0 = not applicable
+struct GradWMfmaPlan { int variant, slots, gy, gz, tilesH, tilesW, ntiles; };
+GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d);
+int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+                       const GradWMfmaPlan &p, hipStream_t s);
+
 // 1x1 / pad 0 / stride 1-2 kernels (conv1x1.hip)
 bool conv1x1_supported(const ConvDims &d, const void *a, const void *b);
 int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s);

@@ -1,0 +1,316 @@
+// Weight gradient of the 3x3 / pad-1 AdderNet convolution on the matrix cores, in full precision.
+//
+//   gw[co,k] = sum_pos xcol[k,pos] * gy[co,pos]  -  w[co,k] * sum_pos gy[co,pos]      (k = (ci, i, j))
+//
+// Unlike the forward and the input gradient (|a-b| and clamp are not multiply-accumulates), the
+// first term of the weight gradient IS a GEMM, G (Co x P) times Xcol^T (P x K), reduced over the
+// positions P = N*Ho*Wo (262 144 for the first ResNet-20 stage at batch 256).  Summing that many
+// O(1) products in fp32 leaves ~1e-4 absolute error whatever the order (an fp32 torch evaluation
+// of the reference formula is off by 1e-3), which is the size of the parity bar itself; AdderNet
+// also singles this gradient out as the full-precision one.  So the products and sums are done in
+// fp64 by v_mfma_f64_16x16x4_f64: fp64 MFMA runs at the rate of v_fma_f32, leaves the VALU free and
+// does the position reduction inside the instruction (no cross-lane fold).
+// Mapping: M = output channels (16 per tile), N = k columns (16 per tile), MFMA-K = 4 adjacent
+// output positions of one row.
+//   A fragment  lane l: gy[co0 + l%16][pos0 + l/16]           from the gy tile in LDS (fp32 -> fp64)
+//   B fragment  lane l: x[ci(k), ho*S + i(k), (wo0 + l/16)*S + j(k)],  k = k0 + l%16, from the
+//               haloed x tile in LDS: the im2col happens in the ds_read addresses.
+//   C/D         lane l, reg r: gw[co0 + 4*r + l/16][k0 + l%16]
+// A wave keeps MT x NT accumulator tiles (8 VGPRs each) in registers for the whole kernel and walks
+// over its share of the positions of every staged tile; PW waves split the positions, MW x NW waves
+// the (co, k) block of the workgroup; the waves are folded in fp64 through LDS at the end.
+// sum_pos gy is collected on the A fragments.  Partials: one fp64 (Co, K) slab per grid.x slot.
+#include "common.hpp"
+#include "tile3x3.hpp"
+
+namespace adder {
+
+typedef double double4v __attribute__((ext_vector_type(4)));
+
+template <int S_, int TH_, int TW_, int NIMG_, int MT_, int NT_, int MW_, int NW_, int PW_>
+struct GwMfmaCfg {
+    static constexpr int S = S_, TH = TH_, TW = TW_, NIMG = NIMG_, MT = MT_, NT = NT_, MW = MW_, NW = NW_, PW = PW_;
+    static constexpr int COB = 16 * MT * MW;          // output channels per workgroup
+    static constexpr int KB = 16 * NT * NW;           // k columns per workgroup
+    static constexpr int CIB = KB / 9;                // = input channels per workgroup
+    static constexpr int NWAVES = MW * NW * PW;
+    static constexpr int NTHREADS = 64 * NWAVES;
+    using XP = PatchCfg<NIMG, CIB, (TH - 1) * S + 3, TW * S, 1, (S == 1) ? 1 : 0, NTHREADS, 3>;
+    static constexpr int GPLANE = TH * TW + 4;        // +4: channel planes start 4 banks apart
+    static constexpr int GBUF = NIMG * COB * GPLANE;
+    static constexpr int GUNITS = NIMG * COB * TH * TW / 4;
+    static constexpr int GITER = ceil_div(GUNITS, NTHREADS);
+    static constexpr int BUF = XP::BUF + GBUF;        // floats per (x, gy) buffer pair
+    static constexpr int STEPS = NIMG * TH * TW / 4;  // MFMA steps (4 positions each) per tile
+    static constexpr int WSTEPS = STEPS / PW;         // ... per wave
+    static constexpr int REGS = MT * NT * 4;          // accumulator values (fp64) per lane
+    static constexpr int RED = 2 * (NWAVES / 2) * (REGS + MT) * 64;  // fp64 fold area, in floats
+    static constexpr int LDS_FLOATS = (2 * BUF > RED) ? 2 * BUF : RED;
+    static constexpr int LDS_BYTES = LDS_FLOATS * 4;
+    static_assert(KB % 9 == 0, "a workgroup's k block must cover whole input channels");
+    static_assert(TW % 4 == 0 && STEPS % PW == 0, "positions must split evenly over the position waves");
+    static_assert((PW & (PW - 1)) == 0, "the fold is a binary tree over the position waves");
+    static_assert(NTHREADS <= 1024 && LDS_BYTES <= 160 * 1024, "workgroup limits");
+    static_assert(XP::BUF % 4 == 0 && GPLANE % 4 == 0, "float4 alignment of the gy tile");
+};
+
+template <class G>
+struct GyStageM { float4 v[G::GITER]; };
+
+template <class G>
+__device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const float *__restrict__ gy, int co0, int Co, int n0,
+                                           int N, int h0, int w0, int Ho, int Wo) {
+#pragma unroll
+    for (int it = 0; it < G::GITER; ++it) {
+        const int u = threadIdx.x + it * G::NTHREADS;
+        const int q = u % (G::TW / 4);
+        const int r = (u / (G::TW / 4)) % G::TH;
+        const int c = (u / (G::TW / 4) / G::TH) % G::COB;
+        const int img = u / (G::TW / 4) / G::TH / G::COB;
+        const int n = n0 + img, co = co0 + c, ho = h0 + r, wo = w0 + 4 * q;
+        const bool ok = (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) && n < N && co < Co && ho < Ho && wo < Wo;
+        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (ok) val = *reinterpret_cast<const float4 *>(gy + (((n * Co + co) * Ho + ho) * Wo + wo));
+        st.v[it] = val;
+    }
+}
+
+template <class G>
+__device__ __forceinline__ void gy_commit_m(const GyStageM<G> &st, float *buf) {
+#pragma unroll
+    for (int it = 0; it < G::GITER; ++it) {
+        const int u = threadIdx.x + it * G::NTHREADS;
+        if (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) {
+            const int q = u % (G::TW / 4);
+            const int r = (u / (G::TW / 4)) % G::TH;
+            const int pc = u / (G::TW / 4) / G::TH;   // = img*COB + c
+            *reinterpret_cast<float4 *>(buf + pc * G::GPLANE + r * G::TW + 4 * q) = st.v[it];
+        }
+    }
+}
+
+template <class G>
+__global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *__restrict__ gy,
+                                                                  const float *__restrict__ x,
+                                                                  double *__restrict__ part,
+                                                                  double *__restrict__ sgpart, int N, int Ci, int H,
+                                                                  int W, int Co, int Ho, int Wo, int tilesH,
+                                                                  int tilesW, int ntiles) {
+    using XP = typename G::XP;
+    constexpr int S = G::S, MT = G::MT, NT = G::NT;
+    extern __shared__ __align__(16) float smem[];
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int pw = wave % G::PW, mw = (wave / G::PW) % G::MW, nw = wave / (G::PW * G::MW);
+    const int co_blk = blockIdx.y * G::COB, k_blk = blockIdx.z * G::KB, ci_blk = blockIdx.z * G::CIB;
+    const int l16 = lane & 15, lk = lane >> 4;
+
+    // per-lane LDS offsets of the fragments at position (img 0, row 0, column group 0)
+    int a_base[MT], b_base[NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) a_base[mt] = XP::BUF + ((mw * MT + mt) * 16 + l16) * G::GPLANE + lk;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int j = (nw * NT + nt) * 16 + l16;        // k column within the workgroup's block
+        const int ci = j / 9, tap = j - ci * 9, ti = tap / 3, tj = tap - ti * 3;
+        b_base[nt] = ci * XP::PLANE + ti * XP::PITCH + XP::LPAD + tj + lk * S;
+    }
+
+    double4v acc[MT][NT];
+    double sgt[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        sgt[mt] = 0.0;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = double4v{0.0, 0.0, 0.0, 0.0};
+    }
+
+    TileStage<XP> xs;
+    GyStageM<G> gs;
+    int tile = blockIdx.x;
+    int n0 = 0, h0 = 0, w0 = 0;
+    auto decode = [&](int t) {
+        const int tw = t % tilesW; t /= tilesW;
+        const int th = t % tilesH; t /= tilesH;
+        n0 = t * G::NIMG; h0 = th * G::TH; w0 = tw * G::TW;
+    };
+    if (tile < ntiles) {
+        decode(tile);
+        tile_fetch<XP>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+        gy_fetch_m<G>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+        tile_commit<XP>(xs, smem);
+        gy_commit_m<G>(gs, smem + XP::BUF);
+    }
+    __syncthreads();
+
+    int cur = 0;
+    for (; tile < ntiles; tile += gridDim.x) {
+        const int next = tile + gridDim.x;
+        if (next < ntiles) {   // next tile's global loads fly during this tile's arithmetic
+            decode(next);
+            tile_fetch<XP>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+            gy_fetch_m<G>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+        }
+        const float *base = smem + cur * G::BUF;
+        auto steps = [&](const int first, const int last) {
+#pragma unroll 4
+            for (int ws = first; ws < last; ++ws) {
+                const int st = pw + ws * G::PW;                 // wave-uniform step: (img, row, column group)
+                const int c4 = st % (G::TW / 4);
+                const int r = (st / (G::TW / 4)) % G::TH;
+                const int img = st / (G::TW / 4) / G::TH;
+                const int a_off = img * G::COB * G::GPLANE + r * G::TW + 4 * c4;
+                const int b_off = img * G::CIB * XP::PLANE + r * S * XP::PITCH + 4 * c4 * S;
+                double a[MT], b[NT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) a[mt] = (double)base[a_base[mt] + a_off];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) b[nt] = (double)base[b_base[nt] + b_off];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    sgt[mt] += a[mt];
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                }
+            }
+        };
+        // the next tile is written to the other LDS buffer half-way through, so that the ds_writes
+        // issue while this tile's queued MFMAs keep the matrix pipe busy
+        steps(0, G::WSTEPS / 2);
+        if (next < ntiles) {
+            tile_commit<XP>(xs, smem + (cur ^ 1) * G::BUF);
+            gy_commit_m<G>(gs, smem + (cur ^ 1) * G::BUF + XP::BUF);
+        }
+        steps(G::WSTEPS / 2, G::WSTEPS);
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // ---- fold the PW position waves of each (mw, nw) block into its pw = 0 wave: binary tree, fp64, via LDS ----
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {           // the four position lanes that share an output channel
+        sgt[mt] += __shfl_xor(sgt[mt], 16, 64);
+        sgt[mt] += __shfl_xor(sgt[mt], 32, 64);
+    }
+    double *red = reinterpret_cast<double *>(smem);
+    constexpr int SLOT = (G::REGS + MT) * 64;   // doubles per sending wave
+    const int blk = nw * G::MW + mw;
+    for (int half = G::PW / 2; half >= 1; half >>= 1) {
+        double *mine = red + (size_t)(blk * (G::PW / 2) + (pw % half)) * SLOT;
+        if (pw >= half && pw < 2 * half) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                mine[(G::REGS + mt) * 64 + lane] = sgt[mt];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) mine[((mt * NT + nt) * 4 + e) * 64 + lane] = acc[mt][nt][e];
+            }
+        }
+        __syncthreads();
+        if (pw < half) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                sgt[mt] += mine[(G::REGS + mt) * 64 + lane];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[mt][nt][e] += mine[((mt * NT + nt) * 4 + e) * 64 + lane];
+            }
+        }
+        __syncthreads();
+    }
+    if (pw != 0) return;
+
+    const int K = Ci * 9;
+    double *dst = part + (size_t)blockIdx.x * Co * K;   // fp64 slabs: partials of opposite sign cancel across slots
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int kcol = k_blk + (nw * NT + nt) * 16 + l16;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int co = co_blk + (mw * MT + mt) * 16 + 4 * e + lk;
+                if (co < Co && kcol < K) dst[(size_t)co * K + kcol] = acc[mt][nt][e];
+            }
+        }
+    if (nw == 0 && blockIdx.z == 0 && lane < 16) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int co = co_blk + (mw * MT + mt) * 16 + lane;
+            if (co < Co) sgpart[(size_t)blockIdx.x * Co + co] = sgt[mt];
+        }
+    }
+}
+
+// ---- host side ------------------------------------------------------------------
+// One blocking for every layer: a workgroup of eight waves owns 16 output channels x 16 input channels
+// (one accumulator row of nine 16x16 fp64 tiles per wave = 72 registers) and 256 positions per staged
+// tile.  Small (co, k) blocks keep the partial slabs at Co*K values per position split whatever the layer.
+//                            S  TH  TW NIMG MT NT MW NW PW
+using GmW32   = GwMfmaCfg<1, 8, 32, 1, 1, 9, 1, 1, 8>;   // outputs 32 wide: 8 rows of one image
+using GmW16   = GwMfmaCfg<1, 16, 16, 1, 1, 9, 1, 1, 8>;  // outputs 16 wide: one image
+using GmW8    = GwMfmaCfg<1, 8, 8, 4, 1, 9, 1, 1, 8>;    // outputs 8 wide:  four images
+using GmW16S2 = GwMfmaCfg<2, 8, 16, 1, 1, 9, 1, 1, 8>;   // stride 2, outputs 16 wide: half an image
+using GmW8S2  = GwMfmaCfg<2, 8, 8, 2, 1, 9, 1, 1, 8>;    // stride 2, outputs 8 wide: two images
+
+template <class G>
+static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
+    p.tilesH = ceil_div(d.Ho, G::TH);
+    p.tilesW = ceil_div(d.Wo, G::TW);
+    p.ntiles = ceil_div(d.N, G::NIMG) * p.tilesH * p.tilesW;
+    p.gy = ceil_div(d.Co, G::COB);
+    p.gz = ceil_div(d.Ci * 9, G::KB);
+    static const int wgs = tune_knob("GWM_WGS", 256);
+    int want = ceil_div(wgs, p.gy * p.gz);
+    p.slots = want < p.ntiles ? want : p.ntiles;
+    if (p.slots < 1) p.slots = 1;
+}
+
+GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
+    GradWMfmaPlan p{};
+    const bool ok = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.W % 4 == 0 && d.Wo % 4 == 0;
+    if (!ok) return p;
+    if (d.stride == 1) p.variant = d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
+    else if (d.stride == 2) p.variant = d.Wo > 8 ? 4 : 5;
+    switch (p.variant) {
+        case 1: plan_one<GmW32>(d, p); break;
+        case 2: plan_one<GmW16>(d, p); break;
+        case 3: plan_one<GmW8>(d, p); break;
+        case 4: plan_one<GmW16S2>(d, p); break;
+        case 5: plan_one<GmW8S2>(d, p); break;
+        default: break;
+    }
+    return p;
+}
+
+template <class G>
+static int launch_one(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+                      const GradWMfmaPlan &p, hipStream_t s) {
+    static bool attr_set = false;
+    if (!attr_set && G::LDS_BYTES > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_mfma_kernel<G>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+        if (e != hipSuccess) return record_hip_error(e);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(grad_w_mfma_kernel<G>, dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
+                       part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles);
+    return check_launch();
+}
+
+int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+                       const GradWMfmaPlan &p, hipStream_t s) {
+    switch (p.variant) {
+        case 1: return launch_one<GmW32>(gy, x, part, sgpart, d, p, s);
+        case 2: return launch_one<GmW16>(gy, x, part, sgpart, d, p, s);
+        case 3: return launch_one<GmW8>(gy, x, part, sgpart, d, p, s);
+        case 4: return launch_one<GmW16S2>(gy, x, part, sgpart, d, p, s);
+        case 5: return launch_one<GmW8S2>(gy, x, part, sgpart, d, p, s);
+        default: return ADDER_ERR_BAD_SHAPE;
+    }
+}
+
+}  // namespace adder

@@ -14,12 +14,15 @@ namespace adder {
 
 // A rectangular patch of an NCHW tensor staged per channel into LDS as
 // [img][cc][ROWS][PITCH]: ICOLS float4-aligned interior columns starting at LDS
-// column LHALO, plus an optional single halo column on either side.
-template <int NIMG_, int CC_, int ROWS_, int ICOLS_, int LHALO_, int RHALO_, int NTHREADS_>
+// column LPAD + LHALO, plus an optional single halo column on either side.  LPAD = 3 puts the
+// interior on a 16-byte boundary (one ds_write_b128 per staged float4) for kernels whose reads
+// do not care about alignment; LPAD = 0 keeps a lane's strips aligned instead.
+template <int NIMG_, int CC_, int ROWS_, int ICOLS_, int LHALO_, int RHALO_, int NTHREADS_, int LPAD_ = 0>
 struct PatchCfg {
     static constexpr int NIMG = NIMG_, CC = CC_, ROWS = ROWS_, ICOLS = ICOLS_, LHALO = LHALO_, RHALO = RHALO_,
-                         NTHREADS = NTHREADS_;
-    static constexpr int PITCH = round_up(LHALO + ICOLS + RHALO, 4);
+                         NTHREADS = NTHREADS_, LPAD = LPAD_;
+    static constexpr int ICOL0 = LPAD + LHALO;          // LDS column of the first interior element
+    static constexpr int PITCH = round_up(ICOL0 + ICOLS + RHALO, 4);
     static constexpr int PLANE = ROWS * PITCH;
     static constexpr int BUF = NIMG * CC * PLANE;  // floats per buffer
     static constexpr int NUV = NIMG * CC * ROWS * (ICOLS / 4);
@@ -86,8 +89,8 @@ __device__ __forceinline__ void tile_commit(const TileStage<P> &st, float *buf) 
         if (P::NUV % P::NTHREADS == 0 || u < P::NUV) {
             const int q = u % (P::ICOLS / 4);
             const int rest = u / (P::ICOLS / 4);  // = (img*CC + cc)*ROWS + r
-            float *dst = buf + rest * P::PITCH + P::LHALO + 4 * q;
-            if (P::LHALO == 0) {
+            float *dst = buf + rest * P::PITCH + P::ICOL0 + 4 * q;
+            if (P::ICOL0 % 4 == 0) {
                 *reinterpret_cast<float4 *>(dst) = st.v[it];
             } else {
                 dst[0] = st.v[it].x; dst[1] = st.v[it].y; dst[2] = st.v[it].z; dst[3] = st.v[it].w;
@@ -100,7 +103,7 @@ __device__ __forceinline__ void tile_commit(const TileStage<P> &st, float *buf) 
         if (P::NUH % P::NTHREADS == 0 || u < P::NUH) {
             const int side = P::LHALO ? u % P::NSIDES : 1;
             const int rest = u / P::NSIDES;
-            buf[rest * P::PITCH + (side ? P::LHALO + P::ICOLS : 0)] = st.h[it];
+            buf[rest * P::PITCH + (side ? P::ICOL0 + P::ICOLS : P::LPAD)] = st.h[it];
         }
     }
 }
