@@ -2,7 +2,7 @@
 // (resnet20.py:28-39: out = relu(bn(conv(x)) [+ residual])).  After the adder kernels these
 // element-wise neighbours dominate a training step; they are HBM-bound, so the point of the fusion
 // is to touch each activation as few times as possible:
-//   forward   pass 1  per-channel sum / sum of squares (fp64)            reads x
+//   forward   pass 1  per-channel sum / sum of squares (fp64 partials)    reads x
 //             pass 2  y = relu(gamma * (x - mean) * rstd + beta + res)    reads x (+ res), writes y
 //   backward  pass 1  per-channel sum(dz), sum(dz * xhat), dz = dy * [y > 0]      reads dy, y, x
 //             pass 2  dx = gamma * rstd * (dz - mean(dz) - xhat * mean(dz * xhat)),
@@ -81,72 +81,68 @@ __global__ __launch_bounds__(kBnThreads) void bn_partial_kernel(const float *__r
     }
 }
 
-// One wave per channel: add the S partials, then mean, rstd and the running statistics.
-// Block 0 also advances num_batches_tracked (nullable), saving PyTorch a launch of its own.
-__global__ __launch_bounds__(64) void bn_fwd_finalize_kernel(const double *__restrict__ part, int S, double count,
-                                                             float eps, float momentum, float *__restrict__ mean,
-                                                             float *__restrict__ rstd,
-                                                             float *__restrict__ running_mean,
-                                                             float *__restrict__ running_var,
-                                                             long long *__restrict__ num_batches) {
-    const int c = blockIdx.x;
-    double s1 = 0.0, s2 = 0.0;
-    for (int s = threadIdx.x; s < S; s += 64) {
-        s1 += part[((size_t)c * S + s) * 2];
-        s2 += part[((size_t)c * S + s) * 2 + 1];
+// Every workgroup of the second pass adds the S partials of its channel itself (same order in every
+// workgroup, so all of them see the same statistics) instead of waiting for a finalize launch.
+__device__ __forceinline__ void bn_reduce_partials(const double *__restrict__ part, int c, int S, double &s1,
+                                                   double &s2) {
+    double a = 0.0, b = 0.0;
+    for (int s = threadIdx.x; s < S; s += kBnThreads) {
+        a += part[((size_t)c * S + s) * 2];
+        b += part[((size_t)c * S + s) * 2 + 1];
     }
-    s1 = wave_sum(s1);
-    s2 = wave_sum(s2);
-    if (threadIdx.x != 0) return;
-    const double mu = s1 / count;
-    double var = s2 / count - mu * mu;
-    if (var < 0.0) var = 0.0;
-    mean[c] = (float)mu;
-    rstd[c] = (float)(1.0 / sqrt(var + (double)eps));
-    if (running_mean) {
-        const double unbiased = count > 1.0 ? var * count / (count - 1.0) : var;
-        running_mean[c] = (float)((1.0 - momentum) * (double)running_mean[c] + momentum * mu);
-        running_var[c] = (float)((1.0 - momentum) * (double)running_var[c] + momentum * unbiased);
-    }
-    if (c == 0 && num_batches) *num_batches += 1;
+    __shared__ double ra[kBnThreads / 64], rb[kBnThreads / 64];
+    a = wave_sum(a);
+    b = wave_sum(b);
+    if ((threadIdx.x & 63) == 0) { ra[threadIdx.x >> 6] = a; rb[threadIdx.x >> 6] = b; }
+    __syncthreads();
+    s1 = (ra[0] + ra[1]) + (ra[2] + ra[3]);
+    s2 = (rb[0] + rb[1]) + (rb[2] + rb[3]);
 }
 
-// One wave per channel: dgamma, dbeta and the two per-channel means the dx pass needs.
-__global__ __launch_bounds__(64) void bn_bwd_finalize_kernel(const double *__restrict__ part, int S, double count,
-                                                             float *__restrict__ dgamma, float *__restrict__ dbeta,
-                                                             float *__restrict__ coef /* [C][2] */) {
-    const int c = blockIdx.x;
-    double s1 = 0.0, s2 = 0.0;
-    for (int s = threadIdx.x; s < S; s += 64) {
-        s1 += part[((size_t)c * S + s) * 2];
-        s2 += part[((size_t)c * S + s) * 2 + 1];
-    }
-    s1 = wave_sum(s1);
-    s2 = wave_sum(s2);
-    if (threadIdx.x != 0) return;
-    dbeta[c] = (float)s1;
-    dgamma[c] = (float)s2;
-    coef[2 * c] = (float)(s1 / count);       // mean(dz)
-    coef[2 * c + 1] = (float)(s2 / count);   // mean(dz * xhat)
-}
-
+// Forward pass 2.  grid = (A, C); block (a, c) finishes the statistics of channel c and normalises the
+// float4 groups a*256 + tid, a*256 + tid + A*256, ... of that channel.  Block (0, c) also stores
+// mean / rstd for the backward pass and updates the running statistics; block (0, 0) advances
+// num_batches_tracked (nullable), saving PyTorch a launch of its own.
 template <int V>
 __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const float *__restrict__ x,
                                                               const float *__restrict__ res,
-                                                              const float *__restrict__ mean,
-                                                              const float *__restrict__ rstd,
+                                                              const double *__restrict__ part, int S, double count,
+                                                              float eps, float momentum,
                                                               const float *__restrict__ gamma,
                                                               const float *__restrict__ beta, float *__restrict__ y,
-                                                              int relu, int C, int HW4, long total4) {
-    for (long i = (long)blockIdx.x * kBnThreads + threadIdx.x; i < total4; i += (long)gridDim.x * kBnThreads) {
-        const int c = (int)((i / HW4) % C);
-        const float sc = gamma[c] * rstd[c], mu = mean[c], sh = beta[c];
-        const Pack<V> v = ld<V>(x, i);
+                                                              float *__restrict__ mean, float *__restrict__ rstd,
+                                                              float *__restrict__ running_mean,
+                                                              float *__restrict__ running_var,
+                                                              long long *__restrict__ num_batches, int relu, int N,
+                                                              int C, int HW4) {
+    const int c = blockIdx.y;
+    double s1, s2;
+    bn_reduce_partials(part, c, S, s1, s2);
+    const double mud = s1 / count;
+    double var = s2 / count - mud * mud;
+    if (var < 0.0) var = 0.0;
+    const float mu = (float)mud, rs = (float)(1.0 / sqrt(var + (double)eps));
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        mean[c] = mu;
+        rstd[c] = rs;
+        if (running_mean) {
+            const double unbiased = count > 1.0 ? var * count / (count - 1.0) : var;
+            running_mean[c] = (float)((1.0 - momentum) * (double)running_mean[c] + momentum * mud);
+            running_var[c] = (float)((1.0 - momentum) * (double)running_var[c] + momentum * unbiased);
+        }
+        if (c == 0 && num_batches) *num_batches += 1;
+    }
+    const float sc = gamma[c] * rs, sh = beta[c];
+    const int total = N * HW4;
+    for (int i = blockIdx.x * kBnThreads + threadIdx.x; i < total; i += gridDim.x * kBnThreads) {
+        const int n = i / HW4, q = i - n * HW4;
+        const size_t off = ((size_t)n * C + c) * HW4 + q;
+        const Pack<V> v = ld<V>(x, off);
         Pack<V> o;
 #pragma unroll
         for (int e = 0; e < V; ++e) o.v[e] = fmaf(v.v[e] - mu, sc, sh);   // subtract first: |x| >> |x - mean| here
         if (res) {
-            const Pack<V> r = ld<V>(res, i);
+            const Pack<V> r = ld<V>(res, off);
 #pragma unroll
             for (int e = 0; e < V; ++e) o.v[e] += r.v[e];
         }
@@ -154,35 +150,47 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const float *__res
 #pragma unroll
             for (int e = 0; e < V; ++e) o.v[e] = fmaxf(o.v[e], 0.f);
         }
-        st<V>(y, i, o);
+        st<V>(y, off, o);
     }
 }
 
+// Backward pass 2, same grid.  Block (0, c) stores dgamma / dbeta.
 template <int V>
 __global__ __launch_bounds__(kBnThreads) void bn_bwd_apply_kernel(const float *__restrict__ dy,
                                                                   const float *__restrict__ y,
                                                                   const float *__restrict__ x,
+                                                                  const double *__restrict__ part, int S, double count,
                                                                   const float *__restrict__ mean,
                                                                   const float *__restrict__ rstd,
                                                                   const float *__restrict__ gamma,
-                                                                  const float *__restrict__ coef,
                                                                   float *__restrict__ dx, float *__restrict__ dres,
-                                                                  int relu, int C, int HW4, long total4) {
-    for (long i = (long)blockIdx.x * kBnThreads + threadIdx.x; i < total4; i += (long)gridDim.x * kBnThreads) {
-        const int c = (int)((i / HW4) % C);
-        const float mu = mean[c], rs = rstd[c], k = gamma[c] * rs, m1 = coef[2 * c], m2 = coef[2 * c + 1];
-        Pack<V> g = ld<V>(dy, i);
+                                                                  float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                                                  int relu, int N, int C, int HW4) {
+    const int c = blockIdx.y;
+    double s1, s2;
+    bn_reduce_partials(part, c, S, s1, s2);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        dbeta[c] = (float)s1;
+        dgamma[c] = (float)s2;
+    }
+    const float m1 = (float)(s1 / count), m2 = (float)(s2 / count);   // mean(dz), mean(dz * xhat)
+    const float mu = mean[c], rs = rstd[c], k = gamma[c] * rs;
+    const int total = N * HW4;
+    for (int i = blockIdx.x * kBnThreads + threadIdx.x; i < total; i += gridDim.x * kBnThreads) {
+        const int n = i / HW4, q = i - n * HW4;
+        const size_t off = ((size_t)n * C + c) * HW4 + q;
+        Pack<V> g = ld<V>(dy, off);
         if (relu) {
-            const Pack<V> yv = ld<V>(y, i);
+            const Pack<V> yv = ld<V>(y, off);
 #pragma unroll
             for (int e = 0; e < V; ++e) g.v[e] = yv.v[e] > 0.f ? g.v[e] : 0.f;
         }
-        if (dres) st<V>(dres, i, g);
-        const Pack<V> v = ld<V>(x, i);
+        if (dres) st<V>(dres, off, g);
+        const Pack<V> v = ld<V>(x, off);
         Pack<V> o;
 #pragma unroll
         for (int e = 0; e < V; ++e) o.v[e] = k * (g.v[e] - m1 - (v.v[e] - mu) * rs * m2);
-        st<V>(dx, i, o);
+        st<V>(dx, off, o);
     }
 }
 
@@ -202,13 +210,16 @@ static bool bn_vec4(int HW, const void *a, const void *b, const void *c, const v
 
 size_t bn_workspace_bytes(int N, int C, int HW) {
     // sized for the scalar layout (the larger of the two) so the choice can depend on pointer alignment
-    return (((size_t)C * bn_splits(N, C, HW) * 2 * sizeof(double) + (size_t)C * 2 * sizeof(float)) + 255) &
-           ~(size_t)255;
+    return ((size_t)C * bn_splits(N, C, HW) * 2 * sizeof(double) + 255) & ~(size_t)255;
 }
 
-static int apply_blocks(long total4) {
-    long b = ceil_div_l(total4, kBnThreads);
-    return (int)(b > 16384 ? 16384 : (b < 1 ? 1 : b));
+// second-pass workgroups per channel: ~4096 over the chip, at least one float4 group per thread
+static int apply_splits(int N, int C, int HW4) {
+    const long per_channel = (long)N * HW4;
+    long a = ceil_div_l(4096, C);
+    const long cap = ceil_div_l(per_channel, kBnThreads);
+    if (a > cap) a = cap;
+    return (int)(a < 1 ? 1 : a);
 }
 
 template <int V>
@@ -219,11 +230,9 @@ static int bn_fwd_v(const float *x, const float *res, const float *gamma, const 
     double *part = reinterpret_cast<double *>(ws);
     hipLaunchKernelGGL((bn_partial_kernel<false, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, nullptr, nullptr, nullptr,
                        nullptr, 0, N, C, HWV, part);
-    hipLaunchKernelGGL(bn_fwd_finalize_kernel, dim3(C), dim3(64), 0, s, part, S, (double)N * HW, eps, momentum, mean,
-                       rstd, running_mean, running_var, num_batches);
-    const long total = (long)N * C * HWV;
-    hipLaunchKernelGGL(bn_apply_kernel<V>, dim3(apply_blocks(total)), dim3(kBnThreads), 0, s, x, res, mean, rstd, gamma,
-                       beta, y, relu, C, HWV, total);
+    hipLaunchKernelGGL(bn_apply_kernel<V>, dim3(apply_splits(N, C, HWV), C), dim3(kBnThreads), 0, s, x, res, part, S,
+                       (double)N * HW, eps, momentum, gamma, beta, y, mean, rstd, running_mean, running_var, num_batches,
+                       relu, N, C, HWV);
     return check_launch();
 }
 
@@ -243,13 +252,10 @@ static int bn_bwd_v(const float *dy, const float *y, const float *x, const float
                     int HW, void *ws, hipStream_t s) {
     const int HWV = HW / V, S = bn_splits(N, C, HWV);
     double *part = reinterpret_cast<double *>(ws);
-    float *coef = reinterpret_cast<float *>(part + (size_t)C * S * 2);
     hipLaunchKernelGGL((bn_partial_kernel<true, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, dy, y, mean, rstd, relu, N,
                        C, HWV, part);
-    hipLaunchKernelGGL(bn_bwd_finalize_kernel, dim3(C), dim3(64), 0, s, part, S, (double)N * HW, dgamma, dbeta, coef);
-    const long total = (long)N * C * HWV;
-    hipLaunchKernelGGL(bn_bwd_apply_kernel<V>, dim3(apply_blocks(total)), dim3(kBnThreads), 0, s, dy, y, x, mean, rstd,
-                       gamma, coef, dx, dres, relu, C, HWV, total);
+    hipLaunchKernelGGL(bn_bwd_apply_kernel<V>, dim3(apply_splits(N, C, HWV), C), dim3(kBnThreads), 0, s, dy, y, x, part,
+                       S, (double)N * HW, mean, rstd, gamma, dx, dres, dgamma, dbeta, relu, N, C, HWV);
     return check_launch();
 }
 
