@@ -25,8 +25,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+PEAK_FP64_MFMA_TFLOPS = 78.6       # MI355X fp64 matrix peak: the 3x3 weight gradient runs on v_mfma_f64_16x16x4_f64
 PEAK_FP32_TFLOPS = 157.3           # MI355X vendor fp32 vector peak (256 CU x 64 lanes x 2 (packed) x 2 (FMA) x 2.4 GHz)
-PEAK_VALU_ISSUE = 256 * 64 * 2.4e9  # lane-instructions per second (one fp32 VALU op per lane per clock)
+# lane-instructions per second: a SIMD starts two vector instructions per 4-cycle slot when two of its
+# waves are ready (one per wave), so 256 CU x 4 SIMD x 2 x 64 lanes / 4 cycles x 2.4 GHz; with an FMA in
+# every slot this is the 157.3 TFLOP/s above.  addernetcuda_amd/valu_issue_probe measures it.
+PEAK_VALU_ISSUE = 2 * 256 * 64 * 2.4e9
 BATCH = 256
 ETA = 0.1
 # HBM bytes per launch of the dominant kernel, from the rocprofv3 counter passes kept under profiles/
@@ -94,12 +98,16 @@ def bench_layers(dev, warmup=5, iters=20):
         for name, fn in ops.items():
             t = event_time(fn, warmup, iters)
             flop, slots = OPS[name]
-            rows.append({
+            row = {
                 "layer": f"{Ci}->{Co} k{k} s{s} p{p} @{H}x{W}", "count": cnt, "op": name, "us": round(t * 1e6, 2),
                 "tflops": round(flop * E / t / 1e12, 2),
                 "frac_fp32_peak": round(flop * E / t / 1e12 / PEAK_FP32_TFLOPS, 4),
-                "valu_issue_util": round(slots * E / t / PEAK_VALU_ISSUE, 4),
-            })
+            }
+            if name == "grad_w" and k == 3:   # fp64 matrix-core kernel (+ finalize and scaling launches)
+                row["frac_fp64_mfma_peak"] = round(2 * E / t / 1e12 / PEAK_FP64_MFMA_TFLOPS, 4)
+            else:
+                row["valu_issue_util"] = round(slots * E / t / PEAK_VALU_ISSUE, 4)
+            rows.append(row)
         del keep
     return rows
 
@@ -120,9 +128,30 @@ def dominant_kernel(dev, steps):
         "algorithmic_bytes": 4 * (2 * BATCH * Ci * H * W + BATCH * Co * H * W + Co * Ci * k * k),
         "avg_launch_us": round(t * 1e6, 2), "flop_per_launch": flop,
         "valu_issue_util": round(OPS["grad_x"][1] * E / t / PEAK_VALU_ISSUE, 4),
-        "note": "fp32 VALU-bound (|a-b| accumulation has no FMA/MFMA form); peak is the packed-FMA vector "
-                "figure, the 3-instruction-per-4-flop inner op caps this kernel at 1/3 of it",
+        "issue_probe_T_lane_instr_per_s": issue_probe(),
+        "note": "fp32 VALU-bound (|a-b| accumulation has no FMA/MFMA form). The 157.3 TFLOP/s peak needs an FMA "
+                "in each of the two vector issue slots a SIMD has per 4 cycles; this op spends 3 instructions on "
+                "4 flop, so 2/3 of the peak (104.9 TFLOP/s) is its ceiling. valu_issue_util is the share of the "
+                "two-slot issue rate; the probe table is that rate measured with a bare instruction stream.",
     }
+
+
+def issue_probe():
+    """Run the stand-alone vector issue-rate probe (a child process) and return its table, or None."""
+    import subprocess
+    exe = os.path.join(ROOT, "addernetcuda_amd", "valu_issue_probe")
+    if not os.path.exists(exe):
+        return None
+    try:
+        out = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    table = {}
+    for line in out.splitlines():
+        f = line.split()
+        if len(f) == 3 and f[0] in ("fwd_pair", "gradx_triple", "sgpr_only"):
+            table.setdefault(f[0], {})[f"{f[1]}_waves_per_simd"] = round(float(f[2]) / 1e12, 2)
+    return table or None
 
 
 def make_step(model, opt, x, y):
