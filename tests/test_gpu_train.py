@@ -1,0 +1,27 @@
+"""The training-script counterpart end to end on a small synthetic set: the loss falls, the evaluation
+pass runs with a batch size the reference would have skipped (main.py:114), and the checkpoint it writes
+has the reference's state_dict keys and reloads into a fresh model."""
+import os
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_two_epochs_learn_and_checkpoint(gpu, tmp_path):
+    from addernetcuda_amd import train
+    from addernetcuda_amd.resnet20 import resnet20
+    args = train.parse_args(["--synthetic", "2000", "--epochs", "6", "--batch-size", "100",
+                             "--test-batch-size", "50", "--output-dir", str(tmp_path), "--seed", "1"])
+    hist = train.run(args)
+    assert len(hist) == 6
+    assert all(torch.isfinite(torch.tensor([h["train_loss"], h["test_loss"]])).all() for h in hist)
+    assert hist[-1]["train_loss"] < hist[0]["train_loss"]
+    assert hist[-1]["accuracy"] > 0.5          # ten classes of clearly separable patterns (0.84 when written)
+    ckpt = os.path.join(str(tmp_path), "addernet.pt")
+    assert os.path.exists(ckpt)
+    state = torch.load(ckpt, map_location="cpu", weights_only=True)
+    assert "layer1.0.conv1.adder" in state and "layer2.0.downsample.0.adder" in state and "bn2.running_mean" in state
+    fresh = resnet20().to(gpu)
+    fresh.load_state_dict(state)               # strict: same keys as the reference's resnet20.py

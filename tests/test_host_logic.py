@@ -86,3 +86,51 @@ def test_resnet20_runs_on_the_cpu_oracle_layer():
     loss.backward()
     g = m.layer1[0].conv1.adder.grad
     assert g.norm().item() == pytest.approx(0.1 * (16 * 16 * 9) ** 0.5, rel=1e-4)
+
+
+# ---- training-script counterpart (addernetcuda_amd/train.py) ----------------------------------
+
+def test_cosine_lr_matches_the_reference_schedule():
+    import math
+    from addernetcuda_amd.train import cosine_lr
+    for epoch in (1, 37, 200, 399):
+        assert cosine_lr(epoch, 400) == pytest.approx(0.025 * (1 + math.cos(float(epoch) / 400 * math.pi)))   # main.py:71
+    assert cosine_lr(400, 400) == pytest.approx(0.0, abs=1e-12)
+
+
+def test_augment_is_crop_of_the_padded_image_with_optional_flip():
+    from addernetcuda_amd.train import augment
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(16, 3, 32, 32)
+    out = augment(x, torch.Generator().manual_seed(5))
+    assert out.shape == x.shape and out.is_contiguous()
+    padded = torch.nn.functional.pad(x, (4, 4, 4, 4))
+    flips = 0
+    for n in range(16):
+        crops = [(dy, dx, f) for dy in range(9) for dx in range(9) for f in (False, True)
+                 if torch.equal(out[n], padded[n, :, dy:dy + 32, dx:dx + 32].flip(2) if f
+                                else padded[n, :, dy:dy + 32, dx:dx + 32])]
+        assert len(crops) == 1, "every output must be exactly one crop of its own padded image"
+        flips += crops[0][2]
+    assert 0 < flips < 16
+
+
+def test_normalise_uses_the_cifar_constants():
+    from addernetcuda_amd.train import normalise, CIFAR_MEAN, CIFAR_STD
+    x = torch.full((1, 3, 32, 32), 255, dtype=torch.uint8)
+    y = normalise(x)
+    for c in range(3):
+        assert y[0, c, 0, 0].item() == pytest.approx((1.0 - CIFAR_MEAN[c]) / CIFAR_STD[c], rel=1e-6)
+
+
+def test_npz_loader_accepts_both_image_layouts(tmp_path):
+    import numpy as np
+    from addernetcuda_amd.train import load_arrays
+    rng = np.random.default_rng(0)
+    nhwc = rng.integers(0, 256, (6, 32, 32, 3), dtype=np.uint8)
+    y = rng.integers(0, 10, 6)
+    p = tmp_path / "d.npz"
+    np.savez(p, x_train=nhwc, y_train=y, x_test=nhwc.transpose(0, 3, 1, 2), y_test=y)
+    d = load_arrays(str(p), torch.device("cpu"))
+    assert d["train"][0].shape == (6, 3, 32, 32) and torch.equal(d["train"][0], d["test"][0])
+    assert d["train"][1].dtype == torch.int64
