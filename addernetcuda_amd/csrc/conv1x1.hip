@@ -13,7 +13,7 @@
 
 namespace adder {
 
-// A lane owns 4/S adjacent outputs of one output row: one aligned float4 of the source row.
+// A lane owns 4/S adjacent outputs of one output row: one float4 of the source row.
 template <int S>
 struct Lane1x1 {
     static constexpr int TN = 4 / S;
@@ -29,7 +29,31 @@ struct Lane1x1 {
     }
 };
 
-template <int S, int TM>
+// Four consecutive floats of a row.  VEC: one aligned float4.  Otherwise (stride 1 on planes whose size is
+// not a multiple of 4, walked as one long row) element by element, `valid` of them inside the row.
+template <bool VEC>
+__device__ __forceinline__ float4 ld4(const float *p, int valid) {
+    if constexpr (VEC) return *reinterpret_cast<const float4 *>(p);
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (valid > 0) v.x = p[0];
+    if (valid > 1) v.y = p[1];
+    if (valid > 2) v.z = p[2];
+    if (valid > 3) v.w = p[3];
+    return v;
+}
+template <bool VEC>
+__device__ __forceinline__ void st4(float *p, const float4 v, int valid) {
+    if constexpr (VEC) {
+        *reinterpret_cast<float4 *>(p) = v;
+    } else {
+        if (valid > 0) p[0] = v.x;
+        if (valid > 1) p[1] = v.y;
+        if (valid > 2) p[2] = v.z;
+        if (valid > 3) p[3] = v.w;
+    }
+}
+
+template <int S, int TM, bool VEC = true>
 __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                       float *__restrict__ y, int N, int Ci, int H, int W,
                                                       int Co, int Ho, int Wo, int gpr, int groups) {
@@ -48,6 +72,7 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
 
     const size_t plane = (size_t)H * W;
     const float *xp = x + (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
+    const int valid = L.ok ? W - L.wo0 * S : 0;   // only read when !VEC
     int ci = 0;
     for (; ci + 4 <= Ci; ci += 4) {
         if ((ci & 63) == 0) {
@@ -58,7 +83,7 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
         }
         float4 xv[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) xv[e] = *reinterpret_cast<const float4 *>(xp + (size_t)(ci + e) * plane);
+        for (int e = 0; e < 4; ++e) xv[e] = ld4<VEC>(xp + (size_t)(ci + e) * plane, valid);
 #pragma unroll
         for (int m = 0; m < TM; ++m)
 #pragma unroll
@@ -70,7 +95,7 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
             }
     }
     for (; ci < Ci; ++ci) {
-        const float4 v = *reinterpret_cast<const float4 *>(xp + (size_t)ci * plane);
+        const float4 v = ld4<VEC>(xp + (size_t)ci * plane, valid);
         const float xs[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
@@ -89,14 +114,14 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
             if (co0 + m >= Co) continue;
             float *dst = y + (((size_t)L.n * Co + co0 + m) * Ho + L.ho) * Wo + L.wo0;
             if constexpr (TN == 4)
-                *reinterpret_cast<float4 *>(dst) = make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]);
+                st4<VEC>(dst, make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]), valid);
             else
                 *reinterpret_cast<float2 *>(dst) = make_float2(tot[m][0], tot[m][1]);
         }
     }
 }
 
-template <int S, int TM>
+template <int S, int TM, bool VEC = true>
 __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict__ gy,
                                                          const float *__restrict__ x,
                                                          const float *__restrict__ w, float *__restrict__ gx,
@@ -108,10 +133,11 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
     uniform_f32_ptr wc = as_uniform(w);
     const size_t plane = (size_t)H * W;
     const size_t xoff = (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
+    const int valid = L.ok ? W - L.wo0 * S : 0;   // only read when !VEC
     float xr[TM][TN], acc[TM][TN], tot[TM][TN];   // two-level sum: acc holds at most 64 output channels
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
-        const float4 v = *reinterpret_cast<const float4 *>(x + xoff + (size_t)min(ci0 + m, Ci - 1) * plane);
+        const float4 v = ld4<VEC>(x + xoff + (size_t)min(ci0 + m, Ci - 1) * plane, valid);
         const float xs[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int t = 0; t < TN; ++t) { xr[m][t] = xs[t * S]; acc[m][t] = tot[m][t] = 0.f; }
@@ -121,7 +147,7 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
     for (int co = 0; co < Co; ++co) {
         float g[TN];
         if constexpr (TN == 4) {
-            const float4 v = *reinterpret_cast<const float4 *>(gp + (size_t)co * gplane);
+            const float4 v = ld4<VEC>(gp + (size_t)co * gplane, valid);
             g[0] = v.x; g[1] = v.y; g[2] = v.z; g[3] = v.w;
         } else {
             const float2 v = *reinterpret_cast<const float2 *>(gp + (size_t)co * gplane);
@@ -147,7 +173,7 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
             if (ci0 + m >= Ci) continue;
             float *dst = gx + xoff + (size_t)(ci0 + m) * plane;
             if constexpr (S == 1) {
-                *reinterpret_cast<float4 *>(dst) = make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]);
+                st4<VEC>(dst, make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]), valid);
             } else {
                 *reinterpret_cast<float4 *>(dst) = make_float4(tot[m][0], 0.f, tot[m][1], 0.f);
                 if (row2) *reinterpret_cast<float4 *>(dst + W) = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -158,7 +184,7 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
 
 // grad_w: a wave owns TM output channels x TC input channels; its lanes walk over position
 // groups, then the 64 lanes are folded through LDS (16 sums per round).
-template <int S, int TM, int TC>
+template <int S, int TM, int TC, bool VEC = true>
 __global__ __launch_bounds__(256) void grad_w_1x1_kernel(const float *__restrict__ gy,
                                                          const float *__restrict__ x, float *__restrict__ part,
                                                          float *__restrict__ sgpart, int N, int Ci, int H,
@@ -177,10 +203,11 @@ __global__ __launch_bounds__(256) void grad_w_1x1_kernel(const float *__restrict
         const Lane1x1<S> L(g0, groups, gpr, Ho);
         const float *xp = x + (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
         const float *gp = gy + (size_t)L.n * Co * gplane + (size_t)L.ho * Wo + L.wo0;
+        const int valid = W - L.wo0 * S;   // only read when !VEC
         float xs[TC][TN], gs[TM][TN];
 #pragma unroll
         for (int c = 0; c < TC; ++c) {
-            const float4 v = *reinterpret_cast<const float4 *>(xp + (size_t)min(ci0 + c, Ci - 1) * plane);
+            const float4 v = ld4<VEC>(xp + (size_t)min(ci0 + c, Ci - 1) * plane, valid);
             const float t4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int t = 0; t < TN; ++t) xs[c][t] = t4[t * S];
@@ -189,7 +216,7 @@ __global__ __launch_bounds__(256) void grad_w_1x1_kernel(const float *__restrict
         for (int m = 0; m < TM; ++m) {
             const float *p = gp + (size_t)min(co0 + m, Co - 1) * gplane;
             if constexpr (TN == 4) {
-                const float4 v = *reinterpret_cast<const float4 *>(p);
+                const float4 v = ld4<VEC>(p, valid);
                 gs[m][0] = v.x; gs[m][1] = v.y; gs[m][2] = v.z; gs[m][3] = v.w;
             } else {
                 const float2 v = *reinterpret_cast<const float2 *>(p);
@@ -245,54 +272,78 @@ __global__ __launch_bounds__(256) void grad_w_1x1_kernel(const float *__restrict
 }
 
 // ---- host side ------------------------------------------------------------------
+// Stride 1: positions are independent, so every (H, W) plane is walked as one row of H*W elements; planes
+// whose size is not a multiple of 4 (7x7) or whose base is not 16-byte aligned take the element-wise loads.
+// Stride 2: one aligned float4 of the source row per lane, whole float2 groups of the output row.
 bool conv1x1_supported(const ConvDims &d, const void *a, const void *b) {
     if (d.kh != 1 || d.kw != 1 || d.pad != 0 || (d.stride != 1 && d.stride != 2)) return false;
-    // one aligned float4 of the source row per lane, whole float4 / float2 groups of the output row
-    if (d.W % 4 != 0 || d.Wo % (4 / d.stride) != 0) return false;
+    if (d.stride == 1) return true;
+    if (d.W % 4 != 0 || d.Wo % 2 != 0) return false;
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) return false;
     return true;
 }
 
-static void lane_space(const ConvDims &d, int &gpr, int &groups) {
-    gpr = d.Wo / (4 / d.stride);
-    groups = d.N * d.Ho * gpr;
+// dimensions the kernels are launched with
+static ConvDims lane_dims(const ConvDims &d) {
+    ConvDims f = d;
+    if (d.stride == 1) { f.H = 1; f.W = d.H * d.W; f.Ho = 1; f.Wo = d.H * d.W; }
+    return f;
+}
+
+static bool vec_ok(const ConvDims &f, const void *a, const void *b, const void *c) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
+    return f.stride == 2 || (f.W % 4 == 0 && (bits & 15) == 0);
+}
+
+static void lane_space(const ConvDims &f, int &gpr, int &groups) {
+    gpr = ceil_div(f.Wo, 4 / f.stride);
+    groups = f.N * f.Ho * gpr;
 }
 
 int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
     constexpr int TM = 8;
+    const ConvDims f = lane_dims(d);
     int gpr, groups;
-    lane_space(d, gpr, groups);
-    const dim3 grid(ceil_div(groups, 256), ceil_div(d.Co, TM));
-    if (d.stride == 1)
-        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM>), grid, dim3(256), 0, s, x, w, y, d.N, d.Ci, d.H, d.W, d.Co, d.Ho,
-                           d.Wo, gpr, groups);
+    lane_space(f, gpr, groups);
+    const dim3 grid(ceil_div(groups, 256), ceil_div(f.Co, TM));
+    if (f.stride == 2)
+        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co, f.Ho,
+                           f.Wo, gpr, groups);
+    else if (vec_ok(f, x, y, nullptr))
+        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM, true>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+                           f.Ho, f.Wo, gpr, groups);
     else
-        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM>), grid, dim3(256), 0, s, x, w, y, d.N, d.Ci, d.H, d.W, d.Co, d.Ho,
-                           d.Wo, gpr, groups);
+        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM, false>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+                           f.Ho, f.Wo, gpr, groups);
     return check_launch();
 }
 
 int launch_grad_x_1x1(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                       hipStream_t s) {
     constexpr int TM = 8;
+    const ConvDims f = lane_dims(d);
     int gpr, groups;
-    lane_space(d, gpr, groups);
-    const dim3 grid(ceil_div(groups, 256), ceil_div(d.Ci, TM));
-    if (d.stride == 1)
-        hipLaunchKernelGGL((grad_x_1x1_kernel<1, TM>), grid, dim3(256), 0, s, gy, x, w, gx, d.N, d.Ci, d.H, d.W,
-                           d.Co, d.Ho, d.Wo, gpr, groups);
+    lane_space(f, gpr, groups);
+    const dim3 grid(ceil_div(groups, 256), ceil_div(f.Ci, TM));
+    if (f.stride == 2)
+        hipLaunchKernelGGL((grad_x_1x1_kernel<2, TM>), grid, dim3(256), 0, s, gy, x, w, gx, f.N, f.Ci, f.H, f.W,
+                           f.Co, f.Ho, f.Wo, gpr, groups);
+    else if (vec_ok(f, gy, x, gx))
+        hipLaunchKernelGGL((grad_x_1x1_kernel<1, TM, true>), grid, dim3(256), 0, s, gy, x, w, gx, f.N, f.Ci, f.H, f.W,
+                           f.Co, f.Ho, f.Wo, gpr, groups);
     else
-        hipLaunchKernelGGL((grad_x_1x1_kernel<2, TM>), grid, dim3(256), 0, s, gy, x, w, gx, d.N, d.Ci, d.H, d.W,
-                           d.Co, d.Ho, d.Wo, gpr, groups);
+        hipLaunchKernelGGL((grad_x_1x1_kernel<1, TM, false>), grid, dim3(256), 0, s, gy, x, w, gx, f.N, f.Ci, f.H,
+                           f.W, f.Co, f.Ho, f.Wo, gpr, groups);
     return check_launch();
 }
 
 static constexpr int kGw1x1TM = 8, kGw1x1TC = 8;
 
 int grad_w_1x1_slots(const ConvDims &d) {
+    const ConvDims f = lane_dims(d);
     int gpr, groups;
-    lane_space(d, gpr, groups);
-    const int blocks_yz = ceil_div(d.Co, kGw1x1TM) * ceil_div(d.Ci, kGw1x1TC);
+    lane_space(f, gpr, groups);
+    const int blocks_yz = ceil_div(f.Co, kGw1x1TM) * ceil_div(f.Ci, kGw1x1TC);
     int want = ceil_div(1024, blocks_yz);                 // ~4 workgroups per CU
     const int cap = ceil_div(groups, 256 * 4);            // at least 4 position groups per lane
     if (want > cap) want = cap;
@@ -301,15 +352,19 @@ int grad_w_1x1_slots(const ConvDims &d) {
 
 int launch_grad_w_1x1(const float *gy, const float *x, float *part, float *sgpart, int slots,
                       const ConvDims &d, hipStream_t s) {
+    const ConvDims f = lane_dims(d);
     int gpr, groups;
-    lane_space(d, gpr, groups);
-    const dim3 grid(slots, ceil_div(d.Co, kGw1x1TM), ceil_div(d.Ci, kGw1x1TC));
-    if (d.stride == 1)
-        hipLaunchKernelGGL((grad_w_1x1_kernel<1, kGw1x1TM, kGw1x1TC>), grid, dim3(256), 0, s, gy, x, part, sgpart,
-                           d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, gpr, groups);
-    else
+    lane_space(f, gpr, groups);
+    const dim3 grid(slots, ceil_div(f.Co, kGw1x1TM), ceil_div(f.Ci, kGw1x1TC));
+    if (f.stride == 2)
         hipLaunchKernelGGL((grad_w_1x1_kernel<2, kGw1x1TM, kGw1x1TC>), grid, dim3(256), 0, s, gy, x, part, sgpart,
-                           d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, gpr, groups);
+                           f.N, f.Ci, f.H, f.W, f.Co, f.Ho, f.Wo, gpr, groups);
+    else if (vec_ok(f, gy, x, nullptr))
+        hipLaunchKernelGGL((grad_w_1x1_kernel<1, kGw1x1TM, kGw1x1TC, true>), grid, dim3(256), 0, s, gy, x, part,
+                           sgpart, f.N, f.Ci, f.H, f.W, f.Co, f.Ho, f.Wo, gpr, groups);
+    else
+        hipLaunchKernelGGL((grad_w_1x1_kernel<1, kGw1x1TM, kGw1x1TC, false>), grid, dim3(256), 0, s, gy, x, part,
+                           sgpart, f.N, f.Ci, f.H, f.W, f.Co, f.Ho, f.Wo, gpr, groups);
     return check_launch();
 }
 

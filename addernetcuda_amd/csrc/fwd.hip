@@ -262,8 +262,10 @@ using FwdW16S2o = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1, 2>;
 using FwdW8S2o  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1, 2>;
 
 int launch_fwd(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
-    const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.W % 4 == 0 &&
-                      (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    // rows that are whole float4 groups are moved as float4 and need 16-byte aligned bases
+    const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 &&
+                      (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
+                      (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0);
     const bool even = d.Ci % 2 == 0;
     if (k3p1 && d.stride == 1) {
         if (d.Wo > 16) return even ? launch_fwd_3x3<FwdW32>(x, w, y, d, s) : launch_fwd_3x3<FwdW32o>(x, w, y, d, s);

@@ -60,6 +60,7 @@ struct GyStageM { float4 v[G::GITER]; };
 template <class G>
 __device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const float *__restrict__ gy, int co0, int Co, int n0,
                                            int N, int h0, int w0, int Ho, int Wo) {
+    const bool vec = (Wo & 3) == 0;
 #pragma unroll
     for (int it = 0; it < G::GITER; ++it) {
         const int u = threadIdx.x + it * G::NTHREADS;
@@ -70,7 +71,17 @@ __device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const float *__restr
         const int n = n0 + img, co = co0 + c, ho = h0 + r, wo = w0 + 4 * q;
         const bool ok = (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) && n < N && co < Co && ho < Ho && wo < Wo;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok) val = *reinterpret_cast<const float4 *>(gy + (((n * Co + co) * Ho + ho) * Wo + wo));
+        if (ok) {
+            const float *row = gy + (((n * Co + co) * Ho + ho) * Wo + wo);
+            if (vec) {
+                val = *reinterpret_cast<const float4 *>(row);
+            } else {   // Wo % 4 != 0: rows are not 16-byte aligned
+                val.x = row[0];
+                if (wo + 1 < Wo) val.y = row[1];
+                if (wo + 2 < Wo) val.z = row[2];
+                if (wo + 3 < Wo) val.w = row[3];
+            }
+        }
         st.v[it] = val;
     }
 }
@@ -271,7 +282,7 @@ static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
 
 GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     GradWMfmaPlan p{};
-    const bool ok = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.W % 4 == 0 && d.Wo % 4 == 0;
+    const bool ok = d.kh == 3 && d.kw == 3 && d.pad == 1;
     if (!ok) return p;
     if (d.stride == 1) p.variant = d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
     else if (d.stride == 2) p.variant = d.Wo > 8 ? 4 : 5;

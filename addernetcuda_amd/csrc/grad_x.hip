@@ -215,7 +215,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
             const int ci = ci_base + m;
             if (ci >= ci_first) {
                 float *dst = gx + (((size_t)n * Ci + ci) * H + hi) * W + wi0;
-                if (TN % 4 == 0 && wi0 + TN <= W) {
+                if (TN % 4 == 0 && (W & 3) == 0 && wi0 + TN <= W) {
 #pragma unroll
                     for (int t = 0; t < TN; t += 4)
                         *reinterpret_cast<float4 *>(dst + t) =
@@ -448,18 +448,18 @@ using GxW8  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1>;
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s) {
     const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
-    if (k3s1p1 && d.W % 4 == 0 && d.Ci >= 8 && (reinterpret_cast<uintptr_t>(gy) & 15) == 0 &&
-        (reinterpret_cast<uintptr_t>(gx) & 15) == 0) {
+    if (k3s1p1 && d.Ci >= 8 &&
+        (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0)) {
         if (d.W > 16) return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s);
         if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s);
     }
-    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.Wo % 4 == 0 && d.W % 2 == 0 && d.Ci >= 8 &&
-        (reinterpret_cast<uintptr_t>(gy) & 15) == 0 && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
+    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.W % 2 == 0 && d.Ci >= 8 &&
+        (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
         if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s);
     }
-    if (conv1x1_supported(d, gy, gx) && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
+    if (conv1x1_supported(d, gy, gx) && (d.stride == 1 || (reinterpret_cast<uintptr_t>(x) & 15) == 0))
         return launch_grad_x_1x1(gy, x, w, gx, d, s);
     constexpr int TM = 8;
     const long total = (long)d.N * d.H * d.W;

@@ -43,13 +43,15 @@ struct TileStage {
 
 // Issue the global loads of one channel chunk into registers.  src is
 // (nimg_total, nchan, H, W); (hb, wb) is the source position of the first
-// interior element of the patch.  Everything outside the tensor reads as zero.  Index arithmetic is
+// interior element of the patch.  Everything outside the tensor reads as zero; W need not be a
+// multiple of 4 (then the float4 groups are read element by element).  Index arithmetic is
 // 32-bit: the C ABI refuses tensors of 2^31 elements or more.
 template <class P>
 __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__restrict__ src,
                                            int chan0, int nchan, int n0, int nimg_total, int hb,
                                            int wb, int H, int W) {
     const int tid = threadIdx.x;
+    const bool vec = (W & 3) == 0;   // wave-uniform; the launchers check the base pointer
 #pragma unroll
     for (int it = 0; it < P::VITER; ++it) {
         const int u = tid + it * P::NTHREADS;
@@ -61,7 +63,17 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
         const bool ok = (P::NUV % P::NTHREADS == 0 || u < P::NUV) && n < nimg_total && ch < nchan &&
                         hi >= 0 && hi < H && wi < W;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok) val = *reinterpret_cast<const float4 *>(src + (((n * nchan + ch) * H + hi) * W + wi));
+        if (ok) {
+            const float *row = src + (((n * nchan + ch) * H + hi) * W + wi);
+            if (vec) {
+                val = *reinterpret_cast<const float4 *>(row);
+            } else {   // rows are not 16-byte aligned (W % 4 != 0): four guarded dword loads
+                val.x = row[0];
+                if (wi + 1 < W) val.y = row[1];
+                if (wi + 2 < W) val.z = row[2];
+                if (wi + 3 < W) val.w = row[3];
+            }
+        }
         st.v[it] = val;
     }
 #pragma unroll

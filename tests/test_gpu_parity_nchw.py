@@ -26,14 +26,22 @@ TILED = [
     (3, 32, 16, 16, 64, 3, 2, 1),   # ResNet-20 strided 3x3, 16 -> 8
     (2, 6, 14, 24, 10, 3, 2, 1),    # strided, channel tails, partial tiles (Ho = 7, Wo = 12)
     (2, 5, 12, 20, 7, 3, 2, 1),     # strided, Wo = 10 (forward tiled, gradients generic)
+    (2, 16, 14, 14, 16, 3, 1, 1),   # ResNet-50 14-wide maps: rows not float4-aligned, 16-wide tile
+    (2, 16, 7, 7, 24, 3, 1, 1),     # 7-wide maps, 8-wide tile
+    (1, 8, 30, 30, 8, 3, 1, 1),     # W = 30 on the 32-wide tile
+    (2, 9, 10, 18, 8, 3, 1, 1),     # odd channel count and W = 18
+    (2, 8, 28, 28, 16, 3, 2, 1),    # strided, Wo = 14
+    (2, 16, 14, 14, 16, 3, 2, 1),   # strided, W = 14 -> Wo = 7
     (2, 16, 32, 32, 32, 1, 2, 0),   # ResNet-20 1x1 stride-2 downsample
     (2, 32, 16, 16, 64, 1, 2, 0),   # second downsample
     (2, 8, 8, 8, 16, 1, 1, 0),      # 1x1 stride 1
     (3, 13, 12, 12, 9, 1, 2, 0),    # 1x1 stride 2 with channel tails
     (2, 9, 6, 12, 20, 1, 1, 0),     # 1x1 stride 1 with channel tails
+    (3, 16, 14, 14, 24, 1, 1, 0),   # 1x1 on a 14x14 plane (walked as one row of 196)
+    (3, 12, 7, 7, 20, 1, 1, 0),     # 1x1 on a 7x7 plane: 49 elements, element-wise loads, partial last group
+    (1, 5, 3, 5, 3, 1, 1, 0),       # 1x1, 15-element planes
 ]
 GENERIC = [
-    (2, 8, 7, 7, 16, 1, 1, 0),      # 1x1, W % 4 != 0
     (2, 4, 9, 9, 6, 3, 2, 1),       # strided 3x3, odd size
     (2, 4, 9, 9, 6, 1, 2, 0),       # strided 1x1, odd size
     (2, 3, 7, 7, 5, 3, 1, 1),       # W % 4 != 0
