@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 // input channels.  Column 0 of a row is input column w0*S-1, so a lane's strip
 // starts at column strip*TN*S, which is 16-byte aligned when TN*S is a multiple of 4.
 // ---------------------------------------------------------------------------
-template <class C>
+template <class C, bool VEC = true>
 __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__restrict__ x,
                                                                 const float *__restrict__ w,
                                                                 float *__restrict__ y, int N, int Ci,
@@ -129,13 +129,13 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     const int nchunks = ceil_div(Ci, C::CC);
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch>(st, x, 0, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+    tile_fetch<typename C::Patch, VEC>(st, x, 0, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int ci0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Ci - ci0);
@@ -225,22 +225,29 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     }
 }
 
-template <class C>
-static int launch_fwd_3x3(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+template <class C, bool VEC>
+static int launch_fwd_3x3_v(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
     const int tilesH = ceil_div(d.Ho, C::TH), tilesW = ceil_div(d.Wo, C::TW);
     const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gy = ceil_div(d.Co, C::TM * C::COW);
     if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     static bool attr_set = false;
     if (!attr_set && C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C, VEC>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(fwd_3x3_kernel<C>, dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
+    hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
                        d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
     return check_launch();
+}
+
+template <class C>
+static int launch_fwd_3x3(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+    // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
+    if (d.W % 4 == 0) return launch_fwd_3x3_v<C, true>(x, w, y, d, s);
+    return launch_fwd_3x3_v<C, false>(x, w, y, d, s);
 }
 
 // Tile shapes per output width.  They are chosen so that (i) a ResNet-20 layer at batch 256

@@ -57,10 +57,9 @@ struct GwMfmaCfg {
 template <class G>
 struct GyStageM { float4 v[G::GITER]; };
 
-template <class G>
+template <class G, bool VEC>
 __device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const float *__restrict__ gy, int co0, int Co, int n0,
                                            int N, int h0, int w0, int Ho, int Wo) {
-    const bool vec = (Wo & 3) == 0;
 #pragma unroll
     for (int it = 0; it < G::GITER; ++it) {
         const int u = threadIdx.x + it * G::NTHREADS;
@@ -73,9 +72,9 @@ __device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const float *__restr
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok) {
             const float *row = gy + (((n * Co + co) * Ho + ho) * Wo + wo);
-            if (vec) {
+            if constexpr (VEC) {
                 val = *reinterpret_cast<const float4 *>(row);
-            } else {   // Wo % 4 != 0: rows are not 16-byte aligned
+            } else {   // rows are not 16-byte aligned (Wo % 4 != 0)
                 val.x = row[0];
                 if (wo + 1 < Wo) val.y = row[1];
                 if (wo + 2 < Wo) val.z = row[2];
@@ -100,7 +99,7 @@ __device__ __forceinline__ void gy_commit_m(const GyStageM<G> &st, float *buf) {
     }
 }
 
-template <class G>
+template <class G, bool VEC = true>
 __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *__restrict__ gy,
                                                                   const float *__restrict__ x,
                                                                   double *__restrict__ part,
@@ -147,8 +146,8 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
     };
     if (tile < ntiles) {
         decode(tile);
-        tile_fetch<XP>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
-        gy_fetch_m<G>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+        tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+        gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         tile_commit<XP>(xs, smem);
         gy_commit_m<G>(gs, smem + XP::BUF);
     }
@@ -159,8 +158,8 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
         const int next = tile + gridDim.x;
         if (next < ntiles) {   // next tile's global loads fly during this tile's arithmetic
             decode(next);
-            tile_fetch<XP>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
-            gy_fetch_m<G>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+            tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+            gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         }
         const float *base = smem + cur * G::BUF;
         auto steps = [&](const int first, const int last) {
@@ -297,19 +296,27 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     return p;
 }
 
-template <class G>
-static int launch_one(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+template <class G, bool VEC>
+static int launch_one_v(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
                       const GradWMfmaPlan &p, hipStream_t s) {
     static bool attr_set = false;
     if (!attr_set && G::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_mfma_kernel<G>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_mfma_kernel<G, VEC>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(grad_w_mfma_kernel<G>, dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
+    hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
                        part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles);
     return check_launch();
+}
+
+template <class G>
+static int launch_one(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+                      const GradWMfmaPlan &p, hipStream_t s) {
+    // element-wise tile loads unless the rows of both x and gy are whole float4 groups
+    if (d.W % 4 == 0 && d.Wo % 4 == 0) return launch_one_v<G, true>(gy, x, part, sgpart, d, p, s);
+    return launch_one_v<G, false>(gy, x, part, sgpart, d, p, s);
 }
 
 int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,

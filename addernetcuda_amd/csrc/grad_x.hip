@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
 //   gx[hi,wi] += hardtanh(w[co,ci,i,j] - x[hi,wi]) * gy[hi+1-i, wi+1-j]
 // In tile coordinates (row 0 = h0-1, column 0 = w0-1) that is row+2-i, t+2-j.
 // ---------------------------------------------------------------------------
-template <class C>
+template <class C, bool VEC = true>
 __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *__restrict__ gy,
                                                                    const float *__restrict__ x,
                                                                    const float *__restrict__ w,
@@ -136,13 +136,13 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     const int nchunks = ceil_div(Co, C::CC);
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch>(st, gy, 0, Co, n0, N, h0 - 1, w0, H, W);
+    tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, h0 - 1, w0, H, W);
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int co0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch>(st, gy, co0 + C::CC, Co, n0, N, h0 - 1, w0, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, gy, co0 + C::CC, Co, n0, N, h0 - 1, w0, H, W);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
@@ -230,8 +230,8 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     }
 }
 
-template <class C>
-static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, float *gx,
+template <class C, bool VEC>
+static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w, float *gx,
                                const ConvDims &d, hipStream_t s) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
@@ -239,14 +239,22 @@ static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, 
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     static bool attr_set = false;
     if (!attr_set && C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C, VEC>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(grad_x_3x3s1_kernel<C>, dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
+    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW);
     return check_launch();
+}
+
+template <class C>
+static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, float *gx,
+                               const ConvDims &d, hipStream_t s) {
+    // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
+    if (d.W % 4 == 0) return launch_grad_x_3x3s1_v<C, true>(gy, x, w, gx, d, s);
+    return launch_grad_x_3x3s1_v<C, false>(gy, x, w, gx, d, s);
 }
 
 // ---------------------------------------------------------------------------
@@ -274,7 +282,7 @@ struct GradX3x3S2Cfg {
     static_assert(TNW % 2 == 0 && TH % 2 == 0, "lanes own 2 x 2 parity blocks");
 };
 
-template <class C>
+template <class C, bool VEC = true>
 __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *__restrict__ gy,
                                                                    const float *__restrict__ x,
                                                                    const float *__restrict__ w,
@@ -327,13 +335,13 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     const int hb = h0 / 2, wb = w0 / 2;
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
+    tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int co0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch>(st, gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
@@ -423,17 +431,25 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     }
 }
 
-template <class C>
-static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, float *gx,
+template <class C, bool VEC>
+static int launch_grad_x_3x3s2_v(const float *gy, const float *x, const float *w, float *gx,
                                const ConvDims &d, hipStream_t s) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     static_assert(C::LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
-    hipLaunchKernelGGL(grad_x_3x3s2_kernel<C>, dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
+    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
     return check_launch();
+}
+
+template <class C>
+static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, float *gx,
+                               const ConvDims &d, hipStream_t s) {
+    // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
+    if (d.Wo % 4 == 0) return launch_grad_x_3x3s2_v<C, true>(gy, x, w, gx, d, s);
+    return launch_grad_x_3x3s2_v<C, false>(gy, x, w, gx, d, s);
 }
 
 //                              TNW BPR TH NIMG TM CIW CC

@@ -43,15 +43,14 @@ struct TileStage {
 
 // Issue the global loads of one channel chunk into registers.  src is
 // (nimg_total, nchan, H, W); (hb, wb) is the source position of the first
-// interior element of the patch.  Everything outside the tensor reads as zero; W need not be a
-// multiple of 4 (then the float4 groups are read element by element).  Index arithmetic is
+// interior element of the patch.  Everything outside the tensor reads as zero.  VEC = false is for
+// tensors whose rows are not float4-aligned (W % 4 != 0): element-wise loads.  Index arithmetic is
 // 32-bit: the C ABI refuses tensors of 2^31 elements or more.
-template <class P>
+template <class P, bool VEC = true>
 __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__restrict__ src,
                                            int chan0, int nchan, int n0, int nimg_total, int hb,
                                            int wb, int H, int W) {
     const int tid = threadIdx.x;
-    const bool vec = (W & 3) == 0;   // wave-uniform; the launchers check the base pointer
 #pragma unroll
     for (int it = 0; it < P::VITER; ++it) {
         const int u = tid + it * P::NTHREADS;
@@ -65,7 +64,7 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok) {
             const float *row = src + (((n * nchan + ch) * H + hi) * W + wi);
-            if (vec) {
+            if constexpr (VEC) {
                 val = *reinterpret_cast<const float4 *>(row);
             } else {   // rows are not 16-byte aligned (W % 4 != 0): four guarded dword loads
                 val.x = row[0];
