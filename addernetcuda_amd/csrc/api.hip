@@ -20,12 +20,6 @@ int check_launch() {
     return e == hipSuccess ? ADDER_OK : record_hip_error(e);
 }
 
-int tune_knob(const char *name, int dflt) {
-    const std::string key = std::string("ADDERNET_") + name;
-    const char *v = std::getenv(key.c_str());
-    return v ? std::atoi(v) : dflt;
-}
-
 static const long kMaxElems = 0x7fffffffL;
 
 static int make_dims(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, ConvDims &d) {

@@ -67,9 +67,6 @@ struct ConvDims {
     __host__ __device__ int K() const { return Ci * kh * kw; }
 };
 
-// Integer tuning knob read once from the environment (ADDERNET_<name>); used to A/B tile shapes.
-int tune_knob(const char *name, int dflt);
-
 // ---- host-side launch plumbing -------------------------------------------------
 int record_hip_error(hipError_t e);  // stores the message, returns ADDER_ERR_HIP
 int check_launch();                  // hipGetLastError -> status

@@ -273,8 +273,7 @@ static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
     p.ntiles = ceil_div(d.N, G::NIMG) * p.tilesH * p.tilesW;
     p.gy = ceil_div(d.Co, G::COB);
     p.gz = ceil_div(d.Ci * 9, G::KB);
-    static const int wgs = tune_knob("GWM_WGS", 256);
-    int want = ceil_div(wgs, p.gy * p.gz);
+    int want = ceil_div(256, p.gy * p.gz);   // one workgroup per CU: the staged tiles fill most of its LDS
     p.slots = want < p.ntiles ? want : p.ntiles;
     if (p.slots < 1) p.slots = 1;
 }
