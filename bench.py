@@ -261,6 +261,9 @@ def main():
     ap.add_argument("--roofline-only", action="store_true",
                     help="launch only the dominant kernel (and one 256 MiB device copy as a counter yardstick); "
                          "meant to run under rocprofv3 --pmc / --kernel-trace")
+    ap.add_argument("--layers-only", action="store_true",
+                    help="run only the per-layer table (7 ResNet-20 layer shapes x forward / grad_X / grad_W); "
+                         "meant to run under rocprofv3 --pmc / --kernel-trace")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (every box here has a single MI355X)")
@@ -276,6 +279,10 @@ def main():
             dst.copy_(src)            # 256 MiB read + 256 MiB written per launch
         torch.cuda.synchronize()
         print(json.dumps({"roofline": dominant_kernel(dev, args.steps), "copy_bytes_each_way": src.numel() * 4}))
+        return
+
+    if args.layers_only:
+        print(json.dumps({"layers": bench_layers(dev, warmup=2, iters=max(3, min(args.steps, 20)))}))
         return
 
     mode = "eager"
