@@ -320,7 +320,7 @@ int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, 
 
 int launch_grad_x_1x1(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                       hipStream_t s) {
-    constexpr int TM = 8;
+    constexpr int TM = 4;   // latency-bound at ResNet sizes: more workgroups beat more reuse per lane
     const ConvDims f = lane_dims(d);
     int gpr, groups;
     lane_space(f, gpr, groups);
