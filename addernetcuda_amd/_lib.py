@@ -23,6 +23,8 @@ _SIGNATURES = {
     "adder_abi_version": (_i, []),
     "adder_out_dim": (_i, [_i, _i, _i, _i]),
     "adder_conv2d_fwd_f32": (_i, [_p, _p, _p] + [_i] * 9 + [_p]),
+    "adder_conv2d_fwd_stats_slots": (_i, [_i] * 9 + [ctypes.POINTER(ctypes.c_int)]),
+    "adder_conv2d_fwd_stats_f32": (_i, [_p, _p, _p, _p, _i] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_workspace_bytes": (_i, [_i] * 9 + [_szp]),
     "adder_conv2d_bwd_f32": (_i, [_p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
     "adder_col_fwd_f32": (_i, [_p, _p, _p, _i, _l, _i, _p]),
@@ -34,6 +36,7 @@ _SIGNATURES = {
     "adder_grad_norm_scale_f32": (_i, [_p, _l, _f, _f, _p, _sz, _p]),
     "adder_bn_act_workspace_bytes": (_i, [_i, _i, _i, _szp]),
     "adder_bn_act_fwd_f32": (_i, [_p] * 10 + [_f, _f, _i, _i, _i, _i, _p, _sz, _p]),
+    "adder_bn_act_fwd_stats_f32": (_i, [_p] * 10 + [_f, _f, _i, _i, _i, _i, _p, _i, _p]),
     "adder_bn_act_bwd_f32": (_i, [_p] * 10 + [_i, _i, _i, _i, _p, _sz, _p]),
 }
 for _name, (_res, _args) in _SIGNATURES.items():

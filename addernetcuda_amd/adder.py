@@ -54,21 +54,36 @@ class _adder_nchw(Function):
     """Fused NCHW forward / backward (replaces adder.py:22-41 + 43-80 in one step each)."""
 
     @staticmethod
-    def forward(ctx, X, W, stride, padding, eta):
+    def forward(ctx, X, W, stride, padding, eta, with_stats=False):
         X, W = X.contiguous(), W.contiguous()
         require_gpu_f32(X, "X")
         require_gpu_f32(W, "W")
         dev = same_device(X, W)
         dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
         out = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
+        stats = None
         with torch.cuda.device(dev):
-            check(lib.adder_conv2d_fwd_f32(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_f32")
+            slots = ctypes.c_int(0)
+            if with_stats:
+                check(lib.adder_conv2d_fwd_stats_slots(*dims, ctypes.byref(slots)), "adder_conv2d_fwd_stats_slots")
+            if slots.value > 0:
+                # partial sums of out and out**2 per channel for the BatchNorm that follows (bn_act.py)
+                stats = torch.empty((W.size(0), slots.value, 2), device=dev, dtype=torch.float64)
+                check(lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots.value, *dims,
+                                                     stream_ptr(dev)), "adder_conv2d_fwd_stats_f32")
+            else:
+                check(lib.adder_conv2d_fwd_f32(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_f32")
         ctx.save_for_backward(X, W)  # the NCHW input, not the 9x larger X_col the reference keeps
         ctx.dims, ctx.eta = dims, eta
-        return out
+        if not with_stats:
+            return out
+        if stats is None:   # no statistics epilogue for this shape: an empty tensor stands for "none"
+            stats = torch.empty(0, device=dev, dtype=torch.float64)
+        ctx.mark_non_differentiable(stats)
+        return out, stats
 
     @staticmethod
-    def backward(ctx, grad_out):
+    def backward(ctx, grad_out, *unused):
         X, W = ctx.saved_tensors
         grad_out = grad_out.contiguous()
         require_gpu_f32(grad_out, "grad_output")
@@ -82,7 +97,7 @@ class _adder_nchw(Function):
                 check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw),
                                                float(ctx.eta or 0.0), ptr(ws), nbytes, *ctx.dims, stream_ptr(dev)),
                       "adder_conv2d_bwd_f32")
-        return gx, gw, None, None, None
+        return gx, gw, None, None, None, None
 
 
 def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
@@ -91,6 +106,15 @@ def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
         # the reference passes only h_filter to unfold (adder.py:32): kernels are square
         raise RuntimeError("adder2d_function expects a square kernel")
     return _adder_nchw.apply(X, W, int(stride), int(padding), eta)
+
+
+def adder2d_function_with_stats(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
+    """``adder2d_function`` that also returns the BatchNorm partial sums of its output, a float64 tensor
+    (Co, slots, 2) for ``BatchNormAct2d(..., stats=)``, or None where the kernel has no such epilogue."""
+    if W.size(2) != W.size(3):
+        raise RuntimeError("adder2d_function expects a square kernel")
+    out, stats = _adder_nchw.apply(X, W, int(stride), int(padding), eta, True)
+    return out, (stats if stats.numel() else None)
 
 
 class adder2d(nn.Module):
@@ -121,6 +145,13 @@ class adder2d(nn.Module):
         if self.bias:
             output = output + self.b.unsqueeze(0).unsqueeze(2).unsqueeze(3)
         return output
+
+    def forward_with_stats(self, x):
+        """(output, stats): ``stats`` are the BatchNorm partial sums of the output for
+        ``BatchNormAct2d.forward(..., stats=stats)``, or None (bias layers, shapes without the epilogue)."""
+        if self.bias:
+            return self.forward(x), None
+        return adder2d_function_with_stats(x, self.adder, self.stride, self.padding, self.eta)
 
     def extra_repr(self):
         return (f"{self.input_channel}, {self.output_channel}, kernel_size={self.kernel_size}, "

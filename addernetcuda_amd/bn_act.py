@@ -25,7 +25,8 @@ def _workspace(N, C, HW, device):
 
 class _bn_act(Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, residual, running_mean, running_var, num_batches, momentum, eps, relu):
+    def forward(ctx, x, weight, bias, residual, running_mean, running_var, num_batches, momentum, eps, relu,
+                stats=None):
         x = x.contiguous()
         if residual is not None:
             residual = residual.contiguous()
@@ -36,11 +37,21 @@ class _bn_act(Function):
         mean = torch.empty(C, dtype=torch.float32, device=dev)
         rstd = torch.empty(C, dtype=torch.float32, device=dev)
         with torch.cuda.device(dev):
-            ws, nbytes = _workspace(N, C, HW, dev)
-            check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mean), ptr(rstd),
-                                           ptr(running_mean), ptr(running_var), ptr(num_batches), float(momentum), float(eps),
-                                           int(relu),
-                                           N, C, HW, ptr(ws), nbytes, stream_ptr(dev)), "adder_bn_act_fwd_f32")
+            if stats is not None:
+                # the layer that produced x already summed x and x*x per channel (adder.forward_with_stats)
+                if stats.dtype != torch.float64 or stats.dim() != 3 or stats.shape[0] != C or stats.shape[2] != 2 \
+                        or not stats.is_contiguous() or stats.device != dev:
+                    raise RuntimeError("stats must be a contiguous float64 tensor (C, slots, 2) on the device of x")
+                check(lib.adder_bn_act_fwd_stats_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mean),
+                                                     ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
+                                                     float(momentum), float(eps), int(relu), N, C, HW, ptr(stats),
+                                                     int(stats.shape[1]), stream_ptr(dev)), "adder_bn_act_fwd_stats_f32")
+            else:
+                ws, nbytes = _workspace(N, C, HW, dev)
+                check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mean),
+                                               ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
+                                               float(momentum), float(eps), int(relu), N, C, HW, ptr(ws), nbytes,
+                                               stream_ptr(dev)), "adder_bn_act_fwd_f32")
         ctx.save_for_backward(x, y if relu else None, weight, mean, rstd)
         ctx.relu, ctx.has_res, ctx.dims = relu, residual is not None, (N, C, HW)
         return y
@@ -59,7 +70,7 @@ class _bn_act(Function):
             check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
                                            ptr(dres), ptr(dgamma), ptr(dbeta), int(ctx.relu), N, C, HW, ptr(ws), nbytes,
                                            stream_ptr(dev)), "adder_bn_act_bwd_f32")
-        return dx, dgamma, dbeta, dres, None, None, None, None, None, None
+        return dx, dgamma, dbeta, dres, None, None, None, None, None, None, None
 
 
 class BatchNormAct2d(nn.BatchNorm2d):
@@ -74,7 +85,9 @@ class BatchNormAct2d(nn.BatchNorm2d):
         return (self.training and x.is_cuda and x.dtype == torch.float32 and self.affine and x.dim() == 4
                 and self.weight.dtype == torch.float32 and self.momentum is not None)
 
-    def forward(self, x, residual=None):
+    def forward(self, x, residual=None, stats=None):
+        """``stats``: optional per-channel partial sums of x and x*x from the layer that produced x
+        (``adder2d.forward_with_stats``); they replace this module's own statistics pass."""
         if not self._fusable(x):
             out = super().forward(x)
             if residual is not None:
@@ -83,4 +96,4 @@ class BatchNormAct2d(nn.BatchNorm2d):
         rm = self.running_mean if self.track_running_stats else None
         rv = self.running_var if self.track_running_stats else None
         nb = self.num_batches_tracked if self.track_running_stats else None   # advanced inside the kernel
-        return _bn_act.apply(x, self.weight, self.bias, residual, rm, rv, nb, self.momentum, self.eps, self.relu)
+        return _bn_act.apply(x, self.weight, self.bias, residual, rm, rv, nb, self.momentum, self.eps, self.relu, stats)

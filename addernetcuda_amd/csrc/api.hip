@@ -54,6 +54,7 @@ const char *adder_strerror(int status) {
         case ADDER_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case ADDER_ERR_HIP: return "HIP runtime error";
         case ADDER_ERR_ALIAS: return "an output overlaps an input";
+        case ADDER_ERR_UNSUPPORTED: return "this variant of the call does not exist for these dimensions or alignments";
         default: return "unknown status";
     }
 }
@@ -75,7 +76,32 @@ int adder_conv2d_fwd_f32(const float *x, const float *w, float *y, int N, int Ci
     const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
                  ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo;
     if (overlaps(y, ny, x, nx) || overlaps(y, ny, w, nw)) return ADDER_ERR_ALIAS;
-    return launch_fwd(x, w, y, d, static_cast<hipStream_t>(stream));
+    return launch_fwd(x, w, y, nullptr, d, static_cast<hipStream_t>(stream));
+}
+
+int adder_conv2d_fwd_stats_slots(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad,
+                                 int *slots) {
+    if (!slots) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    *slots = fwd_stats_slots(d);
+    return ADDER_OK;
+}
+
+int adder_conv2d_fwd_stats_f32(const float *x, const float *w, float *y, double *stats, int stats_slots, int N,
+                               int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, void *stream) {
+    if (!x || !w || !y || !stats) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const int slots = fwd_stats_slots(d);
+    if (slots == 0) return ADDER_ERR_UNSUPPORTED;
+    if (stats_slots != slots) return ADDER_ERR_BAD_SHAPE;
+    const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo, ns = sizeof(double) * 2 * (size_t)Co * slots;
+    if (overlaps(y, ny, x, nx) || overlaps(y, ny, w, nw) || overlaps(stats, ns, x, nx) || overlaps(stats, ns, w, nw) ||
+        overlaps(stats, ns, y, ny))
+        return ADDER_ERR_ALIAS;
+    return launch_fwd(x, w, y, stats, d, static_cast<hipStream_t>(stream));
 }
 
 int adder_conv2d_bwd_workspace_bytes(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
@@ -217,7 +243,21 @@ int adder_bn_act_fwd_f32(const float *x, const float *residual, const float *gam
     if (!ws || ws_bytes < bn_workspace_bytes(N, C, HW) || (reinterpret_cast<uintptr_t>(ws) & 255))
         return ADDER_ERR_WORKSPACE;
     return launch_bn_act_fwd(x, residual, gamma, beta, y, save_mean, save_rstd, running_mean, running_var,
-                             num_batches_tracked, momentum, eps, relu != 0, N, C, HW, ws,
+                             num_batches_tracked, momentum, eps, relu != 0, N, C, HW, ws, nullptr, 0,
+                             static_cast<hipStream_t>(stream));
+}
+
+int adder_bn_act_fwd_stats_f32(const float *x, const float *residual, const float *gamma, const float *beta, float *y,
+                               float *save_mean, float *save_rstd, float *running_mean, float *running_var,
+                               long long *num_batches_tracked, float momentum, float eps, int relu, int N, int C,
+                               int HW, const double *stats, int stats_slots, void *stream) {
+    if (!x || !gamma || !beta || !y || !save_mean || !save_rstd || !stats) return ADDER_ERR_NULL_POINTER;
+    if ((running_mean == nullptr) != (running_var == nullptr)) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_bn(N, C, HW)) return rc;
+    if (stats_slots <= 0) return ADDER_ERR_BAD_SHAPE;
+    if (!(eps > 0.f) || !(momentum >= 0.f && momentum <= 1.f)) return ADDER_ERR_BAD_SHAPE;
+    return launch_bn_act_fwd(x, residual, gamma, beta, y, save_mean, save_rstd, running_mean, running_var,
+                             num_batches_tracked, momentum, eps, relu != 0, N, C, HW, nullptr, stats, stats_slots,
                              static_cast<hipStream_t>(stream));
 }
 

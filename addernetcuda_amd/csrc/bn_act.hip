@@ -213,10 +213,11 @@ size_t bn_workspace_bytes(int N, int C, int HW) {
     return ((size_t)C * bn_splits(N, C, HW) * 2 * sizeof(double) + 255) & ~(size_t)255;
 }
 
-// second-pass workgroups per channel: ~4096 over the chip, at least one float4 group per thread
+// second-pass workgroups per channel: ~1024 over the chip (four per CU; every one of them first adds the
+// channel's partial sums), at least one float4 group per thread
 static int apply_splits(int N, int C, int HW4) {
     const long per_channel = (long)N * HW4;
-    long a = ceil_div_l(4096, C);
+    long a = ceil_div_l(1024, C);
     const long cap = ceil_div_l(per_channel, kBnThreads);
     if (a > cap) a = cap;
     return (int)(a < 1 ? 1 : a);
@@ -225,11 +226,18 @@ static int apply_splits(int N, int C, int HW4) {
 template <int V>
 static int bn_fwd_v(const float *x, const float *res, const float *gamma, const float *beta, float *y, float *mean,
                     float *rstd, float *running_mean, float *running_var, long long *num_batches, float momentum,
-                    float eps, int relu, int N, int C, int HW, void *ws, hipStream_t s) {
-    const int HWV = HW / V, S = bn_splits(N, C, HWV);
-    double *part = reinterpret_cast<double *>(ws);
-    hipLaunchKernelGGL((bn_partial_kernel<false, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, nullptr, nullptr, nullptr,
-                       nullptr, 0, N, C, HWV, part);
+                    float eps, int relu, int N, int C, int HW, void *ws, const double *stats, int stats_slots,
+                    hipStream_t s) {
+    const int HWV = HW / V;
+    int S = stats_slots;
+    const double *part = stats;
+    if (!stats) {   // statistics pass of our own; otherwise the producer of x already wrote the partial sums
+        S = bn_splits(N, C, HWV);
+        double *own = reinterpret_cast<double *>(ws);
+        hipLaunchKernelGGL((bn_partial_kernel<false, V>), dim3(S, C), dim3(kBnThreads), 0, s, x, nullptr, nullptr,
+                           nullptr, nullptr, 0, N, C, HWV, own);
+        part = own;
+    }
     hipLaunchKernelGGL(bn_apply_kernel<V>, dim3(apply_splits(N, C, HWV), C), dim3(kBnThreads), 0, s, x, res, part, S,
                        (double)N * HW, eps, momentum, gamma, beta, y, mean, rstd, running_mean, running_var, num_batches,
                        relu, N, C, HWV);
@@ -238,12 +246,13 @@ static int bn_fwd_v(const float *x, const float *res, const float *gamma, const 
 
 int launch_bn_act_fwd(const float *x, const float *res, const float *gamma, const float *beta, float *y,
                       float *mean, float *rstd, float *running_mean, float *running_var, long long *num_batches,
-                      float momentum, float eps, int relu, int N, int C, int HW, void *ws, hipStream_t s) {
+                      float momentum, float eps, int relu, int N, int C, int HW, void *ws, const double *stats,
+                      int stats_slots, hipStream_t s) {
     if (bn_vec4(HW, x, res, y, nullptr, nullptr))
         return bn_fwd_v<4>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, num_batches, momentum, eps,
-                           relu, N, C, HW, ws, s);
+                           relu, N, C, HW, ws, stats, stats_slots, s);
     return bn_fwd_v<1>(x, res, gamma, beta, y, mean, rstd, running_mean, running_var, num_batches, momentum, eps, relu,
-                       N, C, HW, ws, s);
+                       N, C, HW, ws, stats, stats_slots, s);
 }
 
 template <int V>

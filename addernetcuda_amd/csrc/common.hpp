@@ -62,6 +62,25 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Sum over the 64 lanes without LDS traffic: four DPP steps inside each row of 16 lanes, then the four row
+// sums are read back as scalars.  The result is wave-uniform.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    int t;
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true);   // row_half_mirror
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true);   // row_mirror
+    v += __int_as_float(t);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
 struct ConvDims {
     int N, Ci, H, W, Co, kh, kw, stride, pad, Ho, Wo;
     __host__ __device__ int K() const { return Ci * kh * kw; }
@@ -72,7 +91,8 @@ int record_hip_error(hipError_t e);  // stores the message, returns ADDER_ERR_HI
 int check_launch();                  // hipGetLastError -> status
 
 // Launchers implemented in the kernel translation units.
-int launch_fwd(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s);
+int launch_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s);
+int fwd_stats_slots(const ConvDims &d);   // 0: no statistics epilogue for these dimensions
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s);
 size_t grad_w_workspace_bytes(const ConvDims &d);
@@ -98,7 +118,7 @@ int launch_grad_w_1x1(const float *gy, const float *x, float *part, float *sgpar
 size_t bn_workspace_bytes(int N, int C, int HW);
 int launch_bn_act_fwd(const float *x, const float *res, const float *gamma, const float *beta, float *y,
                       float *mean, float *rstd, float *running_mean, float *running_var, long long *num_batches,
-                      float momentum, float eps, int relu, int N, int C, int HW, void *ws, hipStream_t s);
+                      float momentum, float eps, int relu, int N, int C, int HW, void *ws, const double *stats, int stats_slots, hipStream_t s);
 int launch_bn_act_bwd(const float *dy, const float *y, const float *x, const float *gamma, const float *mean,
                       const float *rstd, float *dx, float *dres, float *dgamma, float *dbeta, int relu, int N,
                       int C, int HW, void *ws, hipStream_t s);

@@ -87,7 +87,8 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 template <class C, bool VEC = true>
 __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__restrict__ x,
                                                                 const float *__restrict__ w,
-                                                                float *__restrict__ y, int N, int Ci,
+                                                                float *__restrict__ y,
+                                                                double *__restrict__ stats, int N, int Ci,
                                                                 int H, int W, int Co, int Ho, int Wo,
                                                                 int tilesH, int tilesW) {
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, S = C::S, STRIP = C::STRIP;
@@ -203,6 +204,37 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     }
 
     const int n = n0 + img, ho = h0 + row, wo = w0 + strip * TN;
+    if (stats) {
+        // BatchNorm statistics of the layer's output on the way out: per wave and output channel the sums of
+        // y and y*y over the wave's valid positions, in the partial-sum layout of the BatchNorm kernels
+        // (slot = position wave of this launch, stats[(co * slots + slot) * 2 + {0, 1}]).
+        // The lanes sum deviations from a pivot (lane 0's first value) in fp32 and lane 0 moves the sums back
+        // to the origin in fp64, so the cancellation in E[y*y] - E[y]^2 happens in double precision.
+        const bool row_ok = lane_ok && n < N && ho < Ho;
+        const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+        float cnt = 0.f;
+#pragma unroll
+        for (int t = 0; t < TN; ++t) cnt += (row_ok && wo + t < Wo) ? 1.f : 0.f;
+        const double count = (double)wave_sum_dpp(cnt);
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const float pivot = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(tot[m][0])));
+            float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int t = 0; t < TN; ++t)
+                if (row_ok && wo + t < Wo) {
+                    const float dv = tot[m][t] - pivot;
+                    s1 += dv;
+                    s2 = fmaf(dv, dv, s2);
+                }
+            const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2), c = (double)pivot;
+            const int co = co_base + m;
+            if (lane == 0 && co < Co) {
+                stats[((size_t)co * slots + slot) * 2] = d1 + count * c;
+                stats[((size_t)co * slots + slot) * 2 + 1] = d2 + 2.0 * c * d1 + count * c * c;
+            }
+        }
+    }
     if (lane_ok && n < N && ho < Ho) {
         const bool vec = TN % 4 == 0 && (Wo & 3) == 0 && wo + TN <= Wo;
 #pragma unroll
@@ -226,7 +258,8 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
 }
 
 template <class C, bool VEC>
-static int launch_fwd_3x3_v(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+static int launch_fwd_3x3_v(const float *x, const float *w, float *y, double *stats, const ConvDims &d,
+                            hipStream_t s) {
     const int tilesH = ceil_div(d.Ho, C::TH), tilesW = ceil_div(d.Wo, C::TW);
     const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gy = ceil_div(d.Co, C::TM * C::COW);
@@ -239,15 +272,23 @@ static int launch_fwd_3x3_v(const float *x, const float *w, float *y, const Conv
         attr_set = true;
     }
     hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
-                       d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
+                       stats, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
     return check_launch();
 }
 
 template <class C>
-static int launch_fwd_3x3(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+static int launch_fwd_3x3(const float *x, const float *w, float *y, double *stats, const ConvDims &d,
+                          hipStream_t s) {
     // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
-    if (d.W % 4 == 0) return launch_fwd_3x3_v<C, true>(x, w, y, d, s);
-    return launch_fwd_3x3_v<C, false>(x, w, y, d, s);
+    if (d.W % 4 == 0) return launch_fwd_3x3_v<C, true>(x, w, y, stats, d, s);
+    return launch_fwd_3x3_v<C, false>(x, w, y, stats, d, s);
+}
+
+// partial-sum slots per channel the statistics epilogue of this tile shape writes
+template <class C>
+static int stats_slots_3x3(const ConvDims &d) {
+    const long gx = (long)ceil_div(d.N, C::NIMG) * ceil_div(d.Ho, C::TH) * ceil_div(d.Wo, C::TW);
+    return (int)(gx * C::POSW);
 }
 
 // Tile shapes per output width.  They are chosen so that (i) a ResNet-20 layer at batch 256
@@ -268,22 +309,44 @@ using FwdW8o    = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1, 1>;
 using FwdW16S2o = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1, 2>;
 using FwdW8S2o  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1, 2>;
 
-int launch_fwd(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+// which tiled kernel serves these dimensions (0 = none): 1..3 stride 1 by output width, 4..5 stride 2
+static int fwd_tiled_variant(const ConvDims &d) {
+    if (d.kh != 3 || d.kw != 3 || d.pad != 1) return 0;
+    if (d.stride == 1) return d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
+    if (d.stride == 2) return d.Wo > 8 ? 4 : 5;
+    return 0;
+}
+
+int fwd_stats_slots(const ConvDims &d) {
+    const bool even = d.Ci % 2 == 0;
+    switch (fwd_tiled_variant(d)) {
+        case 1: return even ? stats_slots_3x3<FwdW32>(d) : stats_slots_3x3<FwdW32o>(d);
+        case 2: return even ? stats_slots_3x3<FwdW16>(d) : stats_slots_3x3<FwdW16o>(d);
+        case 3: return even ? stats_slots_3x3<FwdW8>(d) : stats_slots_3x3<FwdW8o>(d);
+        case 4: return even ? stats_slots_3x3<FwdW16S2>(d) : stats_slots_3x3<FwdW16S2o>(d);
+        case 5: return even ? stats_slots_3x3<FwdW8S2>(d) : stats_slots_3x3<FwdW8S2o>(d);
+        default: return 0;
+    }
+}
+
+// stats (nullable): per-channel partial sums of y and y*y, fwd_stats_slots(d) > 0 slots per channel
+int launch_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s) {
     // rows that are whole float4 groups are moved as float4 and need 16-byte aligned bases
     const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 &&
                       (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                       (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0);
     const bool even = d.Ci % 2 == 0;
     if (k3p1 && d.stride == 1) {
-        if (d.Wo > 16) return even ? launch_fwd_3x3<FwdW32>(x, w, y, d, s) : launch_fwd_3x3<FwdW32o>(x, w, y, d, s);
-        if (d.Wo > 8) return even ? launch_fwd_3x3<FwdW16>(x, w, y, d, s) : launch_fwd_3x3<FwdW16o>(x, w, y, d, s);
-        return even ? launch_fwd_3x3<FwdW8>(x, w, y, d, s) : launch_fwd_3x3<FwdW8o>(x, w, y, d, s);
+        if (d.Wo > 16) return even ? launch_fwd_3x3<FwdW32>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW32o>(x, w, y, stats, d, s);
+        if (d.Wo > 8) return even ? launch_fwd_3x3<FwdW16>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW16o>(x, w, y, stats, d, s);
+        return even ? launch_fwd_3x3<FwdW8>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW8o>(x, w, y, stats, d, s);
     }
     if (k3p1 && d.stride == 2) {
         if (d.Wo > 8)
-            return even ? launch_fwd_3x3<FwdW16S2>(x, w, y, d, s) : launch_fwd_3x3<FwdW16S2o>(x, w, y, d, s);
-        return even ? launch_fwd_3x3<FwdW8S2>(x, w, y, d, s) : launch_fwd_3x3<FwdW8S2o>(x, w, y, d, s);
+            return even ? launch_fwd_3x3<FwdW16S2>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW16S2o>(x, w, y, stats, d, s);
+        return even ? launch_fwd_3x3<FwdW8S2>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW8S2o>(x, w, y, stats, d, s);
     }
+    if (stats) return ADDER_ERR_UNSUPPORTED;   // only the tiled kernels have the statistics epilogue
     if (conv1x1_supported(d, x, y)) return launch_fwd_1x1(x, w, y, d, s);
     constexpr int TM = 8;
     const long total = (long)d.N * d.Ho * d.Wo;

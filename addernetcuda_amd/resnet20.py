@@ -35,10 +35,18 @@ class BasicBlock(nn.Module):
         self.downsample = downsample
         self.stride = stride
 
+    @staticmethod
+    def _conv_bn(conv, bn, x, residual=None):
+        # the adder kernels sum their output per channel on the way out, which saves the BatchNorm its own pass
+        if bn.training and hasattr(conv, "forward_with_stats") and x.is_cuda:
+            out, stats = conv.forward_with_stats(x)
+            return bn(out, residual=residual, stats=stats)
+        return bn(conv(x), residual=residual)
+
     def forward(self, x):
-        out = self.bn1(self.conv1(x))                                   # bn + relu
+        out = self._conv_bn(self.conv1, self.bn1, x)                    # bn + relu
         shortcut = x if self.downsample is None else self.downsample(x)
-        return self.bn2(self.conv2(out), residual=shortcut)             # bn + residual + relu
+        return self._conv_bn(self.conv2, self.bn2, out, shortcut)       # bn + residual + relu
 
 
 class ResNet(nn.Module):

@@ -35,7 +35,8 @@ typedef enum adder_status {
     ADDER_ERR_TOO_LARGE = -3,      /* a tensor exceeds 2^31-1 elements                   */
     ADDER_ERR_WORKSPACE = -4,      /* workspace missing, misaligned or too small         */
     ADDER_ERR_HIP = -5,            /* a HIP call failed; see adder_last_hip_error()      */
-    ADDER_ERR_ALIAS = -6           /* an output overlaps an input                        */
+    ADDER_ERR_ALIAS = -6,          /* an output overlaps an input                        */
+    ADDER_ERR_UNSUPPORTED = -7     /* optional variant not available for these arguments */
 } adder_status;
 
 /* Text for a status code (static storage). */
@@ -61,6 +62,18 @@ ADDER_API int adder_out_dim(int h, int k, int pad, int stride);
 ADDER_API int adder_conv2d_fwd_f32(const float *x, const float *w, float *y,
                          int N, int Ci, int H, int W, int Co, int kh, int kw,
                          int stride, int pad, void *stream);
+
+/* The same forward with the statistics of the BatchNorm that follows it (resnet20.py:28-39: every adder
+ * layer feeds a BatchNorm2d) collected on the way out: stats[(co * slots + s) * 2 + {0, 1}] receive partial
+ * sums of y and y*y over disjoint sets of positions, in fp64; adder_bn_act_fwd_stats_f32 consumes them and
+ * skips its own pass over y.  adder_conv2d_fwd_stats_slots gives `slots` for the dimensions, 0 when the
+ * kernel that serves them has no such epilogue (then, and for x or y not 16-byte aligned, the _stats call
+ * returns ADDER_ERR_UNSUPPORTED and the caller uses the two plain calls). */
+ADDER_API int adder_conv2d_fwd_stats_slots(int N, int Ci, int H, int W, int Co, int kh, int kw,
+                                           int stride, int pad, int *slots);
+ADDER_API int adder_conv2d_fwd_stats_f32(const float *x, const float *w, float *y, double *stats, int stats_slots,
+                                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                                         int stride, int pad, void *stream);
 
 /* Bytes of scratch adder_conv2d_bwd_f32 needs for these dimensions. */
 ADDER_API int adder_conv2d_bwd_workspace_bytes(int N, int Ci, int H, int W, int Co, int kh, int kw,
@@ -137,6 +150,13 @@ ADDER_API int adder_bn_act_fwd_f32(const float *x, const float *residual, const 
                                    float *running_mean, float *running_var, long long *num_batches_tracked,
                                    float momentum, float eps, int relu,
                                    int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);
+/* adder_bn_act_fwd_f32 with the statistics pass already done by the producer of x
+ * (adder_conv2d_fwd_stats_f32): `stats` holds C x stats_slots pairs of partial sums; no workspace. */
+ADDER_API int adder_bn_act_fwd_stats_f32(const float *x, const float *residual, const float *gamma, const float *beta,
+                                         float *y, float *save_mean, float *save_rstd,
+                                         float *running_mean, float *running_var, long long *num_batches_tracked,
+                                         float momentum, float eps, int relu,
+                                         int N, int C, int HW, const double *stats, int stats_slots, void *stream);
 ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const float *x, const float *gamma,
                                    const float *save_mean, const float *save_rstd,
                                    float *dx, float *dresidual, float *dgamma, float *dbeta, int relu,

@@ -70,3 +70,74 @@ def test_eval_mode_and_state_dict_are_those_of_batchnorm2d(gpu):
     assert torch.allclose(a.running_mean, b.running_mean, atol=1e-6) and torch.allclose(a.running_var, b.running_var, atol=1e-5)
     a.eval(), b.eval()
     assert torch.allclose(a(x), F.relu(b(x)), rtol=1e-5, atol=1e-6)
+
+
+# (N, Ci, H, W, Co, k, stride, pad): one case per tiled forward kernel, with channel / tile / width tails
+STATS_CASES = [
+    (3, 16, 32, 32, 16, 3, 1, 1), (2, 32, 16, 16, 32, 3, 1, 1), (5, 64, 8, 8, 64, 3, 1, 1),
+    (2, 5, 12, 20, 7, 3, 1, 1), (2, 16, 32, 32, 32, 3, 2, 1), (3, 32, 16, 16, 64, 3, 2, 1),
+    (2, 16, 14, 14, 20, 3, 1, 1), (2, 9, 10, 18, 8, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", STATS_CASES, ids=str)
+def test_forward_statistics_epilogue_sums_the_output(case, gpu):
+    """The partial sums the adder forward writes for the BatchNorm behind it add up to sum(y) and sum(y*y)
+    per channel, and the output itself is the one the plain call gives."""
+    from addernetcuda_amd import adder
+    N, Ci, H, W, Co, k, s, p = case
+    g = torch.Generator().manual_seed(sum(case))
+    x = torch.randn(N, Ci, H, W, generator=g).to(gpu)
+    w = (torch.randn(Co, Ci, k, k, generator=g) * (2.0 / (Ci * k * k)) ** 0.5).to(gpu)
+    y_plain = adder.adder2d_function(x, w, s, p)
+    y, stats = adder.adder2d_function_with_stats(x, w, s, p)
+    torch.cuda.synchronize()
+    assert stats is not None and stats.dtype == torch.float64 and stats.shape[0] == Co and stats.shape[2] == 2
+    assert torch.equal(y, y_plain)
+    tot = stats.sum(dim=1).cpu()
+    yd = y.double().cpu()
+    assert torch.allclose(tot[:, 0], yd.sum(dim=(0, 2, 3)), rtol=1e-6, atol=1e-6)
+    assert torch.allclose(tot[:, 1], (yd * yd).sum(dim=(0, 2, 3)), rtol=1e-6, atol=1e-6)
+
+
+def test_layers_without_the_epilogue_report_none(gpu):
+    from addernetcuda_amd import adder
+    x = torch.randn(2, 8, 8, 8, device=gpu)
+    for k, s, p in ((1, 1, 0), (1, 2, 0), (5, 1, 2)):
+        w = torch.randn(4, 8, k, k, device=gpu)
+        y, stats = adder.adder2d_function_with_stats(x, w, s, p)
+        assert stats is None and torch.equal(y, adder.adder2d_function(x, w, s, p))
+    layer = adder.adder2d(8, 4, 3, padding=1, bias=True).to(gpu)
+    assert layer.forward_with_stats(x)[1] is None          # the bias would not be in the sums
+
+
+@pytest.mark.parametrize("with_res", [False, True])
+def test_batchnorm_from_precomputed_statistics_equals_its_own_pass(with_res, gpu):
+    from addernetcuda_amd import adder
+    from addernetcuda_amd.bn_act import BatchNormAct2d
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(6, 16, 16, 16, generator=g).to(gpu)
+    layer = adder.adder2d(16, 24, 3, padding=1).to(gpu)
+    res = torch.randn(6, 24, 16, 16, generator=g).to(gpu) if with_res else None
+    # relu off: a ReLU gate that flips on a last-bit difference of the statistics would dominate the comparison
+    a, b = BatchNormAct2d(24, relu=False).to(gpu).train(), BatchNormAct2d(24, relu=False).to(gpu).train()
+    dy = torch.randn(6, 24, 16, 16, generator=g).to(gpu)   # (sum of squares of a normalised tensor is constant)
+    outs = []
+    for bn, fused in ((a, True), (b, False)):
+        xin = x.clone().requires_grad_(True)
+        layer.zero_grad()
+        if fused:
+            y, stats = layer.forward_with_stats(xin)
+            assert stats is not None
+            out = bn(y, residual=res, stats=stats)
+        else:
+            out = bn(layer(xin), residual=res)
+        (out * dy).sum().backward()
+        outs.append((out.detach(), xin.grad, layer.adder.grad.clone(), bn.weight.grad, bn.running_mean.clone(),
+                     bn.running_var.clone()))
+    torch.cuda.synchronize()
+    for got, want, name in zip(outs[0], outs[1], ("y", "dx", "dw", "dgamma", "running_mean", "running_var")):
+        # the two paths add the same numbers in a different order: statistics agree to ~1e-7, what is
+        # back-propagated through them to ~1e-5 of the largest entry
+        assert torch.allclose(got, want, rtol=1e-4, atol=1e-4 * max(1.0, want.abs().max().item())), name
+    assert int(a.num_batches_tracked) == 1
