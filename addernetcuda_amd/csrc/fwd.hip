@@ -291,23 +291,18 @@ static int stats_slots_3x3(const ConvDims &d) {
     return (int)(gx * C::POSW);
 }
 
-// Tile shapes per output width.  They are chosen so that (i) a ResNet-20 layer at batch 256
-// launches >= 2048 waves, (ii) one pipeline unit (one output channel x CQ input channels) has
-// enough vector instructions (18*CQ*TN) to cover a scalar-cache miss, and (iii) the two weight
-// buffers (18*CQ SGPRs) stay far from the 102-SGPR limit: spilled SGPRs come back as
-// v_readlane, i.e. as vector instructions inside the hot loop.
+// Tile shapes per output width, picked by timing sweeps on MI355X.  What they have in common: a ResNet-20
+// layer at batch 256 launches 2048-4096 waves in 256-512 workgroups of eight waves; a lane keeps only
+// 2-4 output channels x 4 positions (few registers, short dependent chains); one pipeline unit is one
+// output channel x one input channel (CQ = 1: 9 weights, 18*TN vector instructions), which keeps the two
+// weight buffers far from the 102-SGPR limit (spilled SGPRs come back as v_readlane inside the hot loop)
+// and works for odd channel counts too.
 //                           TN SPR TH NIMG TM COW CC CQ S
-using FwdW32   = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 2, 1>;    // outputs 32 wide: one image x 16 channels
-using FwdW16   = Tile3x3Cfg<2, 8, 16, 1, 4, 8, 16, 2, 1>;   // outputs 16 wide: one image x 32 channels
-using FwdW8    = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 2, 1>;    // outputs 8 wide: two images x 32 channels
-using FwdW16S2 = Tile3x3Cfg<2, 8, 16, 1, 4, 8, 8, 2, 2>;    // stride 2, outputs 16 wide
-using FwdW8S2  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 2, 2>;    // stride 2, outputs 8 wide
-// same tiles with one input channel per unit, for odd channel counts
-using FwdW32o   = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1, 1>;
-using FwdW16o   = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 16, 1, 1>;
-using FwdW8o    = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1, 1>;
-using FwdW16S2o = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 8, 1, 2>;
-using FwdW8S2o  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1, 2>;
+using FwdW32   = Tile3x3Cfg<4, 8, 16, 1, 4, 4, 8, 1, 1>;    // outputs 32 wide: half an image x 16 channels
+using FwdW16   = Tile3x3Cfg<4, 4, 16, 1, 4, 8, 16, 1, 1>;   // outputs 16 wide: one image x 32 channels
+using FwdW8    = Tile3x3Cfg<4, 2, 8, 4, 2, 8, 16, 1, 1>;    // outputs 8 wide: four images x 16 channels
+using FwdW16S2 = Tile3x3Cfg<2, 8, 16, 1, 4, 8, 8, 1, 2>;    // stride 2, outputs 16 wide: one image x 32 channels
+using FwdW8S2  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 1, 2>;    // stride 2, outputs 8 wide: two images x 32 channels
 
 // which tiled kernel serves these dimensions (0 = none): 1..3 stride 1 by output width, 4..5 stride 2
 static int fwd_tiled_variant(const ConvDims &d) {
@@ -318,13 +313,12 @@ static int fwd_tiled_variant(const ConvDims &d) {
 }
 
 int fwd_stats_slots(const ConvDims &d) {
-    const bool even = d.Ci % 2 == 0;
     switch (fwd_tiled_variant(d)) {
-        case 1: return even ? stats_slots_3x3<FwdW32>(d) : stats_slots_3x3<FwdW32o>(d);
-        case 2: return even ? stats_slots_3x3<FwdW16>(d) : stats_slots_3x3<FwdW16o>(d);
-        case 3: return even ? stats_slots_3x3<FwdW8>(d) : stats_slots_3x3<FwdW8o>(d);
-        case 4: return even ? stats_slots_3x3<FwdW16S2>(d) : stats_slots_3x3<FwdW16S2o>(d);
-        case 5: return even ? stats_slots_3x3<FwdW8S2>(d) : stats_slots_3x3<FwdW8S2o>(d);
+        case 1: return stats_slots_3x3<FwdW32>(d);
+        case 2: return stats_slots_3x3<FwdW16>(d);
+        case 3: return stats_slots_3x3<FwdW8>(d);
+        case 4: return stats_slots_3x3<FwdW16S2>(d);
+        case 5: return stats_slots_3x3<FwdW8S2>(d);
         default: return 0;
     }
 }
@@ -335,16 +329,15 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
     const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 &&
                       (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                       (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0);
-    const bool even = d.Ci % 2 == 0;
-    if (k3p1 && d.stride == 1) {
-        if (d.Wo > 16) return even ? launch_fwd_3x3<FwdW32>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW32o>(x, w, y, stats, d, s);
-        if (d.Wo > 8) return even ? launch_fwd_3x3<FwdW16>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW16o>(x, w, y, stats, d, s);
-        return even ? launch_fwd_3x3<FwdW8>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW8o>(x, w, y, stats, d, s);
-    }
-    if (k3p1 && d.stride == 2) {
-        if (d.Wo > 8)
-            return even ? launch_fwd_3x3<FwdW16S2>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW16S2o>(x, w, y, stats, d, s);
-        return even ? launch_fwd_3x3<FwdW8S2>(x, w, y, stats, d, s) : launch_fwd_3x3<FwdW8S2o>(x, w, y, stats, d, s);
+    if (k3p1) {
+        switch (fwd_tiled_variant(d)) {
+            case 1: return launch_fwd_3x3<FwdW32>(x, w, y, stats, d, s);
+            case 2: return launch_fwd_3x3<FwdW16>(x, w, y, stats, d, s);
+            case 3: return launch_fwd_3x3<FwdW8>(x, w, y, stats, d, s);
+            case 4: return launch_fwd_3x3<FwdW16S2>(x, w, y, stats, d, s);
+            case 5: return launch_fwd_3x3<FwdW8S2>(x, w, y, stats, d, s);
+            default: break;
+        }
     }
     if (stats) return ADDER_ERR_UNSUPPORTED;   // only the tiled kernels have the statistics epilogue
     if (conv1x1_supported(d, x, y)) return launch_fwd_1x1(x, w, y, d, s);

@@ -273,7 +273,8 @@ static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
     p.ntiles = ceil_div(d.N, G::NIMG) * p.tilesH * p.tilesW;
     p.gy = ceil_div(d.Co, G::COB);
     p.gz = ceil_div(d.Ci * 9, G::KB);
-    int want = ceil_div(256, p.gy * p.gz);   // one workgroup per CU: the staged tiles fill most of its LDS
+    // ~2048 waves over the chip (two per SIMD; a workgroup's staged tiles fill a good part of a CU's LDS)
+    int want = ceil_div(2048 / (G::NTHREADS / 64), p.gy * p.gz);
     p.slots = want < p.ntiles ? want : p.ntiles;
     if (p.slots < 1) p.slots = 1;
 }

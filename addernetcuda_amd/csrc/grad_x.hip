@@ -453,24 +453,28 @@ static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, 
 }
 
 //                              TNW BPR TH NIMG TM CIW CC
-using GxS2W32 = GradX3x3S2Cfg<2, 16, 32, 1, 4, 4, 16>;   // inputs 32 wide: one image x 16 channels, 16 waves
+using GxS2W32 = GradX3x3S2Cfg<2, 16, 16, 1, 4, 4, 16>;   // inputs 32 wide: half an image x 16 channels, 8 waves
 using GxS2W16 = GradX3x3S2Cfg<2, 8, 16, 1, 4, 8, 16>;    // inputs 16 wide: one image x 32 channels, 8 waves
 
+// Stride-1 tile shapes, picked by timing sweeps on MI355X: eight waves per workgroup, four input channels
+// x 2-4 positions per lane (few registers; more channels per lane were 20 % slower on every map size).
 //                        TN SPR TH NIMG TM COW CC CQ
-using GxW32 = Tile3x3Cfg<4, 8, 32, 1, 8, 2, 4, 1>;
-using GxW16 = Tile3x3Cfg<2, 8, 16, 1, 8, 4, 16, 1>;
-using GxW8  = Tile3x3Cfg<1, 8, 8, 1, 8, 4, 16, 1>;
+using GxW32 = Tile3x3Cfg<4, 8, 16, 1, 4, 4, 8, 1>;    // inputs 32 wide: half an image x 16 channels
+using GxW16 = Tile3x3Cfg<4, 4, 16, 1, 4, 8, 16, 1>;   // inputs 16 wide: one image x 32 channels
+using GxW8  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 1>;    // inputs 8 wide: two images x 32 channels
+static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
+              "the launcher checks Ci against one TM per stride");
 
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s) {
     const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
-    if (k3s1p1 && d.Ci >= 8 &&
+    if (k3s1p1 && d.Ci >= GxW32::TM &&
         (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0)) {
         if (d.W > 16) return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s);
         if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s);
     }
-    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.W % 2 == 0 && d.Ci >= 8 &&
+    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.W % 2 == 0 && d.Ci >= GxS2W32::TM &&
         (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
         if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s);
