@@ -36,8 +36,8 @@ def test_status_strings_and_version():
     from addernetcuda_amd._lib import lib
     assert lib.adder_abi_version() == 1
     assert lib.adder_strerror(0) == b"ok"
-    seen = {lib.adder_strerror(c) for c in range(-6, 1)}
-    assert len(seen) == 7 and b"unknown status" not in seen
+    seen = {lib.adder_strerror(c) for c in range(-7, 1)}
+    assert len(seen) == 8 and b"unknown status" not in seen
     assert lib.adder_strerror(-99) == b"unknown status"
 
 
@@ -110,3 +110,29 @@ def test_workspace_is_large_enough_for_the_partials_of_big_layers():
                  (64, 256, 56, 56, 64, 1, 1, 1, 0)]:
         assert lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)) == 0
         assert need.value % 256 == 0 and need.value < (2 << 30)
+
+
+def test_statistics_variants_validate_without_a_gpu():
+    """adder_conv2d_fwd_stats_* / adder_bn_act_fwd_stats_f32: slot counts are a host-side function of the
+    dimensions; bad arguments are refused before any HIP call."""
+    from addernetcuda_amd._lib import lib
+    slots = ctypes.c_int(-1)
+    dims32 = (256, 16, 32, 32, 16, 3, 3, 1, 1)
+    assert lib.adder_conv2d_fwd_stats_slots(*dims32, ctypes.byref(slots)) == 0 and slots.value > 0
+    n32 = slots.value
+    assert lib.adder_conv2d_fwd_stats_slots(128, 16, 32, 32, 16, 3, 3, 1, 1, ctypes.byref(slots)) == 0
+    assert slots.value * 2 == n32                                  # slots follow the number of position waves
+    for k, s, p in ((1, 1, 0), (1, 2, 0), (5, 1, 2), (3, 3, 1)):
+        assert lib.adder_conv2d_fwd_stats_slots(4, 8, 16, 16, 8, k, k, s, p, ctypes.byref(slots)) == 0
+        assert slots.value == 0                                    # no statistics epilogue for these kernels
+    assert lib.adder_conv2d_fwd_stats_slots(*dims32, None) == -1
+    fake = ctypes.c_void_p(4096)
+    assert lib.adder_conv2d_fwd_stats_f32(fake, fake, fake, None, n32, *dims32, None) == -1
+    assert lib.adder_conv2d_fwd_stats_f32(fake, fake, ctypes.c_void_p(1 << 40), ctypes.c_void_p(1 << 41), n32 + 1,
+                                          *dims32, None) == -2     # slot count must be the one reported
+    assert lib.adder_conv2d_fwd_stats_f32(fake, fake, ctypes.c_void_p(1 << 40), ctypes.c_void_p(1 << 41), 4,
+                                          4, 8, 16, 16, 8, 1, 1, 1, 0, None) == -7
+    bn = lib.adder_bn_act_fwd_stats_f32
+    args = [fake] * 10 + [0.1, 1e-5, 1, 4, 8, 64]
+    assert bn(*args, None, 4, None) == -1
+    assert bn(*args, fake, 0, None) == -2
