@@ -53,6 +53,24 @@ __device__ __forceinline__ void st4(float *p, const float4 v, int valid) {
     }
 }
 
+template <bool VEC>
+__device__ __forceinline__ float2 ld2(const float *p, int valid) {
+    if constexpr (VEC) return *reinterpret_cast<const float2 *>(p);
+    float2 v = make_float2(0.f, 0.f);
+    if (valid > 0) v.x = p[0];
+    if (valid > 1) v.y = p[1];
+    return v;
+}
+template <bool VEC>
+__device__ __forceinline__ void st2(float *p, const float2 v, int valid) {
+    if constexpr (VEC) {
+        *reinterpret_cast<float2 *>(p) = v;
+    } else {
+        if (valid > 0) p[0] = v.x;
+        if (valid > 1) p[1] = v.y;
+    }
+}
+
 template <int S, int TM, bool VEC = true>
 __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                       float *__restrict__ y, int N, int Ci, int H, int W,
@@ -116,7 +134,7 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
             if constexpr (TN == 4)
                 st4<VEC>(dst, make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]), valid);
             else
-                *reinterpret_cast<float2 *>(dst) = make_float2(tot[m][0], tot[m][1]);
+                st2<VEC>(dst, make_float2(tot[m][0], tot[m][1]), L.ok ? Wo - L.wo0 : 0);
         }
     }
 }
@@ -150,7 +168,7 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
             const float4 v = ld4<VEC>(gp + (size_t)co * gplane, valid);
             g[0] = v.x; g[1] = v.y; g[2] = v.z; g[3] = v.w;
         } else {
-            const float2 v = *reinterpret_cast<const float2 *>(gp + (size_t)co * gplane);
+            const float2 v = ld2<VEC>(gp + (size_t)co * gplane, L.ok ? Wo - L.wo0 : 0);
             g[0] = v.x; g[1] = v.y;
         }
 #pragma unroll
@@ -175,8 +193,8 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
             if constexpr (S == 1) {
                 st4<VEC>(dst, make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]), valid);
             } else {
-                *reinterpret_cast<float4 *>(dst) = make_float4(tot[m][0], 0.f, tot[m][1], 0.f);
-                if (row2) *reinterpret_cast<float4 *>(dst + W) = make_float4(0.f, 0.f, 0.f, 0.f);
+                st4<VEC>(dst, make_float4(tot[m][0], 0.f, tot[m][1], 0.f), valid);
+                if (row2) st4<VEC>(dst + W, make_float4(0.f, 0.f, 0.f, 0.f), valid);
             }
         }
     }
@@ -219,7 +237,7 @@ __global__ __launch_bounds__(256) void grad_w_1x1_kernel(const float *__restrict
                 const float4 v = ld4<VEC>(p, valid);
                 gs[m][0] = v.x; gs[m][1] = v.y; gs[m][2] = v.z; gs[m][3] = v.w;
             } else {
-                const float2 v = *reinterpret_cast<const float2 *>(p);
+                const float2 v = ld2<VEC>(p, Wo - L.wo0);
                 gs[m][0] = v.x; gs[m][1] = v.y;
             }
         }
@@ -274,13 +292,10 @@ __global__ __launch_bounds__(256) void grad_w_1x1_kernel(const float *__restrict
 // ---- host side ------------------------------------------------------------------
 // Stride 1: positions are independent, so every (H, W) plane is walked as one row of H*W elements; planes
 // whose size is not a multiple of 4 (7x7) or whose base is not 16-byte aligned take the element-wise loads.
-// Stride 2: one aligned float4 of the source row per lane, whole float2 groups of the output row.
-bool conv1x1_supported(const ConvDims &d, const void *a, const void *b) {
-    if (d.kh != 1 || d.kw != 1 || d.pad != 0 || (d.stride != 1 && d.stride != 2)) return false;
-    if (d.stride == 1) return true;
-    if (d.W % 4 != 0 || d.Wo % 2 != 0) return false;
-    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) return false;
-    return true;
+// Stride 2: one float4 of the source row per lane (two of its elements are sampled) and a float2 of the
+// output row; rows that are not whole aligned groups (W % 4, Wo % 2, base pointers) are read element-wise.
+bool conv1x1_supported(const ConvDims &d, const void *, const void *) {
+    return d.kh == 1 && d.kw == 1 && d.pad == 0 && (d.stride == 1 || d.stride == 2);
 }
 
 // dimensions the kernels are launched with
@@ -292,7 +307,8 @@ static ConvDims lane_dims(const ConvDims &d) {
 
 static bool vec_ok(const ConvDims &f, const void *a, const void *b, const void *c) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
-    return f.stride == 2 || (f.W % 4 == 0 && (bits & 15) == 0);
+    if (f.stride == 2) return f.W % 4 == 0 && f.Wo % 2 == 0 && (bits & 15) == 0;
+    return f.W % 4 == 0 && (bits & 15) == 0;
 }
 
 static void lane_space(const ConvDims &f, int &gpr, int &groups) {
@@ -306,9 +322,12 @@ int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, 
     int gpr, groups;
     lane_space(f, gpr, groups);
     const dim3 grid(ceil_div(groups, 256), ceil_div(f.Co, TM));
-    if (f.stride == 2)
-        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co, f.Ho,
-                           f.Wo, gpr, groups);
+    if (f.stride == 2 && vec_ok(f, x, y, nullptr))
+        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM, true>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+                           f.Ho, f.Wo, gpr, groups);
+    else if (f.stride == 2)
+        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM, false>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+                           f.Ho, f.Wo, gpr, groups);
     else if (vec_ok(f, x, y, nullptr))
         hipLaunchKernelGGL((fwd_1x1_kernel<1, TM, true>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
                            f.Ho, f.Wo, gpr, groups);
@@ -325,9 +344,12 @@ int launch_grad_x_1x1(const float *gy, const float *x, const float *w, float *gx
     int gpr, groups;
     lane_space(f, gpr, groups);
     const dim3 grid(ceil_div(groups, 256), ceil_div(f.Ci, TM));
-    if (f.stride == 2)
-        hipLaunchKernelGGL((grad_x_1x1_kernel<2, TM>), grid, dim3(256), 0, s, gy, x, w, gx, f.N, f.Ci, f.H, f.W,
+    if (f.stride == 2 && vec_ok(f, gy, x, gx))
+        hipLaunchKernelGGL((grad_x_1x1_kernel<2, TM, true>), grid, dim3(256), 0, s, gy, x, w, gx, f.N, f.Ci, f.H, f.W,
                            f.Co, f.Ho, f.Wo, gpr, groups);
+    else if (f.stride == 2)
+        hipLaunchKernelGGL((grad_x_1x1_kernel<2, TM, false>), grid, dim3(256), 0, s, gy, x, w, gx, f.N, f.Ci, f.H,
+                           f.W, f.Co, f.Ho, f.Wo, gpr, groups);
     else if (vec_ok(f, gy, x, gx))
         hipLaunchKernelGGL((grad_x_1x1_kernel<1, TM, true>), grid, dim3(256), 0, s, gy, x, w, gx, f.N, f.Ci, f.H, f.W,
                            f.Co, f.Ho, f.Wo, gpr, groups);
@@ -356,9 +378,12 @@ int launch_grad_w_1x1(const float *gy, const float *x, float *part, float *sgpar
     int gpr, groups;
     lane_space(f, gpr, groups);
     const dim3 grid(slots, ceil_div(f.Co, kGw1x1TM), ceil_div(f.Ci, kGw1x1TC));
-    if (f.stride == 2)
-        hipLaunchKernelGGL((grad_w_1x1_kernel<2, kGw1x1TM, kGw1x1TC>), grid, dim3(256), 0, s, gy, x, part, sgpart,
-                           f.N, f.Ci, f.H, f.W, f.Co, f.Ho, f.Wo, gpr, groups);
+    if (f.stride == 2 && vec_ok(f, gy, x, nullptr))
+        hipLaunchKernelGGL((grad_w_1x1_kernel<2, kGw1x1TM, kGw1x1TC, true>), grid, dim3(256), 0, s, gy, x, part,
+                           sgpart, f.N, f.Ci, f.H, f.W, f.Co, f.Ho, f.Wo, gpr, groups);
+    else if (f.stride == 2)
+        hipLaunchKernelGGL((grad_w_1x1_kernel<2, kGw1x1TM, kGw1x1TC, false>), grid, dim3(256), 0, s, gy, x, part,
+                           sgpart, f.N, f.Ci, f.H, f.W, f.Co, f.Ho, f.Wo, gpr, groups);
     else if (vec_ok(f, gy, x, nullptr))
         hipLaunchKernelGGL((grad_w_1x1_kernel<1, kGw1x1TM, kGw1x1TC, true>), grid, dim3(256), 0, s, gy, x, part,
                            sgpart, f.N, f.Ci, f.H, f.W, f.Co, f.Ho, f.Wo, gpr, groups);

@@ -479,7 +479,7 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s);
     }
-    if (conv1x1_supported(d, gy, gx) && (d.stride == 1 || (reinterpret_cast<uintptr_t>(x) & 15) == 0))
+    if (conv1x1_supported(d, gy, gx))
         return launch_grad_x_1x1(gy, x, w, gx, d, s);
     constexpr int TM = 8;
     const long total = (long)d.N * d.H * d.W;

@@ -47,6 +47,24 @@ RESNET20_LAYERS = [
     (1, 32, 16, 16, 64, 3, 2, 1),
     (5, 64, 8, 8, 64, 3, 1, 1),
 ]
+# adder layers of the two other model configurations the reference ships (vgg.py / resnet50.py shapes at the
+# batch sizes its README quotes): (count, Ci, H, W, Co, k, stride, pad); batch 128 and 64
+VGG_SMALL_LAYERS = [
+    (1, 128, 32, 32, 128, 3, 1, 1), (1, 128, 16, 16, 256, 3, 1, 1), (1, 256, 16, 16, 256, 3, 1, 1),
+    (1, 256, 8, 8, 512, 3, 1, 1), (1, 512, 8, 8, 512, 3, 1, 1),
+]
+RESNET50_LAYERS = [
+    (4, 64, 56, 56, 256, 1, 1, 0), (1, 64, 56, 56, 64, 1, 1, 0), (3, 64, 56, 56, 64, 3, 1, 1),
+    (2, 256, 56, 56, 64, 1, 1, 0), (1, 256, 56, 56, 512, 1, 2, 0), (1, 256, 56, 56, 128, 1, 1, 0),
+    (1, 128, 56, 56, 128, 3, 2, 1), (4, 128, 28, 28, 512, 1, 1, 0), (3, 512, 28, 28, 128, 1, 1, 0),
+    (3, 128, 28, 28, 128, 3, 1, 1), (1, 512, 28, 28, 1024, 1, 2, 0), (1, 512, 28, 28, 256, 1, 1, 0),
+    (1, 256, 28, 28, 256, 3, 2, 1), (6, 256, 14, 14, 1024, 1, 1, 0), (5, 1024, 14, 14, 256, 1, 1, 0),
+    (5, 256, 14, 14, 256, 3, 1, 1), (1, 1024, 14, 14, 2048, 1, 2, 0), (1, 1024, 14, 14, 512, 1, 1, 0),
+    (1, 512, 14, 14, 512, 3, 2, 1), (3, 512, 7, 7, 2048, 1, 1, 0), (2, 2048, 7, 7, 512, 1, 1, 0),
+    (2, 512, 7, 7, 512, 3, 1, 1),
+]
+LAYER_SETS = {"resnet20": (BATCH, RESNET20_LAYERS), "vgg_small": (128, VGG_SMALL_LAYERS),
+              "resnet50": (64, RESNET50_LAYERS)}
 # flops per (co, k, position) term and the fewest fp32 VALU instructions that implement it
 OPS = {"fwd": (2, 2), "grad_x": (4, 3), "grad_w": (3, 1)}
 
@@ -91,10 +109,11 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
     return E, ops, keep
 
 
-def bench_layers(dev, warmup=5, iters=20):
+def bench_layers(dev, warmup=5, iters=20, which="resnet20"):
     rows = []
-    for cnt, Ci, H, W, Co, k, s, p in RESNET20_LAYERS:
-        E, ops, keep = layer_ops(BATCH, Ci, H, W, Co, k, s, p, dev)
+    batch, layers = LAYER_SETS[which]
+    for cnt, Ci, H, W, Co, k, s, p in layers:
+        E, ops, keep = layer_ops(batch, Ci, H, W, Co, k, s, p, dev)
         for name, fn in ops.items():
             t = event_time(fn, warmup, iters)
             flop, slots = OPS[name]
@@ -264,6 +283,9 @@ def main():
     ap.add_argument("--layers-only", action="store_true",
                     help="run only the per-layer table (7 ResNet-20 layer shapes x forward / grad_X / grad_W); "
                          "meant to run under rocprofv3 --pmc / --kernel-trace")
+    ap.add_argument("--layer-set", choices=sorted(LAYER_SETS), default="resnet20",
+                    help="with --layers-only: the adder layers of ResNet-20 (batch 256), the VGG-small stack "
+                         "(batch 128) or ResNet-50 at 224x224 (batch 64)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (every box here has a single MI355X)")
@@ -282,7 +304,9 @@ def main():
         return
 
     if args.layers_only:
-        print(json.dumps({"layers": bench_layers(dev, warmup=2, iters=max(3, min(args.steps, 20)))}))
+        rows = bench_layers(dev, warmup=2, iters=max(3, min(args.steps, 20)), which=args.layer_set)
+        print(json.dumps({"layer_set": args.layer_set, "batch": LAYER_SETS[args.layer_set][0], "layers": rows,
+                          "adder_kernel_ms_per_step": round(sum(r["us"] * r["count"] for r in rows) / 1e3, 3)}))
         return
 
     mode = "eager"

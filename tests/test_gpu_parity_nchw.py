@@ -40,10 +40,12 @@ TILED = [
     (3, 16, 14, 14, 24, 1, 1, 0),   # 1x1 on a 14x14 plane (walked as one row of 196)
     (3, 12, 7, 7, 20, 1, 1, 0),     # 1x1 on a 7x7 plane: 49 elements, element-wise loads, partial last group
     (1, 5, 3, 5, 3, 1, 1, 0),       # 1x1, 15-element planes
+    (2, 16, 14, 14, 24, 1, 2, 0),   # 1x1 stride 2, 14 -> 7 (ResNet-50's last downsample): odd output width
+    (2, 6, 9, 9, 10, 1, 2, 0),      # 1x1 stride 2 on odd maps: the last column and row have no right / lower neighbour
+    (2, 4, 6, 10, 8, 1, 2, 0),      # 1x1 stride 2, W = 10 (even, not a multiple of 4), Wo = 5
 ]
 GENERIC = [
     (2, 4, 9, 9, 6, 3, 2, 1),       # strided 3x3, odd size
-    (2, 4, 9, 9, 6, 1, 2, 0),       # strided 1x1, odd size
     (2, 3, 7, 7, 5, 3, 1, 1),       # W % 4 != 0
     (1, 4, 11, 9, 6, 5, 1, 2),      # 5x5
     (2, 3, 11, 9, 4, 3, 3, 2),      # stride 3, floor output size
