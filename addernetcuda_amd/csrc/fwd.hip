@@ -91,7 +91,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
                                                                 double *__restrict__ stats, int N, int Ci,
                                                                 int H, int W, int Co, int Ho, int Wo,
                                                                 int tilesH, int tilesW) {
-    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, S = C::S, STRIP = C::STRIP;
+    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, S = C::S, STRIP = C::STRIP, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
 
     int b = blockIdx.x;
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     const int row = (p / C::SPR) % C::TH;
     const int img = p / (C::SPR * C::TH);
     const int co_base = (blockIdx.y * C::COW + cw) * TM;
-    const int K = Ci * 9;
+    const int K = Ci * KK;
     uniform_f32_ptr wc = as_uniform(w);
 
     // wave-uniform weight row offsets (clamped so tail channels read valid memory)
@@ -130,13 +130,13 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     const int nchunks = ceil_div(Ci, C::CC);
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch, VEC>(st, x, 0, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+    tile_fetch<typename C::Patch, VEC>(st, x, 0, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W);
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int ci0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Ci - ci0);
@@ -144,41 +144,41 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
         // group cc+CQ and the weights of the next output channel are requested right after
         // the first subtract of the current one, i.e. after the wait for the current
         // operands and with the rest of the arithmetic still ahead to hide the latency.
-        float xr[2][CQ][3][STRIP];
-        float wv[2][CQ * 9];
+        float xr[2][CQ][KS][STRIP];
+        float wv[2][CQ * KK];
 #pragma unroll
         for (int q = 0; q < CQ; ++q)
 #pragma unroll
-            for (int i = 0; i < 3; ++i)
+            for (int i = 0; i < KS; ++i)
                 lds_read_strip<STRIP, C::STRIP_ALIGN>(lbase + q * C::PLANE + i * C::PITCH, xr[0][q][i]);
 #pragma unroll
-        for (int e = 0; e < CQ * 9; ++e) wv[0][e] = wc[wrow[0] + ci0 * 9 + e];
+        for (int e = 0; e < CQ * KK; ++e) wv[0][e] = wc[wrow[0] + ci0 * KK + e];
 
         auto half = [&](const int cc, const int cur) {
             // cur = 0/1: which xr buffer holds channel group cc
-            const int kofs = (ci0 + cc) * 9;
+            const int kofs = (ci0 + cc) * KK;
             const bool more = cc + CQ < ccnt;
-            const int knext = more ? kofs + CQ * 9 : kofs;  // clamped: stays inside the weight row
+            const int knext = more ? kofs + CQ * KK : kofs;  // clamped: stays inside the weight row
 #pragma unroll
             for (int m = 0; m < TM; ++m) {
 #pragma unroll
-                for (int idx = 0; idx < CQ * 9 * TN; ++idx) {
-                    const int t = idx % TN, j = (idx / TN) % 3, i = (idx / TN / 3) % 3, q = idx / TN / 9;
-                    acc[m][t] -= fabsf(wv[m & 1][q * 9 + i * 3 + j] - xr[cur][q][i][t * S + j]);
+                for (int idx = 0; idx < CQ * KK * TN; ++idx) {
+                    const int t = idx % TN, j = (idx / TN) % KS, i = (idx / TN / KS) % KS, q = idx / TN / KK;
+                    acc[m][t] -= fabsf(wv[m & 1][q * KK + i * KS + j] - xr[cur][q][i][t * S + j]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
                         if (m + 1 < TM) {
 #pragma unroll
-                            for (int e = 0; e < CQ * 9; ++e) wv[(m + 1) & 1][e] = wc[wrow[m + 1] + kofs + e];
+                            for (int e = 0; e < CQ * KK; ++e) wv[(m + 1) & 1][e] = wc[wrow[m + 1] + kofs + e];
                         } else {
 #pragma unroll
-                            for (int e = 0; e < CQ * 9; ++e) wv[(m + 1) & 1][e] = wc[wrow[0] + knext + e];
+                            for (int e = 0; e < CQ * KK; ++e) wv[(m + 1) & 1][e] = wc[wrow[0] + knext + e];
                         }
                         if (m == 0 && more) {
 #pragma unroll
                             for (int q2 = 0; q2 < CQ; ++q2)
 #pragma unroll
-                                for (int i2 = 0; i2 < 3; ++i2)
+                                for (int i2 = 0; i2 < KS; ++i2)
                                     lds_read_strip<STRIP, C::STRIP_ALIGN>(
                                         lbase + (cc + CQ + q2) * C::PLANE + i2 * C::PITCH, xr[cur ^ 1][q2][i2]);
                         }
@@ -303,13 +303,29 @@ using FwdW16   = Tile3x3Cfg<4, 4, 16, 1, 4, 8, 16, 1, 1>;   // outputs 16 wide: 
 using FwdW8    = Tile3x3Cfg<4, 2, 8, 4, 2, 8, 16, 1, 1>;    // outputs 8 wide: four images x 16 channels
 using FwdW16S2 = Tile3x3Cfg<2, 8, 16, 1, 4, 8, 8, 1, 2>;    // stride 2, outputs 16 wide: one image x 32 channels
 using FwdW8S2  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 1, 2>;    // stride 2, outputs 8 wide: two images x 32 channels
+// 1x1, stride 1: every (H, W) plane is one row of H*W positions; a unit is one output channel x 8 input
+// channels (8 weights, 64 vector instructions), eight output-channel waves share the staged x tile.
+using Fwd1x1   = Tile3x3Cfg<4, 64, 1, 1, 4, 8, 16, 8, 1, 1>;   // 256 positions of one image x 32 channels
+using Fwd1x1s  = Tile3x3Cfg<4, 16, 1, 4, 4, 8, 16, 8, 1, 1>;   // planes of <= 64 positions: four images
 
-// which tiled kernel serves these dimensions (0 = none): 1..3 stride 1 by output width, 4..5 stride 2
+// which tiled kernel serves these dimensions (0 = none): 1..3 3x3 stride 1 by output width, 4..5 3x3 stride 2,
+// 6..7 1x1 stride 1 by plane size
 static int fwd_tiled_variant(const ConvDims &d) {
+    // (below 64 input channels the plain 1x1 kernel of conv1x1.hip is as fast or faster)
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci % Fwd1x1::CQ == 0 && d.Ci >= 64)
+        return d.H * d.W > 64 ? 6 : 7;
     if (d.kh != 3 || d.kw != 3 || d.pad != 1) return 0;
     if (d.stride == 1) return d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
     if (d.stride == 2) return d.Wo > 8 ? 4 : 5;
     return 0;
+}
+
+// a stride-1 1x1 layer seen as N x Ci "images" of one row of H*W positions
+static ConvDims as_one_row(const ConvDims &d) {
+    ConvDims f = d;
+    f.H = f.Ho = 1;
+    f.W = f.Wo = d.H * d.W;
+    return f;
 }
 
 int fwd_stats_slots(const ConvDims &d) {
@@ -319,6 +335,8 @@ int fwd_stats_slots(const ConvDims &d) {
         case 3: return stats_slots_3x3<FwdW8>(d);
         case 4: return stats_slots_3x3<FwdW16S2>(d);
         case 5: return stats_slots_3x3<FwdW8S2>(d);
+        case 6: return stats_slots_3x3<Fwd1x1>(as_one_row(d));
+        case 7: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
         default: return 0;
     }
 }
@@ -329,8 +347,15 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
     const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 &&
                       (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                       (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0);
+    const int variant = fwd_tiled_variant(d);
+    if (variant >= 6) {
+        const ConvDims f = as_one_row(d);
+        if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0)
+            return variant == 6 ? launch_fwd_3x3<Fwd1x1>(x, w, y, stats, f, s)
+                                : launch_fwd_3x3<Fwd1x1s>(x, w, y, stats, f, s);
+    }
     if (k3p1) {
-        switch (fwd_tiled_variant(d)) {
+        switch (variant) {
             case 1: return launch_fwd_3x3<FwdW32>(x, w, y, stats, d, s);
             case 2: return launch_fwd_3x3<FwdW16>(x, w, y, stats, d, s);
             case 3: return launch_fwd_3x3<FwdW8>(x, w, y, stats, d, s);

@@ -89,7 +89,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
                                                                    float *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int tilesH,
                                                                    int tilesW) {
-    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ;
+    constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
 
     int b = blockIdx.x;
@@ -111,8 +111,8 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     // below ci_first belong to the previous group and are not stored.
     const int ci_first = (blockIdx.y * C::COW + cw) * TM;
     const int ci_base = __builtin_amdgcn_readfirstlane(min(ci_first, Ci - TM));
-    const int K = Ci * 9;
-    uniform_f32_ptr wc = as_uniform(w) + ci_base * 9;
+    const int K = Ci * KK;
+    uniform_f32_ptr wc = as_uniform(w) + ci_base * KK;
 
     const int n = n0 + img, hi = h0 + row, wi0 = w0 + strip * TN;
     const bool pos_ok = lane_ok && n < N && hi < H;
@@ -136,13 +136,13 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     const int nchunks = ceil_div(Co, C::CC);
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, h0 - 1, w0, H, W);
+    tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, h0 - C::PAD, w0, H, W);
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int co0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, gy, co0 + C::CC, Co, n0, N, h0 - 1, w0, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, gy, co0 + C::CC, Co, n0, N, h0 - C::PAD, w0, H, W);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
@@ -153,12 +153,12 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
         static_assert(CQ == 1, "pipeline is written for one output channel per step");
         // input channels per unit: keeps ~100 vector instructions per unit and both weight
         // buffers (2 * 9 * HM SGPRs) well inside the scalar register file
-        constexpr int HM = TN >= 4 ? 1 : 2, NU = TM / HM, HW = HM * 9;
-        static_assert(TM % HM == 0 && NU % 2 == 0, "even number of units per output channel");
-        float gr[2][3][TN + 2];
+        constexpr int HM = KS == 1 ? TM : (TN >= 4 ? 1 : 2), NU = TM / HM, HW = HM * KK;
+        static_assert(TM % HM == 0 && (NU % 2 == 0 || NU == 1), "one unit or an even number of units per output channel");
+        float gr[2][KS][TN + KS - 1];
         float wv[2][HW];
 #pragma unroll
-        for (int i = 0; i < 3; ++i) lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + i * C::PITCH, gr[0][i]);
+        for (int i = 0; i < KS; ++i) lds_read_strip<TN + KS - 1, C::STRIP_ALIGN>(lbase + i * C::PITCH, gr[0][i]);
 #pragma unroll
         for (int e = 0; e < HW; ++e) wv[0][e] = wc[co0 * K + e];
 
@@ -168,25 +168,27 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
             const int knext = more ? kofs + K : kofs;
 #pragma unroll
             for (int h = 0; h < NU; ++h) {
+                // weight buffer of this unit: the buffers alternate from unit to unit, also across channels
+                const int wb = (cur * (NU & 1) + h) & 1;
 #pragma unroll
-                for (int idx = 0; idx < HM * 9 * TN; ++idx) {
-                    const int t = idx % TN, j = (idx / TN) % 3, i = (idx / TN / 3) % 3, mm = idx / TN / 9;
+                for (int idx = 0; idx < HM * KK * TN; ++idx) {
+                    const int t = idx % TN, j = (idx / TN) % KS, i = (idx / TN / KS) % KS, mm = idx / TN / KK;
                     const int m = h * HM + mm;
-                    acc[m][t] = fmaf(hardtanh(wv[h & 1][mm * 9 + i * 3 + j] - xr[m][t]), gr[cur][2 - i][t + 2 - j],
+                    acc[m][t] = fmaf(hardtanh(wv[wb][mm * KK + i * KS + j] - xr[m][t]), gr[cur][KS - 1 - i][t + KS - 1 - j],
                                      acc[m][t]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
                         if (h + 1 < NU) {
 #pragma unroll
-                            for (int e = 0; e < HW; ++e) wv[(h + 1) & 1][e] = wc[kofs + (h + 1) * HW + e];
+                            for (int e = 0; e < HW; ++e) wv[wb ^ 1][e] = wc[kofs + (h + 1) * HW + e];
                         } else {
 #pragma unroll
-                            for (int e = 0; e < HW; ++e) wv[0][e] = wc[knext + e];
+                            for (int e = 0; e < HW; ++e) wv[wb ^ 1][e] = wc[knext + e];
                         }
                         if (h == 0 && more) {
 #pragma unroll
-                            for (int i2 = 0; i2 < 3; ++i2)
-                                lds_read_strip<TN + 2, C::STRIP_ALIGN>(lbase + (cc + 1) * C::PLANE + i2 * C::PITCH,
+                            for (int i2 = 0; i2 < KS; ++i2)
+                                lds_read_strip<TN + KS - 1, C::STRIP_ALIGN>(lbase + (cc + 1) * C::PLANE + i2 * C::PITCH,
                                                                        gr[cur ^ 1][i2]);
                         }
                         __builtin_amdgcn_sched_barrier(0);
@@ -462,6 +464,9 @@ using GxS2W16 = GradX3x3S2Cfg<2, 8, 16, 1, 4, 8, 16>;    // inputs 16 wide: one 
 using GxW32 = Tile3x3Cfg<4, 8, 16, 1, 4, 4, 8, 1>;    // inputs 32 wide: half an image x 16 channels
 using GxW16 = Tile3x3Cfg<4, 4, 16, 1, 4, 8, 16, 1>;   // inputs 16 wide: one image x 32 channels
 using GxW8  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 1>;    // inputs 8 wide: two images x 32 channels
+// 1x1, stride 1: (H, W) planes walked as one row; a unit is one output channel x the lane's 8 input channels
+using Gx1x1  = Tile3x3Cfg<2, 64, 1, 1, 8, 8, 16, 1, 1, 1>;    // 128 positions of one image x 64 channels
+using Gx1x1s = Tile3x3Cfg<4, 16, 1, 4, 8, 8, 16, 1, 1, 1>;    // planes of <= 64 positions: four images
 static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
               "the launcher checks Ci against one TM per stride");
 
@@ -478,6 +483,13 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
         if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);
         return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s);
+    }
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 64) {
+        ConvDims f = d;   // every (H, W) plane as one row of H*W positions
+        f.H = f.Ho = 1;
+        f.W = f.Wo = d.H * d.W;
+        if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0)
+            return f.W > 64 ? launch_grad_x_3x3s1<Gx1x1>(gy, x, w, gx, f, s) : launch_grad_x_3x3s1<Gx1x1s>(gy, x, w, gx, f, s);
     }
     if (conv1x1_supported(d, gy, gx))
         return launch_grad_x_1x1(gy, x, w, gx, d, s);

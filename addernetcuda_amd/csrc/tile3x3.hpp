@@ -119,22 +119,24 @@ __device__ __forceinline__ void tile_commit(const TileStage<P> &st, float *buf) 
     }
 }
 
-// Geometry of the tiled 3x3 / pad-1 kernels (see the header comment).
-template <int TN_, int SPR_, int TH_, int NIMG_, int TM_, int COW_, int CC_, int CQ_, int S_ = 1>
+// Geometry of the tiled kernels (see the header comment).  KS = 3: 3x3 taps, pad 1.  KS = 1: a single tap,
+// pad 0 -- no halo; the forward uses it for 1x1 layers, whose (H, W) planes it walks as one long row.
+template <int TN_, int SPR_, int TH_, int NIMG_, int TM_, int COW_, int CC_, int CQ_, int S_ = 1, int KS_ = 3>
 struct Tile3x3Cfg {
     static constexpr int TN = TN_, SPR = SPR_, TH = TH_, NIMG = NIMG_, TM = TM_, COW = COW_,
-                         CC = CC_, CQ = CQ_, S = S_;
+                         CC = CC_, CQ = CQ_, S = S_, KS = KS_, KK = KS_ * KS_, PAD = KS_ / 2;
     static constexpr int TW = TN * SPR;
     static constexpr int LANES = NIMG * TH * SPR;
     static constexpr int POSW = ceil_div(LANES, 64);
     static constexpr int NTHREADS = 64 * POSW * COW;
-    // stride 2 never reads past the interior on the right
-    using Patch = PatchCfg<NIMG, CC, (TH - 1) * S + 3, TW * S, 1, (S == 1) ? 1 : 0, NTHREADS>;
+    // stride 2 never reads past the interior on the right; a single tap has no halo at all
+    using Patch = PatchCfg<NIMG, CC, (TH - 1) * S + KS, TW * S, PAD, (S == 1) ? PAD : 0, NTHREADS>;
     static constexpr int PITCH = Patch::PITCH, PLANE = Patch::PLANE, BUF = Patch::BUF;
     static constexpr int LDS_BYTES = 2 * BUF * 4;
-    static constexpr int STRIP = (TN - 1) * S + 3;  // floats a lane reads per tile row
+    static constexpr int STRIP = (TN - 1) * S + KS;  // floats a lane reads per tile row
     static constexpr int STRIP_ALIGN = ((TN * S) % 4 == 0) ? 4 : ((TN * S) % 2 == 0 ? 2 : 1);
     static_assert(S == 1 || S == 2, "stride 1 or 2");
+    static_assert(KS == 1 || KS == 3, "one tap or 3x3 taps");
     static_assert(CC % CQ == 0, "CC must be a multiple of CQ");
 };
 
