@@ -41,6 +41,8 @@ TILED = [
     (3, 64, 14, 14, 72, 1, 1, 0),   # tiled 1x1 kernels (>= 64 channels): 196-position planes, channel tail on Co
     (5, 72, 7, 7, 64, 1, 1, 0),     # tiled 1x1, 49-position planes (four images per tile, N = 5), Ci = 72
     (2, 64, 20, 20, 64, 1, 1, 0),   # tiled 1x1, 400-position planes: several tiles per plane
+    (2, 64, 28, 28, 72, 1, 2, 0),   # 1x1 stride 2 with many channels, Wo = 14
+    (3, 68, 14, 14, 64, 1, 2, 0),   # 1x1 stride 2, W = 14 -> Wo = 7, Ci = 68
     (3, 12, 7, 7, 20, 1, 1, 0),     # 1x1 on a 7x7 plane: 49 elements, element-wise loads, partial last group
     (1, 5, 3, 5, 3, 1, 1, 0),       # 1x1, 15-element planes
     (2, 16, 14, 14, 24, 1, 2, 0),   # 1x1 stride 2, 14 -> 7 (ResNet-50's last downsample): odd output width
