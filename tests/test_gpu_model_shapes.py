@@ -40,3 +40,23 @@ def test_layer_matches_oracle(case, gpu):
     assert_close(y, c_oracle.conv2d_fwd(x, w, s, p), f"forward {case}")
     assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p), f"grad_X {case}")
     assert_close(wg.grad, c_oracle.conv2d_grad_w(gy, x, w, s, p), f"grad_W {case}")
+
+
+@pytest.mark.parametrize("case", [(2, 64, 28, 28, 96, 1, 2, 0), (2, 128, 14, 14, 64, 1, 2, 0), (1, 64, 9, 9, 64, 1, 3, 0)], ids=str)
+def test_strided_1x1_with_many_channels_runs_on_the_subsampled_input(case, gpu):
+    """adder2d_function turns these into the stride-1 layer on x[:, :, ::s, ::s]; results and both gradients
+    (the input gradient scattered back with exact zeros in between) must be those of the strided layer."""
+    from addernetcuda_amd import adder
+    from oracle import c_oracle
+    N, Ci, H, W, Co, k, s, p = case
+    x, w, gy = make_case(*case)
+    xg, wg = x.to(gpu).requires_grad_(True), w.to(gpu).requires_grad_(True)
+    y = adder.adder2d_function(xg, wg, s, p, eta=0.0)
+    y.backward(gy.to(gpu))
+    torch.cuda.synchronize()
+    assert_close(y, c_oracle.conv2d_fwd(x, w, s, p), "y")
+    assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p), "grad_x")
+    assert_close(wg.grad, c_oracle.conv2d_grad_w(gy, x, w, s, p), "grad_w")
+    mask = torch.ones(H, W, dtype=torch.bool)
+    mask[::s, ::s] = False
+    assert (xg.grad.cpu()[:, :, mask] == 0).all()
