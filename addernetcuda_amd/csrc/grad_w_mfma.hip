@@ -1,4 +1,4 @@
-// Weight gradient of the 3x3 / pad-1 AdderNet convolution on the matrix cores, in full precision.
+// Weight gradient of the AdderNet convolution (3x3 / pad 1, or 1x1 / stride 1) on the matrix cores, in full precision.
 //
 //   gw[co,k] = sum_pos xcol[k,pos] * gy[co,pos]  -  w[co,k] * sum_pos gy[co,pos]      (k = (ci, i, j))
 //
@@ -27,15 +27,17 @@ namespace adder {
 
 typedef double double4v __attribute__((ext_vector_type(4)));
 
-template <int S_, int TH_, int TW_, int NIMG_, int MT_, int NT_, int MW_, int NW_, int PW_>
+template <int S_, int TH_, int TW_, int NIMG_, int MT_, int NT_, int MW_, int NW_, int PW_, int KS_ = 3>
 struct GwMfmaCfg {
     static constexpr int S = S_, TH = TH_, TW = TW_, NIMG = NIMG_, MT = MT_, NT = NT_, MW = MW_, NW = NW_, PW = PW_;
+    static constexpr int KS = KS_, KK = KS_ * KS_, PAD = KS_ / 2;   // 3x3 taps with pad 1, or a single tap
     static constexpr int COB = 16 * MT * MW;          // output channels per workgroup
     static constexpr int KB = 16 * NT * NW;           // k columns per workgroup
-    static constexpr int CIB = KB / 9;                // = input channels per workgroup
+    static constexpr int CIB = KB / KK;               // = input channels per workgroup
     static constexpr int NWAVES = MW * NW * PW;
     static constexpr int NTHREADS = 64 * NWAVES;
-    using XP = PatchCfg<NIMG, CIB, (TH - 1) * S + 3, TW * S, 1, (S == 1) ? 1 : 0, NTHREADS, 3>;
+    // LPAD puts the interior columns on a 16-byte boundary (3 + one halo column, or no halo at all)
+    using XP = PatchCfg<NIMG, CIB, (TH - 1) * S + KS, TW * S, PAD, (S == 1) ? PAD : 0, NTHREADS, PAD ? 3 : 0>;
     static constexpr int GPLANE = TH * TW + 4;        // +4: channel planes start 4 banks apart
     static constexpr int GBUF = NIMG * COB * GPLANE;
     static constexpr int GUNITS = NIMG * COB * TH * TW / 4;
@@ -47,7 +49,7 @@ struct GwMfmaCfg {
     static constexpr int RED = 2 * (NWAVES / 2) * (REGS + MT) * 64;  // fp64 fold area, in floats
     static constexpr int LDS_FLOATS = (2 * BUF > RED) ? 2 * BUF : RED;
     static constexpr int LDS_BYTES = LDS_FLOATS * 4;
-    static_assert(KB % 9 == 0, "a workgroup's k block must cover whole input channels");
+    static_assert(KB % KK == 0, "a workgroup's k block must cover whole input channels");
     static_assert(TW % 4 == 0 && STEPS % PW == 0, "positions must split evenly over the position waves");
     static_assert((PW & (PW - 1)) == 0, "the fold is a binary tree over the position waves");
     static_assert(NTHREADS <= 1024 && LDS_BYTES <= 160 * 1024, "workgroup limits");
@@ -122,8 +124,8 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int j = (nw * NT + nt) * 16 + l16;        // k column within the workgroup's block
-        const int ci = j / 9, tap = j - ci * 9, ti = tap / 3, tj = tap - ti * 3;
-        b_base[nt] = ci * XP::PLANE + ti * XP::PITCH + XP::LPAD + tj + lk * S;
+        const int ci = j / G::KK, tap = j - ci * G::KK, ti = tap / G::KS, tj = tap - ti * G::KS;
+        b_base[nt] = ci * XP::PLANE + ti * XP::PITCH + XP::ICOL0 - G::PAD + tj + lk * S;
     }
 
     double4v acc[MT][NT];
@@ -146,7 +148,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
     };
     if (tile < ntiles) {
         decode(tile);
-        tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+        tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W);
         gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         tile_commit<XP>(xs, smem);
         gy_commit_m<G>(gs, smem + XP::BUF);
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
         const int next = tile + gridDim.x;
         if (next < ntiles) {   // next tile's global loads fly during this tile's arithmetic
             decode(next);
-            tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - 1, w0 * S, H, W);
+            tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W);
             gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         }
         const float *base = smem + cur * G::BUF;
@@ -233,7 +235,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
     }
     if (pw != 0) return;
 
-    const int K = Ci * 9;
+    const int K = Ci * G::KK;
     double *dst = part + (size_t)blockIdx.x * Co * K;   // fp64 slabs: partials of opposite sign cancel across slots
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -265,6 +267,11 @@ using GmW16   = GwMfmaCfg<1, 16, 16, 1, 1, 9, 1, 1, 8>;  // outputs 16 wide: one
 using GmW8    = GwMfmaCfg<1, 8, 8, 4, 1, 9, 1, 1, 8>;    // outputs 8 wide:  four images
 using GmW16S2 = GwMfmaCfg<2, 8, 16, 1, 1, 9, 1, 1, 8>;   // stride 2, outputs 16 wide: half an image
 using GmW8S2  = GwMfmaCfg<2, 8, 8, 2, 1, 9, 1, 1, 8>;    // stride 2, outputs 8 wide: two images
+// 1x1, stride 1: a plain (Co x positions) x (positions x Ci) product; (H, W) planes walked as one row.
+// 64 output channels x 64 input channels per workgroup (sixteen accumulator tiles per wave), 128 positions
+// per staged tile; every wave does four steps of 16 MFMAs on 4 + 4 LDS reads per tile.
+using Gm1x1   = GwMfmaCfg<1, 1, 128, 1, 4, 4, 1, 1, 8, 1>;
+using Gm1x1s  = GwMfmaCfg<1, 1, 64, 2, 4, 4, 1, 1, 8, 1>;    // planes of <= 64 positions: two images
 
 template <class G>
 static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
@@ -272,15 +279,30 @@ static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
     p.tilesW = ceil_div(d.Wo, G::TW);
     p.ntiles = ceil_div(d.N, G::NIMG) * p.tilesH * p.tilesW;
     p.gy = ceil_div(d.Co, G::COB);
-    p.gz = ceil_div(d.Ci * 9, G::KB);
+    p.gz = ceil_div(d.Ci * G::KK, G::KB);
     // ~2048 waves over the chip (two per SIMD; a workgroup's staged tiles fill a good part of a CU's LDS)
     int want = ceil_div(2048 / (G::NTHREADS / 64), p.gy * p.gz);
     p.slots = want < p.ntiles ? want : p.ntiles;
     if (p.slots < 1) p.slots = 1;
 }
 
+// a stride-1 1x1 layer seen as images of one row of H*W positions
+static ConvDims mfma_one_row(const ConvDims &d) {
+    ConvDims f = d;
+    f.H = f.Ho = 1;
+    f.W = f.Wo = d.H * d.W;
+    return f;
+}
+
 GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     GradWMfmaPlan p{};
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 64) {
+        const ConvDims f = mfma_one_row(d);
+        p.variant = f.W > 64 ? 6 : 7;
+        if (p.variant == 6) plan_one<Gm1x1>(f, p);
+        else plan_one<Gm1x1s>(f, p);
+        return p;
+    }
     const bool ok = d.kh == 3 && d.kw == 3 && d.pad == 1;
     if (!ok) return p;
     if (d.stride == 1) p.variant = d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
@@ -327,6 +349,8 @@ int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sg
         case 3: return launch_one<GmW8>(gy, x, part, sgpart, d, p, s);
         case 4: return launch_one<GmW16S2>(gy, x, part, sgpart, d, p, s);
         case 5: return launch_one<GmW8S2>(gy, x, part, sgpart, d, p, s);
+        case 6: return launch_one<Gm1x1>(gy, x, part, sgpart, mfma_one_row(d), p, s);
+        case 7: return launch_one<Gm1x1s>(gy, x, part, sgpart, mfma_one_row(d), p, s);
         default: return ADDER_ERR_BAD_SHAPE;
     }
 }
