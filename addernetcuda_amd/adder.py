@@ -80,10 +80,13 @@ class _adder_nchw(Function):
         if stats is None:   # no statistics epilogue for this shape: an empty tensor stands for "none"
             stats = torch.empty(0, device=dev, dtype=torch.float64)
         ctx.mark_non_differentiable(stats)
+        ctx.set_materialize_grads(False)   # no zero-filled "gradient" of stats on the way back
         return out, stats
 
     @staticmethod
     def backward(ctx, grad_out, *unused):
+        if grad_out is None:
+            return None, None, None, None, None, None
         X, W = ctx.saved_tensors
         grad_out = grad_out.contiguous()
         require_gpu_f32(grad_out, "grad_output")

@@ -84,7 +84,11 @@ class ResNet(nn.Module):
     def forward(self, x):
         x = self.bn1(self.conv1(x))
         x = self.layer3(self.layer2(self.layer1(x)))
-        x = self.bn2(self.fc(self.avgpool(x)))
+        if x.shape[2] == 8 and x.shape[3] == 8:
+            x = x.mean(dim=(2, 3), keepdim=True)   # AvgPool2d(8) of an 8x8 map, as one reduction kernel
+        else:
+            x = self.avgpool(x)
+        x = self.bn2(self.fc(x))
         return x.view(x.size(0), -1)
 
 

@@ -123,7 +123,7 @@ def run(args):
     net = resnet20(eta=args.eta).to(dev)
     if args.resume:
         net.load_state_dict(torch.load(args.resume, map_location=dev, weights_only=True))
-    opt = torch.optim.SGD(net.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4)
+    opt = torch.optim.SGD(net.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4, fused=True)
     os.makedirs(args.output_dir, exist_ok=True)
     gen = torch.Generator(device=dev).manual_seed(args.seed)
     best, history = 0.0, []
