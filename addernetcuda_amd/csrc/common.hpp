@@ -18,6 +18,10 @@ __device__ __forceinline__ uniform_f32_ptr as_uniform(const float *p) {
     return (uniform_f32_ptr)p;
 }
 
+// Clamp to [0, 1]: the compiler folds it into the clamp output modifier of the instruction that
+// produces v, so it costs no instruction of its own.
+__device__ __forceinline__ float sat01(float v) { return __builtin_amdgcn_fmed3f(v, 0.f, 1.f); }
+
 // hardtanh of adder.cu:17 (x<-1 -> -1, x<=1 -> x, else 1) is one v_med3_f32.
 __device__ __forceinline__ float hardtanh(float v) {
     return __builtin_amdgcn_fmed3f(v, -1.0f, 1.0f);

@@ -152,13 +152,18 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
     const size_t plane = (size_t)H * W;
     const size_t xoff = (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
     const int valid = L.ok ? W - L.wo0 * S : 0;   // only read when !VEC
-    float xr[TM][TN], acc[TM][TN], tot[TM][TN];   // two-level sum: acc holds at most 64 output channels
+    // clamp(w - x, -1, 1) = 2 * sat(0.5 w + cr) - 1 with cr = 0.5 - 0.5 x and sat the [0, 1] clamp modifier of
+    // v_fma_f32: two instructions per term; sg collects the gy sum that the "- 1" multiplies
+    float cr[TM][TN], acc[TM][TN], tot[TM][TN];   // two-level sum: acc holds at most 64 output channels
+    float sg[TN], sgt[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) sg[t] = sgt[t] = 0.f;
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const float4 v = ld4<VEC>(x + xoff + (size_t)min(ci0 + m, Ci - 1) * plane, valid);
         const float xs[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int t = 0; t < TN; ++t) { xr[m][t] = xs[t * S]; acc[m][t] = tot[m][t] = 0.f; }
+        for (int t = 0; t < TN; ++t) { cr[m][t] = fmaf(-0.5f, xs[t * S], 0.5f); acc[m][t] = tot[m][t] = 0.f; }
     }
     const size_t gplane = (size_t)Ho * Wo;
     const float *gp = gy + (size_t)L.n * Co * gplane + (size_t)L.ho * Wo + L.wo0;
@@ -175,15 +180,23 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
         for (int m = 0; m < TM; ++m) {
             const float wv = wc[co * Ci + min(ci0 + m, Ci - 1)];
 #pragma unroll
-            for (int t = 0; t < TN; ++t) acc[m][t] = fmaf(hardtanh(wv - xr[m][t]), g[t], acc[m][t]);
+            for (int t = 0; t < TN; ++t) acc[m][t] = fmaf(sat01(fmaf(wv, 0.5f, cr[m][t])), g[t], acc[m][t]);
         }
+#pragma unroll
+        for (int t = 0; t < TN; ++t) sg[t] += g[t];
         if ((co & 63) == 63 || co + 1 == Co) {
 #pragma unroll
             for (int m = 0; m < TM; ++m)
 #pragma unroll
                 for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+#pragma unroll
+            for (int t = 0; t < TN; ++t) { sgt[t] += sg[t]; sg[t] = 0.f; }
         }
     }
+#pragma unroll
+    for (int m = 0; m < TM; ++m)
+#pragma unroll
+        for (int t = 0; t < TN; ++t) tot[m][t] = fmaf(2.f, tot[m][t], -sgt[t]);
     if (L.ok) {
         const bool row2 = S == 2 && L.ho * 2 + 1 < H;  // the odd row below: never sampled by stride 2
 #pragma unroll

@@ -6,11 +6,21 @@
 // adder.cu:133-192 (CONV_INPUT), and the permute + F.fold (col2im) autograd
 // runs after them for adder.py:32-33.  hardtanh is adder.cu:17.
 //
-// Three fp32 VALU instructions per term: v_sub (SGPR weight - own x),
-// v_med3 (clamp), v_fma (times gy).  Lanes own input positions, so x and the
-// accumulators stay in registers for the whole kernel, weights are SGPR
-// operands, and the haloed gy tile is staged in LDS with zeros outside the
-// output so invalid taps vanish without predication.
+// The generic kernel spends three fp32 VALU instructions per term: v_sub (SGPR
+// weight - own x), v_med3 (clamp), v_fma (times gy).  The tiled kernels spend two:
+//   hardtanh(w - x) = 2 * sat(0.5 * w + (0.5 - 0.5 * x)) - 1,   sat = clamp to [0, 1],
+// and sat is the clamp output modifier of v_fma_f32, so with cr = 0.5 - 0.5 x kept per
+// own position the term is  v_fma_f32 d, s_w, 0.5, v_cr clamp ; v_fmac_f32 acc, d, g  and
+//   gx = 2 * sum d * g - sum g,
+// where the second sum (over the output channels and the taps a position met) does not
+// depend on the input channel: it is a box sum of the channel-summed gy tile, which the
+// workgroup collects once per chunk in LDS.  d lies in [0, 1], so the sums keep the
+// magnitude they have in the three-instruction form; 0.5 * w + cr is exact wherever
+// w - x is (small integers, the golden fixtures), and the rounding of cr is at most
+// one ulp of (|x| + 1) / 2 -- for terms that do not saturate, |x| <= |w| + 1.
+// Lanes own input positions, so cr and the accumulators stay in registers for the whole
+// kernel, weights are SGPR operands, and the haloed gy tile is staged in LDS with zeros
+// outside the output so invalid taps vanish without predication.
 #include "common.hpp"
 #include "tile3x3.hpp"
 
@@ -83,7 +93,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
 // In tile coordinates (row 0 = h0-1, column 0 = w0-1) that is row+2-i, t+2-j.
 // ---------------------------------------------------------------------------
 template <class C, bool VEC = true>
-__global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *__restrict__ gy,
+__global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const float *__restrict__ gy,
                                                                    const float *__restrict__ x,
                                                                    const float *__restrict__ w,
                                                                    float *__restrict__ gx, int N, int Ci,
@@ -118,18 +128,26 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
     const bool pos_ok = lane_ok && n < N && hi < H;
     const int nc = min(n, N - 1), hc = min(hi, H - 1);
 
-    // own x values and accumulators live in registers for the whole kernel
-    // (two-level sum: acc collects one chunk of output channels, tot the chunks)
-    float xr[TM][TN], acc[TM][TN], tot[TM][TN];
+    // cr = 0.5 - 0.5 x of the own positions and the accumulators live in registers for the whole
+    // kernel (two-level sum: acc collects one chunk of output channels, tot the chunks)
+    float cr[TM][TN], acc[TM][TN], tot[TM][TN];
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
         const float *src = x + (((size_t)nc * Ci + ci) * H + hc) * W;
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
-            xr[m][t] = src[min(wi0 + t, W - 1)];
+            cr[m][t] = fmaf(-0.5f, src[min(wi0 + t, W - 1)], 0.5f);
             acc[m][t] = tot[m][t] = 0.f;
         }
+    }
+    // per tile position, the sum of gy over all output channels (threads own plane elements)
+    constexpr int GN = C::NIMG * C::PLANE, GITER = ceil_div(GN, C::NTHREADS);
+    float *gplane = smem + 2 * C::BUF;
+#pragma unroll
+    for (int it = 0; it < GITER; ++it) {
+        const int e = threadIdx.x + it * C::NTHREADS;
+        if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
     }
 
     const int lane_off = img * C::CC * C::PLANE + row * C::PITCH + strip * TN;
@@ -174,8 +192,8 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
                 for (int idx = 0; idx < HM * KK * TN; ++idx) {
                     const int t = idx % TN, j = (idx / TN) % KS, i = (idx / TN / KS) % KS, mm = idx / TN / KK;
                     const int m = h * HM + mm;
-                    acc[m][t] = fmaf(hardtanh(wv[wb][mm * KK + i * KS + j] - xr[m][t]), gr[cur][KS - 1 - i][t + KS - 1 - j],
-                                     acc[m][t]);
+                    acc[m][t] = fmaf(sat01(fmaf(wv[wb][mm * KK + i * KS + j], 0.5f, cr[m][t])),
+                                     gr[cur][KS - 1 - i][t + KS - 1 - j], acc[m][t]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
                         if (h + 1 < NU) {
@@ -207,8 +225,41 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s1_kernel(const float *
 #pragma unroll
             for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
 
+        // channel sum of this chunk (planes past Co were staged as zeros)
+#pragma unroll
+        for (int it = 0; it < GITER; ++it) {
+            const int e = threadIdx.x + it * C::NTHREADS;
+            if (GN % C::NTHREADS == 0 || e < GN) {
+                const float *src = smem + (c & 1) * C::BUF + (e / C::PLANE) * C::CC * C::PLANE + e % C::PLANE;
+                float sum = 0.f;
+#pragma unroll
+                for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
+                gplane[e] += sum;   // always the same thread for a given e: no race
+            }
+        }
+
         if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
         __syncthreads();
+    }
+
+    // sum over (co, taps) of the gy values a position met = box sum of the channel-sum plane
+    // (the loop's last barrier has made every thread's part of the plane visible)
+    {
+        float gs[KS][TN + KS - 1];
+#pragma unroll
+        for (int i = 0; i < KS; ++i)
+            lds_read_strip<TN + KS - 1, C::STRIP_ALIGN>(gplane + img * C::PLANE + row * C::PITCH + strip * TN + i * C::PITCH,
+                                                        gs[i]);
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            float sg = 0.f;
+#pragma unroll
+            for (int i = 0; i < KS; ++i)
+#pragma unroll
+                for (int j = 0; j < KS; ++j) sg += gs[i][t + j];
+#pragma unroll
+            for (int m = 0; m < TM; ++m) tot[m][t] = fmaf(2.f, tot[m][t], -sg);
+        }
     }
 
     if (pos_ok) {
@@ -240,13 +291,14 @@ static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     static bool attr_set = false;
-    if (!attr_set && C::LDS_BYTES > 48 * 1024) {
+    constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
+    if (!attr_set && LDS_BYTES > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C, VEC>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
+    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW);
     return check_launch();
 }
@@ -317,7 +369,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     const int n = n0 + img, hi0 = h0 + 2 * brow, wi0 = w0 + bcol * TNW;
     const int nc = min(n, N - 1);
 
-    float xr[TM][2][TNW], acc[TM][2][TNW], tot[TM][2][TNW];
+    float cr[TM][2][TNW], acc[TM][2][TNW], tot[TM][2][TNW];   // cr = 0.5 - 0.5 x, as in the stride-1 kernel
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
@@ -326,10 +378,17 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
             const float *src = x + (((size_t)nc * Ci + ci) * H + min(hi0 + rp, H - 1)) * W;
 #pragma unroll
             for (int t = 0; t < TNW; ++t) {
-                xr[m][rp][t] = src[min(wi0 + t, W - 1)];
+                cr[m][rp][t] = fmaf(-0.5f, src[min(wi0 + t, W - 1)], 0.5f);
                 acc[m][rp][t] = tot[m][rp][t] = 0.f;
             }
         }
+    }
+    constexpr int GN = C::NIMG * C::PLANE, GITER = ceil_div(GN, C::NTHREADS);
+    float *gplane = smem + 2 * C::BUF;   // per tile position, the sum of gy over all output channels
+#pragma unroll
+    for (int it = 0; it < GITER; ++it) {
+        const int e = threadIdx.x + it * C::NTHREADS;
+        if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
     }
 
     const int lane_off = img * C::CC * C::PLANE + brow * C::PITCH + bcol * (TNW / 2);
@@ -371,7 +430,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
                     const int cp = idx % (TNW / 2), bb = (idx / (TNW / 2)) % 3, a = (idx / (TNW / 2) / 3) % 3,
                               mm = idx / TERMS;
                     const int m = h * HM + mm, t = 2 * cp + RP[bb];
-                    acc[m][RP[a]][t] = fmaf(hardtanh(wv[h & 1][mm * 9 + RI[a] * 3 + RI[bb]] - xr[m][RP[a]][t]),
+                    acc[m][RP[a]][t] = fmaf(sat01(fmaf(wv[h & 1][mm * 9 + RI[a] * 3 + RI[bb]], 0.5f, cr[m][RP[a]][t])),
                                             gr[cur][RG[a]][cp + RG[bb]], acc[m][RP[a]][t]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
@@ -405,8 +464,46 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 #pragma unroll
                 for (int t = 0; t < TNW; ++t) { tot[m][rp][t] += acc[m][rp][t]; acc[m][rp][t] = 0.f; }
 
+        // channel sum of this chunk (planes past Co were staged as zeros)
+#pragma unroll
+        for (int it = 0; it < GITER; ++it) {
+            const int e = threadIdx.x + it * C::NTHREADS;
+            if (GN % C::NTHREADS == 0 || e < GN) {
+                const float *src = smem + (c & 1) * C::BUF + (e / C::PLANE) * C::CC * C::PLANE + e % C::PLANE;
+                float sum = 0.f;
+#pragma unroll
+                for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
+                gplane[e] += sum;   // always the same thread for a given e: no race
+            }
+        }
+
         if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
         __syncthreads();
+    }
+
+    // clamp = 2 * sat - 1: take off the sum of the gy values each position met (same taps as above)
+    {
+        constexpr int RP[3] = {0, 1, 1}, RG[3] = {0, 1, 0};
+        float gs[2][GSTRIP], sg[2][TNW];
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+            lds_read_strip<GSTRIP, 1>(gplane + img * C::PLANE + (brow + r) * C::PITCH + bcol * (TNW / 2), gs[r]);
+#pragma unroll
+        for (int rp = 0; rp < 2; ++rp)
+#pragma unroll
+            for (int t = 0; t < TNW; ++t) sg[rp][t] = 0.f;
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+#pragma unroll
+            for (int bb = 0; bb < 3; ++bb)
+#pragma unroll
+                for (int cp = 0; cp < TNW / 2; ++cp) sg[RP[a]][2 * cp + RP[bb]] += gs[RG[a]][cp + RG[bb]];
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+#pragma unroll
+            for (int rp = 0; rp < 2; ++rp)
+#pragma unroll
+                for (int t = 0; t < TNW; ++t) tot[m][rp][t] = fmaf(2.f, tot[m][rp][t], -sg[rp][t]);
     }
 
     if (lane_ok && n < N) {
@@ -440,8 +537,9 @@ static int launch_grad_x_3x3s2_v(const float *gy, const float *x, const float *w
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    static_assert(C::LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
-    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), C::LDS_BYTES, s,
+    constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
+    static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
+    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
     return check_launch();
 }
