@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
 //   gx[hi,wi] += hardtanh(w[co,ci,i,j] - x[hi,wi]) * gy[hi+1-i, wi+1-j]
 // In tile coordinates (row 0 = h0-1, column 0 = w0-1) that is row+2-i, t+2-j.
 // ---------------------------------------------------------------------------
-template <class C, bool VEC = true>
+template <class C, bool VEC = true, bool SAT = true>
 __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const float *__restrict__ gy,
                                                                    const float *__restrict__ x,
                                                                    const float *__restrict__ w,
@@ -128,8 +128,9 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
     const bool pos_ok = lane_ok && n < N && hi < H;
     const int nc = min(n, N - 1), hc = min(hi, H - 1);
 
-    // cr = 0.5 - 0.5 x of the own positions and the accumulators live in registers for the whole
-    // kernel (two-level sum: acc collects one chunk of output channels, tot the chunks)
+    // cr = 0.5 - 0.5 x of the own positions (x itself in the three-instruction form, SAT = false) and the
+    // accumulators live in registers for the whole kernel (two-level sum: acc collects one chunk of
+    // output channels, tot the chunks)
     float cr[TM][TN], acc[TM][TN], tot[TM][TN];
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
@@ -137,17 +138,20 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
         const float *src = x + (((size_t)nc * Ci + ci) * H + hc) * W;
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
-            cr[m][t] = fmaf(-0.5f, src[min(wi0 + t, W - 1)], 0.5f);
+            const float xv = src[min(wi0 + t, W - 1)];
+            cr[m][t] = SAT ? fmaf(-0.5f, xv, 0.5f) : xv;
             acc[m][t] = tot[m][t] = 0.f;
         }
     }
     // per tile position, the sum of gy over all output channels (threads own plane elements)
     constexpr int GN = C::NIMG * C::PLANE, GITER = ceil_div(GN, C::NTHREADS);
     float *gplane = smem + 2 * C::BUF;
+    if constexpr (SAT) {
 #pragma unroll
-    for (int it = 0; it < GITER; ++it) {
-        const int e = threadIdx.x + it * C::NTHREADS;
-        if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
+        for (int it = 0; it < GITER; ++it) {
+            const int e = threadIdx.x + it * C::NTHREADS;
+            if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
+        }
     }
 
     const int lane_off = img * C::CC * C::PLANE + row * C::PITCH + strip * TN;
@@ -192,8 +196,9 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
                 for (int idx = 0; idx < HM * KK * TN; ++idx) {
                     const int t = idx % TN, j = (idx / TN) % KS, i = (idx / TN / KS) % KS, mm = idx / TN / KK;
                     const int m = h * HM + mm;
-                    acc[m][t] = fmaf(sat01(fmaf(wv[wb][mm * KK + i * KS + j], 0.5f, cr[m][t])),
-                                     gr[cur][KS - 1 - i][t + KS - 1 - j], acc[m][t]);
+                    const float wgt = wv[wb][mm * KK + i * KS + j];
+                    const float d = SAT ? sat01(fmaf(wgt, 0.5f, cr[m][t])) : hardtanh(wgt - cr[m][t]);
+                    acc[m][t] = fmaf(d, gr[cur][KS - 1 - i][t + KS - 1 - j], acc[m][t]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
                         if (h + 1 < NU) {
@@ -226,15 +231,17 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
             for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
 
         // channel sum of this chunk (planes past Co were staged as zeros)
+        if constexpr (SAT) {
 #pragma unroll
-        for (int it = 0; it < GITER; ++it) {
-            const int e = threadIdx.x + it * C::NTHREADS;
-            if (GN % C::NTHREADS == 0 || e < GN) {
-                const float *src = smem + (c & 1) * C::BUF + (e / C::PLANE) * C::CC * C::PLANE + e % C::PLANE;
-                float sum = 0.f;
+            for (int it = 0; it < GITER; ++it) {
+                const int e = threadIdx.x + it * C::NTHREADS;
+                if (GN % C::NTHREADS == 0 || e < GN) {
+                    const float *src = smem + (c & 1) * C::BUF + (e / C::PLANE) * C::CC * C::PLANE + e % C::PLANE;
+                    float sum = 0.f;
 #pragma unroll
-                for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
-                gplane[e] += sum;   // always the same thread for a given e: no race
+                    for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
+                    gplane[e] += sum;   // always the same thread for a given e: no race
+                }
             }
         }
 
@@ -244,7 +251,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 
     // sum over (co, taps) of the gy values a position met = box sum of the channel-sum plane
     // (the loop's last barrier has made every thread's part of the plane visible)
-    {
+    if constexpr (SAT) {
         float gs[KS][TN + KS - 1];
 #pragma unroll
         for (int i = 0; i < KS; ++i)
@@ -283,7 +290,13 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
     }
 }
 
-template <class C, bool VEC>
+// The two-instruction form doubles a sum of products whose factors lie in [0, 1] and takes a second
+// sum off it, which about triples the rounding error of the three-instruction form (measured against
+// fp64: 0.2 of the parity tolerance |err| <= 1e-4 + 1e-5 |gx| at 144 terms per output, 0.4 at 576, 0.9
+// at 4608).  Layers with more terms per output than this keep the three-instruction form.
+static constexpr int kSatMaxTerms = 2304;
+
+template <class C, bool VEC, bool SAT>
 static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w, float *gx,
                                const ConvDims &d, hipStream_t s) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
@@ -293,12 +306,12 @@ static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w
     static bool attr_set = false;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     if (!attr_set && LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C, VEC>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C, VEC, SAT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
+    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW);
     return check_launch();
 }
@@ -307,8 +320,14 @@ template <class C>
 static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, float *gx,
                                const ConvDims &d, hipStream_t s) {
     // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
-    if (d.W % 4 == 0) return launch_grad_x_3x3s1_v<C, true>(gy, x, w, gx, d, s);
-    return launch_grad_x_3x3s1_v<C, false>(gy, x, w, gx, d, s);
+    const bool vec = d.W % 4 == 0;
+    if constexpr (C::KS == 3) {   // (a single tap never has that many terms per output)
+        if (d.Co * C::KK > kSatMaxTerms)
+            return vec ? launch_grad_x_3x3s1_v<C, true, false>(gy, x, w, gx, d, s)
+                       : launch_grad_x_3x3s1_v<C, false, false>(gy, x, w, gx, d, s);
+    }
+    return vec ? launch_grad_x_3x3s1_v<C, true, true>(gy, x, w, gx, d, s)
+               : launch_grad_x_3x3s1_v<C, false, true>(gy, x, w, gx, d, s);
 }
 
 // ---------------------------------------------------------------------------
@@ -336,7 +355,7 @@ struct GradX3x3S2Cfg {
     static_assert(TNW % 2 == 0 && TH % 2 == 0, "lanes own 2 x 2 parity blocks");
 };
 
-template <class C, bool VEC = true>
+template <class C, bool VEC = true, bool SAT = true>
 __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *__restrict__ gy,
                                                                    const float *__restrict__ x,
                                                                    const float *__restrict__ w,
@@ -378,17 +397,20 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
             const float *src = x + (((size_t)nc * Ci + ci) * H + min(hi0 + rp, H - 1)) * W;
 #pragma unroll
             for (int t = 0; t < TNW; ++t) {
-                cr[m][rp][t] = fmaf(-0.5f, src[min(wi0 + t, W - 1)], 0.5f);
+                const float xv = src[min(wi0 + t, W - 1)];
+                cr[m][rp][t] = SAT ? fmaf(-0.5f, xv, 0.5f) : xv;
                 acc[m][rp][t] = tot[m][rp][t] = 0.f;
             }
         }
     }
     constexpr int GN = C::NIMG * C::PLANE, GITER = ceil_div(GN, C::NTHREADS);
     float *gplane = smem + 2 * C::BUF;   // per tile position, the sum of gy over all output channels
+    if constexpr (SAT) {
 #pragma unroll
-    for (int it = 0; it < GITER; ++it) {
-        const int e = threadIdx.x + it * C::NTHREADS;
-        if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
+        for (int it = 0; it < GITER; ++it) {
+            const int e = threadIdx.x + it * C::NTHREADS;
+            if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
+        }
     }
 
     const int lane_off = img * C::CC * C::PLANE + brow * C::PITCH + bcol * (TNW / 2);
@@ -430,8 +452,9 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
                     const int cp = idx % (TNW / 2), bb = (idx / (TNW / 2)) % 3, a = (idx / (TNW / 2) / 3) % 3,
                               mm = idx / TERMS;
                     const int m = h * HM + mm, t = 2 * cp + RP[bb];
-                    acc[m][RP[a]][t] = fmaf(sat01(fmaf(wv[h & 1][mm * 9 + RI[a] * 3 + RI[bb]], 0.5f, cr[m][RP[a]][t])),
-                                            gr[cur][RG[a]][cp + RG[bb]], acc[m][RP[a]][t]);
+                    const float wgt = wv[h & 1][mm * 9 + RI[a] * 3 + RI[bb]];
+                    const float d = SAT ? sat01(fmaf(wgt, 0.5f, cr[m][RP[a]][t])) : hardtanh(wgt - cr[m][RP[a]][t]);
+                    acc[m][RP[a]][t] = fmaf(d, gr[cur][RG[a]][cp + RG[bb]], acc[m][RP[a]][t]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
                         if (h + 1 < NU) {
@@ -465,15 +488,17 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
                 for (int t = 0; t < TNW; ++t) { tot[m][rp][t] += acc[m][rp][t]; acc[m][rp][t] = 0.f; }
 
         // channel sum of this chunk (planes past Co were staged as zeros)
+        if constexpr (SAT) {
 #pragma unroll
-        for (int it = 0; it < GITER; ++it) {
-            const int e = threadIdx.x + it * C::NTHREADS;
-            if (GN % C::NTHREADS == 0 || e < GN) {
-                const float *src = smem + (c & 1) * C::BUF + (e / C::PLANE) * C::CC * C::PLANE + e % C::PLANE;
-                float sum = 0.f;
+            for (int it = 0; it < GITER; ++it) {
+                const int e = threadIdx.x + it * C::NTHREADS;
+                if (GN % C::NTHREADS == 0 || e < GN) {
+                    const float *src = smem + (c & 1) * C::BUF + (e / C::PLANE) * C::CC * C::PLANE + e % C::PLANE;
+                    float sum = 0.f;
 #pragma unroll
-                for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
-                gplane[e] += sum;   // always the same thread for a given e: no race
+                    for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
+                    gplane[e] += sum;   // always the same thread for a given e: no race
+                }
             }
         }
 
@@ -482,7 +507,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     }
 
     // clamp = 2 * sat - 1: take off the sum of the gy values each position met (same taps as above)
-    {
+    if constexpr (SAT) {
         constexpr int RP[3] = {0, 1, 1}, RG[3] = {0, 1, 0};
         float gs[2][GSTRIP], sg[2][TNW];
 #pragma unroll
@@ -530,7 +555,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     }
 }
 
-template <class C, bool VEC>
+template <class C, bool VEC, bool SAT>
 static int launch_grad_x_3x3s2_v(const float *gy, const float *x, const float *w, float *gx,
                                const ConvDims &d, hipStream_t s) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
@@ -539,7 +564,7 @@ static int launch_grad_x_3x3s2_v(const float *gy, const float *x, const float *w
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
-    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
+    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
     return check_launch();
 }
@@ -548,8 +573,12 @@ template <class C>
 static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, float *gx,
                                const ConvDims &d, hipStream_t s) {
     // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
-    if (d.Wo % 4 == 0) return launch_grad_x_3x3s2_v<C, true>(gy, x, w, gx, d, s);
-    return launch_grad_x_3x3s2_v<C, false>(gy, x, w, gx, d, s);
+    const bool vec = d.Wo % 4 == 0;
+    if (d.Co * 4 > kSatMaxTerms)   // an input position meets at most four of the nine taps per output channel
+        return vec ? launch_grad_x_3x3s2_v<C, true, false>(gy, x, w, gx, d, s)
+                   : launch_grad_x_3x3s2_v<C, false, false>(gy, x, w, gx, d, s);
+    return vec ? launch_grad_x_3x3s2_v<C, true, true>(gy, x, w, gx, d, s)
+               : launch_grad_x_3x3s2_v<C, false, true>(gy, x, w, gx, d, s);
 }
 
 //                              TNW BPR TH NIMG TM CIW CC

@@ -66,7 +66,7 @@ RESNET50_LAYERS = [
 LAYER_SETS = {"resnet20": (BATCH, RESNET20_LAYERS), "vgg_small": (128, VGG_SMALL_LAYERS),
               "resnet50": (64, RESNET50_LAYERS)}
 # flops per (co, k, position) term and the fewest fp32 VALU instructions that implement it
-OPS = {"fwd": (2, 2), "grad_x": (4, 3), "grad_w": (3, 1)}
+OPS = {"fwd": (2, 2), "grad_x": (4, 2), "grad_w": (3, 1)}
 
 
 def event_time(fn, warmup, iters):
@@ -149,9 +149,10 @@ def dominant_kernel(dev, steps):
         "valu_issue_util": round(OPS["grad_x"][1] * E / t / PEAK_VALU_ISSUE, 4),
         "issue_probe_T_lane_instr_per_s": issue_probe(),
         "note": "fp32 VALU-bound (|a-b| accumulation has no FMA/MFMA form). The 157.3 TFLOP/s peak needs an FMA "
-                "in each of the two vector issue slots a SIMD has per 4 cycles; this op spends 3 instructions on "
-                "4 flop, so 2/3 of the peak (104.9 TFLOP/s) is its ceiling. valu_issue_util is the share of the "
-                "two-slot issue rate; the probe table is that rate measured with a bare instruction stream.",
+                "in each of the two vector issue slots a SIMD has per 4 cycles; this op spends 2 instructions "
+                "(v_fma with the clamp modifier, v_fmac) on the 4 flop of a term (sub, clamp, mul, add), so the "
+                "peak itself is its ceiling. valu_issue_util is the share of the two-slot issue rate taken by "
+                "those 2 instructions per term; the probe table is that rate measured with a bare instruction stream.",
     }
 
 
@@ -168,7 +169,7 @@ def issue_probe():
     table = {}
     for line in out.splitlines():
         f = line.split()
-        if len(f) == 3 and f[0] in ("fwd_pair", "gradx_triple", "sgpr_only"):
+        if len(f) == 3 and f[0] in ("fwd_pair", "gradx_pair", "sgpr_only"):
             table.setdefault(f[0], {})[f"{f[1]}_waves_per_simd"] = round(float(f[2]) / 1e12, 2)
     return table or None
 

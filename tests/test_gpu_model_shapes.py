@@ -24,6 +24,7 @@ SHAPES = [
     (2, 2048, 7, 7, 512, 1, 1, 0),     # K = 2048
     (3, 24, 32, 32, 48, 1, 1, 0),      # DenseNet-BC bottleneck 1x1 (densenet.py:12-14)
     (3, 48, 32, 32, 12, 3, 1, 1),      # DenseNet-BC growth conv, Co = 12
+    (1, 32, 16, 16, 640, 3, 2, 1),     # strided 3x3 with > 2304 terms per input position (three-instruction grad_X form)
 ]
 
 
