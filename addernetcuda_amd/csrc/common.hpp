@@ -18,6 +18,18 @@ __device__ __forceinline__ uniform_f32_ptr as_uniform(const float *p) {
     return (uniform_f32_ptr)p;
 }
 
+// Touch `rows` runs of `len` floats, `pitch` floats apart, with one vector load per 128-byte line, so that
+// the scalar weight loads of a kernel's main loop -- which run only one unit ahead and would otherwise wait
+// for HBM on every new line, all workgroups at the same place -- find their lines in L2.
+__device__ __forceinline__ void l2_warm(const float *p, int rows, int pitch, int len) {
+    const int lines = (len + 31) / 32;
+    for (int i = threadIdx.x; i < rows * lines; i += blockDim.x) {
+        const int r = i / lines, l = i - r * lines;
+        const float v = p[(size_t)r * pitch + min(l * 32, len - 1)];
+        asm volatile("" ::"v"(v));
+    }
+}
+
 // Clamp to [0, 1]: the compiler folds it into the clamp output modifier of the instruction that
 // produces v, so it costs no instruction of its own.
 __device__ __forceinline__ float sat01(float v) { return __builtin_amdgcn_fmed3f(v, 0.f, 1.f); }

@@ -131,6 +131,10 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
 
     TileStage<typename C::Patch> st;
     tile_fetch<typename C::Patch, VEC>(st, x, 0, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W);
+    {   // this workgroup's output channels: one contiguous run of weights
+        const int co_blk = blockIdx.y * C::COW * TM;
+        l2_warm(w + (size_t)co_blk * K, 1, 0, min(C::COW * TM, Co - co_blk) * K);
+    }
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 

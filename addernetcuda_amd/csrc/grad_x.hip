@@ -159,6 +159,10 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 
     TileStage<typename C::Patch> st;
     tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, h0 - C::PAD, w0, H, W);
+    {   // this workgroup's input channels: one run of weights per output channel
+        const int ci_blk = min((int)blockIdx.y * C::COW * TM, Ci - TM);
+        l2_warm(w + ci_blk * KK, Co, K, min(C::COW * TM, Ci - ci_blk) * KK);
+    }
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 
@@ -419,6 +423,10 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 
     TileStage<typename C::Patch> st;
     tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
+    {   // this workgroup's input channels: one run of weights per output channel
+        const int ci_blk = min((int)blockIdx.y * C::CIW * TM, Ci - TM);
+        l2_warm(w + ci_blk * 9, Co, K, min(C::CIW * TM, Ci - ci_blk) * 9);
+    }
     tile_commit<typename C::Patch>(st, smem);
     __syncthreads();
 

@@ -28,6 +28,7 @@ struct PatchCfg {
     static constexpr int NUV = NIMG * CC * ROWS * (ICOLS / 4);
     static constexpr int VITER = ceil_div(NUV, NTHREADS);
     static constexpr int NSIDES = LHALO + RHALO;
+    static constexpr int SIDE_DIV = NSIDES ? NSIDES : 1;   // divisor of the halo loops (which are empty without a halo)
     static constexpr int NUH = NIMG * CC * ROWS * NSIDES;
     static constexpr int HITER = NSIDES ? ceil_div(NUH, NTHREADS) : 0;
     static_assert(ICOLS % 4 == 0, "interior must cover whole float4 groups of the source");
@@ -78,8 +79,8 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
 #pragma unroll
     for (int it = 0; it < P::HITER; ++it) {
         const int u = tid + it * P::NTHREADS;
-        const int side = P::LHALO ? u % P::NSIDES : 1;  // 0 = left, 1 = right
-        const int rest = u / P::NSIDES;
+        const int side = P::LHALO ? u % P::SIDE_DIV : 1;  // 0 = left, 1 = right
+        const int rest = u / P::SIDE_DIV;
         const int r = rest % P::ROWS;
         const int cc = rest / P::ROWS % P::CC;
         const int img = rest / P::ROWS / P::CC;
@@ -112,8 +113,8 @@ __device__ __forceinline__ void tile_commit(const TileStage<P> &st, float *buf) 
     for (int it = 0; it < P::HITER; ++it) {
         const int u = tid + it * P::NTHREADS;
         if (P::NUH % P::NTHREADS == 0 || u < P::NUH) {
-            const int side = P::LHALO ? u % P::NSIDES : 1;
-            const int rest = u / P::NSIDES;
+            const int side = P::LHALO ? u % P::SIDE_DIV : 1;
+            const int rest = u / P::SIDE_DIV;
             buf[rest * P::PITCH + (side ? P::ICOL0 + P::ICOLS : P::LPAD)] = st.h[it];
         }
     }
