@@ -88,6 +88,8 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
 #pragma unroll
         for (int t = 0; t < TN; ++t) acc[m][t] = tot[m][t] = 0.f;
 
+    l2_warm(w + (size_t)co0 * Ci, 1, 0, min(TM, Co - co0) * Ci);   // the scalar weight loads below run one step ahead
+
     const size_t plane = (size_t)H * W;
     const float *xp = x + (size_t)L.n * Ci * plane + (size_t)(L.ho * S) * W + L.wo0 * S;
     const int valid = L.ok ? W - L.wo0 * S : 0;   // only read when !VEC
@@ -165,26 +167,43 @@ __global__ __launch_bounds__(256) void grad_x_1x1_kernel(const float *__restrict
 #pragma unroll
         for (int t = 0; t < TN; ++t) { cr[m][t] = fmaf(-0.5f, xs[t * S], 0.5f); acc[m][t] = tot[m][t] = 0.f; }
     }
+    l2_warm(w + min(ci0, Ci - 1), Co, Ci, min(TM, Ci - ci0));   // one run of TM weights per output channel
     const size_t gplane = (size_t)Ho * Wo;
     const float *gp = gy + (size_t)L.n * Co * gplane + (size_t)L.ho * Wo + L.wo0;
-    for (int co = 0; co < Co; ++co) {
-        float g[TN];
-        if constexpr (TN == 4) {
-            const float4 v = ld4<VEC>(gp + (size_t)co * gplane, valid);
-            g[0] = v.x; g[1] = v.y; g[2] = v.z; g[3] = v.w;
-        } else {
-            const float2 v = ld2<VEC>(gp + (size_t)co * gplane, L.ok ? Wo - L.wo0 : 0);
-            g[0] = v.x; g[1] = v.y;
+    // eight output channels per round: their gy loads are issued together (little arithmetic per load, so
+    // the loop is bound by how many loads are in flight); channels past Co load nothing and count as gy = 0
+    constexpr int UN = 8;
+    for (int co0 = 0; co0 < Co; co0 += UN) {
+        float g[UN][TN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const bool live = co0 + u < Co;
+            const float *src = gp + (size_t)min(co0 + u, Co - 1) * gplane;
+            if constexpr (TN == 4) {
+                const float4 v = ld4<VEC>(src, live ? valid : 0);
+                g[u][0] = v.x; g[u][1] = v.y; g[u][2] = v.z; g[u][3] = v.w;
+            } else {
+                const float2 v = ld2<VEC>(src, live && L.ok ? Wo - L.wo0 : 0);
+                g[u][0] = v.x; g[u][1] = v.y;
+            }
+            if (VEC && !live) {
+#pragma unroll
+                for (int t = 0; t < TN; ++t) g[u][t] = 0.f;
+            }
         }
 #pragma unroll
-        for (int m = 0; m < TM; ++m) {
-            const float wv = wc[co * Ci + min(ci0 + m, Ci - 1)];
+        for (int u = 0; u < UN; ++u) {
+            const int co = min(co0 + u, Co - 1);
 #pragma unroll
-            for (int t = 0; t < TN; ++t) acc[m][t] = fmaf(sat01(fmaf(wv, 0.5f, cr[m][t])), g[t], acc[m][t]);
+            for (int m = 0; m < TM; ++m) {
+                const float wv = wc[co * Ci + min(ci0 + m, Ci - 1)];
+#pragma unroll
+                for (int t = 0; t < TN; ++t) acc[m][t] = fmaf(sat01(fmaf(wv, 0.5f, cr[m][t])), g[u][t], acc[m][t]);
+            }
+#pragma unroll
+            for (int t = 0; t < TN; ++t) sg[t] += g[u][t];
         }
-#pragma unroll
-        for (int t = 0; t < TN; ++t) sg[t] += g[t];
-        if ((co & 63) == 63 || co + 1 == Co) {
+        if ((co0 & 63) == 64 - UN || co0 + UN >= Co) {
 #pragma unroll
             for (int m = 0; m < TM; ++m)
 #pragma unroll

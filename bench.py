@@ -35,7 +35,7 @@ BATCH = 256
 ETA = 0.1
 # HBM bytes per launch of the dominant kernel, from the rocprofv3 counter passes kept under profiles/
 # (34.9 MB fetched + 16.8 MB written; cannot be read without the profiler attached)
-DOMINANT_TRAFFIC_BYTES = 51.7e6
+DOMINANT_TRAFFIC_BYTES = 51.6e6
 
 # distinct adder-layer shapes of ResNet-20 at 32x32 input: (count, Ci, H, W, Co, k, stride, pad)
 RESNET20_LAYERS = [
