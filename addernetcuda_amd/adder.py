@@ -108,17 +108,7 @@ def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
     if W.size(2) != W.size(3):
         # the reference passes only h_filter to unfold (adder.py:32): kernels are square
         raise RuntimeError("adder2d_function expects a square kernel")
-    X, stride = _subsample_1x1(X, W, stride, padding)
     return _adder_nchw.apply(X, W, int(stride), int(padding), eta)
-
-
-def _subsample_1x1(X, W, stride, padding):
-    """A 1x1 layer with stride s and no padding only ever reads every s-th row and column of its input, so it
-    is the stride-1 layer on that subsampled input (autograd scatters the input gradient back into zeros).
-    With many channels this is worth the copy: the stride-1 1x1 layers have LDS-tiled kernels."""
-    if W.size(2) == 1 and int(padding) == 0 and int(stride) > 1 and W.size(1) >= 64:
-        return X[:, :, ::int(stride), ::int(stride)].contiguous(), 1
-    return X, stride
 
 
 def adder2d_function_with_stats(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
@@ -126,7 +116,6 @@ def adder2d_function_with_stats(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
     (Co, slots, 2) for ``BatchNormAct2d(..., stats=)``, or None where the kernel has no such epilogue."""
     if W.size(2) != W.size(3):
         raise RuntimeError("adder2d_function expects a square kernel")
-    X, stride = _subsample_1x1(X, W, stride, padding)
     out, stats = _adder_nchw.apply(X, W, int(stride), int(padding), eta, True)
     return out, (stats if stats.numel() else None)
 

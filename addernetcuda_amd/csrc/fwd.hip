@@ -84,13 +84,13 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 // input channels.  Column 0 of a row is input column w0*S-1, so a lane's strip
 // starts at column strip*TN*S, which is 16-byte aligned when TN*S is a multiple of 4.
 // ---------------------------------------------------------------------------
-template <class C, bool VEC = true>
+template <class C, bool VEC = true, bool SUB = false>
 __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__restrict__ x,
                                                                 const float *__restrict__ w,
                                                                 float *__restrict__ y,
                                                                 double *__restrict__ stats, int N, int Ci,
                                                                 int H, int W, int Co, int Ho, int Wo,
-                                                                int tilesH, int tilesW) {
+                                                                int tilesH, int tilesW, const Subsample sub) {
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, S = C::S, STRIP = C::STRIP, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
 
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     const int nchunks = ceil_div(Ci, C::CC);
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch, VEC>(st, x, 0, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W);
+    tile_fetch<typename C::Patch, VEC, SUB>(st, x, 0, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W, sub);
     {   // this workgroup's output channels: one contiguous run of weights
         const int co_blk = blockIdx.y * C::COW * TM;
         l2_warm(w + (size_t)co_blk * K, 1, 0, min(C::COW * TM, Co - co_blk) * K);
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
 
     for (int c = 0; c < nchunks; ++c) {
         const int ci0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC, SUB>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W, sub);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Ci - ci0);
@@ -261,22 +261,22 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     }
 }
 
-template <class C, bool VEC>
+template <class C, bool VEC, bool SUB = false>
 static int launch_fwd_3x3_v(const float *x, const float *w, float *y, double *stats, const ConvDims &d,
-                            hipStream_t s) {
+                            hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
     const int tilesH = ceil_div(d.Ho, C::TH), tilesW = ceil_div(d.Wo, C::TW);
     const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gy = ceil_div(d.Co, C::TM * C::COW);
     if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     static bool attr_set = false;
     if (!attr_set && C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C, VEC>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C, VEC, SUB>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
-                       stats, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
+    hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC, SUB>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
+                       stats, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, sub);
     return check_launch();
 }
 
@@ -313,24 +313,28 @@ using Fwd1x1   = Tile3x3Cfg<4, 64, 1, 1, 4, 8, 16, 8, 1, 1>;   // 256 positions 
 using Fwd1x1s  = Tile3x3Cfg<4, 16, 1, 4, 4, 8, 16, 8, 1, 1>;   // planes of <= 64 positions: four images
 
 // which tiled kernel serves these dimensions (0 = none): 1..3 3x3 stride 1 by output width, 4..5 3x3 stride 2,
-// 6..7 1x1 stride 1 by plane size
+// 6..7 1x1 stride 1 by plane size, 8..9 1x1 with a stride (the sampled positions walked like a stride-1 plane)
 static int fwd_tiled_variant(const ConvDims &d) {
     // (below 64 input channels the plain 1x1 kernel of conv1x1.hip is as fast or faster)
-    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci % Fwd1x1::CQ == 0 && d.Ci >= 64)
-        return d.H * d.W > 64 ? 6 : 7;
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.Ci % Fwd1x1::CQ == 0 && d.Ci >= 64) {
+        if (d.stride == 1) return d.H * d.W > 64 ? 6 : 7;
+        return d.Ho * d.Wo > 64 ? 8 : 9;
+    }
     if (d.kh != 3 || d.kw != 3 || d.pad != 1) return 0;
     if (d.stride == 1) return d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
     if (d.stride == 2) return d.Wo > 8 ? 4 : 5;
     return 0;
 }
 
-// a stride-1 1x1 layer seen as N x Ci "images" of one row of H*W positions
+// a 1x1 layer seen as N x Ci "images" of one row of Ho*Wo positions (the whole plane when the stride is 1)
 static ConvDims as_one_row(const ConvDims &d) {
     ConvDims f = d;
     f.H = f.Ho = 1;
-    f.W = f.Wo = d.H * d.W;
+    f.W = f.Wo = d.Ho * d.Wo;
+    f.stride = 1;
     return f;
 }
+static Subsample sampling_of(const ConvDims &d) { return Subsample{d.stride, d.Wo, d.W, d.H * d.W}; }
 
 int fwd_stats_slots(const ConvDims &d) {
     switch (fwd_tiled_variant(d)) {
@@ -341,6 +345,8 @@ int fwd_stats_slots(const ConvDims &d) {
         case 5: return stats_slots_3x3<FwdW8S2>(d);
         case 6: return stats_slots_3x3<Fwd1x1>(as_one_row(d));
         case 7: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
+        case 8: return stats_slots_3x3<Fwd1x1>(as_one_row(d));
+        case 9: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
         default: return 0;
     }
 }
@@ -352,7 +358,12 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
                       (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                       (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0);
     const int variant = fwd_tiled_variant(d);
-    if (variant >= 6) {
+    if (variant >= 8) {   // x is read element by element; y is a dense row per plane
+        const ConvDims f = as_one_row(d);
+        if (f.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0)
+            return variant == 8 ? launch_fwd_3x3_v<Fwd1x1, false, true>(x, w, y, stats, f, s, sampling_of(d))
+                                : launch_fwd_3x3_v<Fwd1x1s, false, true>(x, w, y, stats, f, s, sampling_of(d));
+    } else if (variant >= 6) {
         const ConvDims f = as_one_row(d);
         if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0)
             return variant == 6 ? launch_fwd_3x3<Fwd1x1>(x, w, y, stats, f, s)

@@ -215,7 +215,8 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
     // float4 loads need 16-byte aligned bases; tensors whose rows are read element by element do not
     // (1x1 layers on the matrix cores walk whole planes as rows: their row length is H*W)
     const bool rows_1x1 = p.variant == 2 && d.kh == 1;
-    const bool need_x16 = p.variant == 2 && (rows_1x1 ? d.H * d.W : d.W) % 4 == 0;
+    const bool need_x16 = p.variant == 2 && !(rows_1x1 && d.stride > 1) &&   // (a strided 1x1 layer samples x element-wise)
+                          (rows_1x1 ? d.H * d.W : d.W) % 4 == 0;
     const bool need_g16 = p.variant == 2 && (rows_1x1 ? d.Ho * d.Wo : d.Wo) % 4 == 0;
     if (p.variant && ((need_x16 && (reinterpret_cast<uintptr_t>(x) & 15)) ||
                       (need_g16 && (reinterpret_cast<uintptr_t>(gy) & 15))))

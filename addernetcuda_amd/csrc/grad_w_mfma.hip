@@ -101,13 +101,15 @@ __device__ __forceinline__ void gy_commit_m(const GyStageM<G> &st, float *buf) {
     }
 }
 
-template <class G, bool VEC = true>
+// SUB (single tap only): x is a sampled tensor (see Subsample), read element by element at the sampled
+// positions; gy is dense.  VEC then only says how gy is read.
+template <class G, bool VEC = true, bool SUB = false>
 __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *__restrict__ gy,
                                                                   const float *__restrict__ x,
                                                                   double *__restrict__ part,
                                                                   double *__restrict__ sgpart, int N, int Ci, int H,
                                                                   int W, int Co, int Ho, int Wo, int tilesH,
-                                                                  int tilesW, int ntiles) {
+                                                                  int tilesW, int ntiles, const Subsample sub) {
     using XP = typename G::XP;
     constexpr int S = G::S, MT = G::MT, NT = G::NT;
     extern __shared__ __align__(16) float smem[];
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
     };
     if (tile < ntiles) {
         decode(tile);
-        tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W);
+        tile_fetch<XP, VEC && !SUB, SUB>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
         gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         tile_commit<XP>(xs, smem);
         gy_commit_m<G>(gs, smem + XP::BUF);
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
         const int next = tile + gridDim.x;
         if (next < ntiles) {   // next tile's global loads fly during this tile's arithmetic
             decode(next);
-            tile_fetch<XP, VEC>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W);
+            tile_fetch<XP, VEC && !SUB, SUB>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
             gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         }
         const float *base = smem + cur * G::BUF;
@@ -286,20 +288,21 @@ static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
     if (p.slots < 1) p.slots = 1;
 }
 
-// a stride-1 1x1 layer seen as images of one row of H*W positions
+// a 1x1 layer seen as images of one row of Ho*Wo positions (the whole plane when the stride is 1)
 static ConvDims mfma_one_row(const ConvDims &d) {
     ConvDims f = d;
     f.H = f.Ho = 1;
-    f.W = f.Wo = d.H * d.W;
+    f.W = f.Wo = d.Ho * d.Wo;
+    f.stride = 1;
     return f;
 }
 
 GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     GradWMfmaPlan p{};
-    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 64) {
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.Ci >= 64 && d.Co >= 64) {
         const ConvDims f = mfma_one_row(d);
-        p.variant = f.W > 64 ? 6 : 7;
-        if (p.variant == 6) plan_one<Gm1x1>(f, p);
+        p.variant = (f.W > 64 ? 6 : 7) + (d.stride > 1 ? 2 : 0);   // 8, 9: x sampled at every stride-th row and column
+        if (f.W > 64) plan_one<Gm1x1>(f, p);
         else plan_one<Gm1x1s>(f, p);
         return p;
     }
@@ -318,18 +321,18 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     return p;
 }
 
-template <class G, bool VEC>
+template <class G, bool VEC, bool SUB = false>
 static int launch_one_v(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
-                      const GradWMfmaPlan &p, hipStream_t s) {
+                      const GradWMfmaPlan &p, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
     static bool attr_set = false;
     if (!attr_set && G::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_mfma_kernel<G, VEC>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_mfma_kernel<G, VEC, SUB>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
-                       part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles);
+    hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC, SUB>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
+                       part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles, sub);
     return check_launch();
 }
 
@@ -351,6 +354,17 @@ int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sg
         case 5: return launch_one<GmW8S2>(gy, x, part, sgpart, d, p, s);
         case 6: return launch_one<Gm1x1>(gy, x, part, sgpart, mfma_one_row(d), p, s);
         case 7: return launch_one<Gm1x1s>(gy, x, part, sgpart, mfma_one_row(d), p, s);
+        case 8:
+        case 9: {
+            const ConvDims f = mfma_one_row(d);
+            const Subsample sub{d.stride, d.Wo, d.W, d.H * d.W};
+            const bool vec = f.Wo % 4 == 0;
+            if (p.variant == 8)
+                return vec ? launch_one_v<Gm1x1, true, true>(gy, x, part, sgpart, f, p, s, sub)
+                           : launch_one_v<Gm1x1, false, true>(gy, x, part, sgpart, f, p, s, sub);
+            return vec ? launch_one_v<Gm1x1s, true, true>(gy, x, part, sgpart, f, p, s, sub)
+                       : launch_one_v<Gm1x1s, false, true>(gy, x, part, sgpart, f, p, s, sub);
+        }
         default: return ADDER_ERR_BAD_SHAPE;
     }
 }

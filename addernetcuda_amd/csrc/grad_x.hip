@@ -92,13 +92,17 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
 //   gx[hi,wi] += hardtanh(w[co,ci,i,j] - x[hi,wi]) * gy[hi+1-i, wi+1-j]
 // In tile coordinates (row 0 = h0-1, column 0 = w0-1) that is row+2-i, t+2-j.
 // ---------------------------------------------------------------------------
-template <class C, bool VEC = true, bool SAT = true>
+// SUB (single tap only): x and gx are sampled tensors (see Subsample); the kernel walks the sampled
+// positions as one row per plane, reads x there, and stores each result together with the zeros of the
+// s x s block of input positions around it that the layer never read.
+template <class C, bool VEC = true, bool SAT = true, bool SUB = false>
 __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const float *__restrict__ gy,
                                                                    const float *__restrict__ x,
                                                                    const float *__restrict__ w,
                                                                    float *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int tilesH,
-                                                                   int tilesW) {
+                                                                   int tilesW, const Subsample sub) {
+    static_assert(!SUB || C::KS == 1, "sampling is for single-tap layers");
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
 
@@ -132,13 +136,25 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
     // accumulators live in registers for the whole kernel (two-level sum: acc collects one chunk of
     // output channels, tot the chunks)
     float cr[TM][TN], acc[TM][TN], tot[TM][TN];
+    int xoff[TN];   // offset of the own positions in their plane
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        const int pos = min(wi0 + t, W - 1);
+        if constexpr (SUB) {
+            const int ho = pos / sub.wv;
+            xoff[t] = ho * sub.s * sub.pitch + (pos - ho * sub.wv) * sub.s;
+        } else {
+            xoff[t] = hc * W + pos;
+        }
+    }
+    const int xplane = SUB ? sub.plane : H * W;
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
-        const float *src = x + (((size_t)nc * Ci + ci) * H + hc) * W;
+        const float *src = x + ((size_t)nc * Ci + ci) * xplane;
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
-            const float xv = src[min(wi0 + t, W - 1)];
+            const float xv = src[xoff[t]];
             cr[m][t] = SAT ? fmaf(-0.5f, xv, 0.5f) : xv;
             acc[m][t] = tot[m][t] = 0.f;
         }
@@ -278,6 +294,19 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
         for (int m = 0; m < TM; ++m) {
             const int ci = ci_base + m;
             if (ci >= ci_first) {
+                if constexpr (SUB) {
+                    float *plane = gx + ((size_t)n * Ci + ci) * sub.plane;
+                    const int rows = sub.plane / sub.pitch;
+#pragma unroll
+                    for (int t = 0; t < TN; ++t) {
+                        if (wi0 + t >= W) continue;
+                        const int r0 = xoff[t] / sub.pitch, c0 = xoff[t] - r0 * sub.pitch;
+                        for (int a = 0; a < sub.s && r0 + a < rows; ++a)
+                            for (int b = 0; b < sub.s && c0 + b < sub.pitch; ++b)
+                                plane[xoff[t] + a * sub.pitch + b] = (a | b) ? 0.f : tot[m][t];
+                    }
+                    continue;
+                }
                 float *dst = gx + (((size_t)n * Ci + ci) * H + hi) * W + wi0;
                 if (TN % 4 == 0 && (W & 3) == 0 && wi0 + TN <= W) {
 #pragma unroll
@@ -300,9 +329,9 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 // at 4608).  Layers with more terms per output than this keep the three-instruction form.
 static constexpr int kSatMaxTerms = 2304;
 
-template <class C, bool VEC, bool SAT>
+template <class C, bool VEC, bool SAT, bool SUB = false>
 static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s) {
+                               const ConvDims &d, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
@@ -310,13 +339,13 @@ static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w
     static bool attr_set = false;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     if (!attr_set && LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C, VEC, SAT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C, VEC, SAT, SUB>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
-                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW);
+    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
+                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW, sub);
     return check_launch();
 }
 
@@ -625,6 +654,21 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         f.W = f.Wo = d.H * d.W;
         if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0)
             return f.W > 64 ? launch_grad_x_3x3s1<Gx1x1>(gy, x, w, gx, f, s) : launch_grad_x_3x3s1<Gx1x1s>(gy, x, w, gx, f, s);
+    }
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride > 1 && d.Ci >= 64 && d.Co >= 64) {
+        ConvDims f = d;   // the sampled positions of every plane as one row; x and gx are read / written in place
+        f.H = f.Ho = 1;
+        f.W = f.Wo = d.Ho * d.Wo;
+        f.stride = 1;
+        const Subsample sub{d.stride, d.Wo, d.W, d.H * d.W};
+        const bool vec = f.W % 4 == 0;
+        if (!vec || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) {
+            if (f.W > 64)
+                return vec ? launch_grad_x_3x3s1_v<Gx1x1, true, true, true>(gy, x, w, gx, f, s, sub)
+                           : launch_grad_x_3x3s1_v<Gx1x1, false, true, true>(gy, x, w, gx, f, s, sub);
+            return vec ? launch_grad_x_3x3s1_v<Gx1x1s, true, true, true>(gy, x, w, gx, f, s, sub)
+                       : launch_grad_x_3x3s1_v<Gx1x1s, false, true, true>(gy, x, w, gx, f, s, sub);
+        }
     }
     if (conv1x1_supported(d, gy, gx))
         return launch_grad_x_1x1(gy, x, w, gx, d, s);

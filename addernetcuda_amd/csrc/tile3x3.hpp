@@ -36,6 +36,13 @@ struct PatchCfg {
     static_assert(RHALO == 0 || RHALO == 1, "at most one halo column per side");
 };
 
+// A tensor that is read at every s-th row and column only (a strided single-tap layer): the kernels walk
+// the sampled positions of a plane, `wv` per row, as one long row; `pitch` and `plane` are the row length
+// and the plane size of the tensor as it lies in memory.
+struct Subsample {
+    int s, wv, pitch, plane;
+};
+
 template <class P>
 struct TileStage {
     float4 v[P::VITER];
@@ -47,10 +54,13 @@ struct TileStage {
 // interior element of the patch.  Everything outside the tensor reads as zero.  VEC = false is for
 // tensors whose rows are not float4-aligned (W % 4 != 0): element-wise loads.  Index arithmetic is
 // 32-bit: the C ABI refuses tensors of 2^31 elements or more.
-template <class P, bool VEC = true>
+// SUB: src is sampled as described by `sub`; (H, W) = (1, sampled positions per plane).
+template <class P, bool VEC = true, bool SUB = false>
 __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__restrict__ src,
                                            int chan0, int nchan, int n0, int nimg_total, int hb,
-                                           int wb, int H, int W) {
+                                           int wb, int H, int W, const Subsample sub = Subsample{1, 0, 0, 0}) {
+    static_assert(!(SUB && VEC), "sampled tensors are read element by element");
+    static_assert(!SUB || (P::ROWS == 1 && P::NSIDES == 0), "sampling is for single-tap tiles walked as one row");
     const int tid = threadIdx.x;
 #pragma unroll
     for (int it = 0; it < P::VITER; ++it) {
@@ -64,6 +74,18 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
                         hi >= 0 && hi < H && wi < W;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok) {
+            if constexpr (SUB) {
+                const float *base = src + (size_t)(n * nchan + ch) * sub.plane;
+                int ho = wi / sub.wv, wo = wi - ho * sub.wv;
+                float e[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    e[k] = wi + k < W ? base[ho * sub.s * sub.pitch + wo * sub.s] : 0.f;
+                    if (++wo == sub.wv) { wo = 0; ++ho; }
+                }
+                st.v[it] = make_float4(e[0], e[1], e[2], e[3]);
+                continue;
+            }
             const float *row = src + (((n * nchan + ch) * H + hi) * W + wi);
             if constexpr (VEC) {
                 val = *reinterpret_cast<const float4 *>(row);

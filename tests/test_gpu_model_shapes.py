@@ -43,10 +43,12 @@ def test_layer_matches_oracle(case, gpu):
     assert_close(wg.grad, c_oracle.conv2d_grad_w(gy, x, w, s, p), f"grad_W {case}")
 
 
-@pytest.mark.parametrize("case", [(2, 64, 28, 28, 96, 1, 2, 0), (2, 128, 14, 14, 64, 1, 2, 0), (1, 64, 9, 9, 64, 1, 3, 0)], ids=str)
-def test_strided_1x1_with_many_channels_runs_on_the_subsampled_input(case, gpu):
-    """adder2d_function turns these into the stride-1 layer on x[:, :, ::s, ::s]; results and both gradients
-    (the input gradient scattered back with exact zeros in between) must be those of the strided layer."""
+@pytest.mark.parametrize("case", [(2, 64, 28, 28, 96, 1, 2, 0), (2, 128, 14, 14, 64, 1, 2, 0), (1, 64, 9, 9, 64, 1, 3, 0),
+                                  (3, 64, 7, 7, 128, 1, 2, 0), (2, 72, 10, 6, 64, 1, 2, 0), (5, 64, 8, 8, 64, 1, 4, 0)], ids=str)
+def test_strided_1x1_with_many_channels_walks_the_sampled_positions(case, gpu):
+    """From 64 channels on, the tiled kernels walk the sampled positions x[:, :, ::s, ::s] of a strided 1x1
+    layer like a stride-1 plane; results and both gradients (the input gradient stored together with the
+    exact zeros in between) must be those of the strided layer."""
     from addernetcuda_amd import adder
     from oracle import c_oracle
     N, Ci, H, W, Co, k, s, p = case

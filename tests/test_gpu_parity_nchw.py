@@ -128,3 +128,19 @@ def test_clamp_saturates_both_ways(gpu):
         xg = x.to(gpu).requires_grad_(True)
         adder.adder2d_function(xg, w.to(gpu), 1, 1).backward(gy.to(gpu))
         assert_close(xg.grad, -sign * expect, f"saturated sign={sign}")
+
+
+@pytest.mark.parametrize("x_scale", [0.05, 20.0, 3000.0])
+@pytest.mark.parametrize("case", [(4, 16, 16, 16, 32, 3, 1, 1), (4, 32, 16, 16, 32, 3, 2, 1), (4, 64, 8, 8, 64, 1, 1, 0),
+                                  (4, 16, 16, 16, 32, 1, 2, 0)], ids=str)
+def test_grad_x_does_not_degrade_with_the_scale_of_x(case, x_scale, gpu):
+    """The tiled grad_X kernels evaluate hardtanh(w - x) as 2 * sat(0.5 w + (0.5 - 0.5 x)) - 1; the
+    rounding of 0.5 - 0.5 x must not show for activations much smaller or larger than the weights
+    (terms that do not saturate have |x| <= |w| + 1 whatever the scale of x)."""
+    from addernetcuda_amd import adder
+    from oracle import c_oracle
+    s, p = case[6], case[7]
+    x, w, gy = make_case(*case, w_init="normal", x_scale=x_scale)
+    xg = x.to(gpu).requires_grad_(True)
+    adder.adder2d_function(xg, w.to(gpu), s, p, eta=0.0).backward(gy.to(gpu))
+    assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p), f"grad_X x_scale={x_scale} {case}")
