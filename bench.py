@@ -244,7 +244,7 @@ def graph_matches_eager(dev, replays=4):
     return ok, worst, losses
 
 
-def cpu_baseline(repeats=5):
+def cpu_baseline(repeats=15):   # ~10 s of host work
     """The CPU oracle's ResNet-20 training step at batch 8 (seeded), median of `repeats`, scaled to batch 256."""
     from addernetcuda_amd.resnet20 import resnet20
     from oracle import adder_oracle
