@@ -35,9 +35,10 @@ _SIGNATURES = {
     "adder_norm_scale_workspace_bytes": (_i, [_l, _szp]),
     "adder_grad_norm_scale_f32": (_i, [_p, _l, _f, _f, _p, _sz, _p]),
     "adder_bn_act_workspace_bytes": (_i, [_i, _i, _i, _szp]),
-    "adder_bn_act_fwd_f32": (_i, [_p] * 10 + [_f, _f, _i, _i, _i, _i, _p, _sz, _p]),
-    "adder_bn_act_fwd_stats_f32": (_i, [_p] * 10 + [_f, _f, _i, _i, _i, _i, _p, _i, _p]),
-    "adder_bn_act_bwd_f32": (_i, [_p] * 10 + [_i, _i, _i, _i, _p, _sz, _p]),
+    "adder_bn_act_mask_words": (_i, [_i, _i, _i, _szp]),
+    "adder_bn_act_fwd_f32": (_i, [_p] * 11 + [_f, _f, _i, _i, _i, _i, _p, _sz, _p]),
+    "adder_bn_act_fwd_stats_f32": (_i, [_p] * 11 + [_f, _f, _i, _i, _i, _i, _p, _i, _p]),
+    "adder_bn_act_bwd_f32": (_i, [_p] * 11 + [_i, _i, _i, _i, _p, _sz, _p]),
 }
 for _name, (_res, _args) in _SIGNATURES.items():
     _fn = getattr(lib, _name)

@@ -36,38 +36,47 @@ class _bn_act(Function):
         y = torch.empty_like(x)
         mean = torch.empty(C, dtype=torch.float32, device=dev)
         rstd = torch.empty(C, dtype=torch.float32, device=dev)
+        # the backward needs y only for its sign: one bit per element where the kernels offer it
+        mask = None
+        if relu and all(t is None or t.data_ptr() % 16 == 0 for t in (x, y, residual)):
+            words = ctypes.c_size_t(0)
+            check(lib.adder_bn_act_mask_words(N, C, HW, ctypes.byref(words)), "adder_bn_act_mask_words")
+            if words.value:
+                mask = torch.empty(words.value, dtype=torch.int32, device=dev)
         with torch.cuda.device(dev):
             if stats is not None:
                 # the layer that produced x already summed x and x*x per channel (adder.forward_with_stats)
                 if stats.dtype != torch.float64 or stats.dim() != 3 or stats.shape[0] != C or stats.shape[2] != 2 \
                         or not stats.is_contiguous() or stats.device != dev:
                     raise RuntimeError("stats must be a contiguous float64 tensor (C, slots, 2) on the device of x")
-                check(lib.adder_bn_act_fwd_stats_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mean),
-                                                     ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
+                check(lib.adder_bn_act_fwd_stats_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mask),
+                                                     ptr(mean), ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
                                                      float(momentum), float(eps), int(relu), N, C, HW, ptr(stats),
                                                      int(stats.shape[1]), stream_ptr(dev)), "adder_bn_act_fwd_stats_f32")
             else:
                 ws, nbytes = _workspace(N, C, HW, dev)
-                check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mean),
-                                               ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
+                check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mask),
+                                               ptr(mean), ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
                                                float(momentum), float(eps), int(relu), N, C, HW, ptr(ws), nbytes,
                                                stream_ptr(dev)), "adder_bn_act_fwd_f32")
-        ctx.save_for_backward(x, y if relu else None, weight, mean, rstd)
+        ctx.save_for_backward(x, y if relu and mask is None else None, weight, mean, rstd, mask)
         ctx.relu, ctx.has_res, ctx.dims = relu, residual is not None, (N, C, HW)
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, y, weight, mean, rstd = ctx.saved_tensors
+        x, y, weight, mean, rstd, mask = ctx.saved_tensors
         dy = dy.contiguous()
         N, C, HW = ctx.dims
         dev = x.device
         dx = torch.empty_like(x)
         dres = torch.empty_like(x) if ctx.has_res else None
         dgamma, dbeta = torch.empty_like(weight), torch.empty_like(weight)
+        if mask is not None and dy.data_ptr() % 16:
+            dy = dy.clone()   # the masked kernels move float4 groups
         with torch.cuda.device(dev):
             ws, nbytes = _workspace(N, C, HW, dev)
-            check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
+            check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(mask), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
                                            ptr(dres), ptr(dgamma), ptr(dbeta), int(ctx.relu), N, C, HW, ptr(ws), nbytes,
                                            stream_ptr(dev)), "adder_bn_act_bwd_f32")
         return dx, dgamma, dbeta, dres, None, None, None, None, None, None, None

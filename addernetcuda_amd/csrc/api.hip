@@ -61,7 +61,7 @@ const char *adder_strerror(int status) {
 
 const char *adder_last_hip_error(void) { return g_last_hip_error.c_str(); }
 
-int adder_abi_version(void) { return 1; }
+int adder_abi_version(void) { return 2; }
 
 int adder_out_dim(int h, int k, int pad, int stride) {
     if (h <= 0 || k <= 0 || pad < 0 || stride <= 0 || h + 2 * pad < k) return 0;
@@ -232,45 +232,63 @@ int adder_bn_act_workspace_bytes(int N, int C, int HW, size_t *bytes) {
     return ADDER_OK;
 }
 
+int adder_bn_act_mask_words(int N, int C, int HW, size_t *words) {
+    if (!words) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_bn(N, C, HW)) return rc;
+    *words = bn_mask_words(N, C, HW);
+    return ADDER_OK;
+}
+
+// a sign mask needs ReLU, a shape that has one, and float4-aligned tensors
+static int check_mask(const void *mask, int relu, int N, int C, int HW) {
+    if (!mask) return ADDER_OK;
+    if (!relu || bn_mask_words(N, C, HW) == 0) return ADDER_ERR_UNSUPPORTED;
+    return ADDER_OK;
+}
+
 int adder_bn_act_fwd_f32(const float *x, const float *residual, const float *gamma, const float *beta, float *y,
-                         float *save_mean, float *save_rstd, float *running_mean, float *running_var,
-                         long long *num_batches_tracked, float momentum, float eps, int relu, int N, int C, int HW,
-                         void *ws, size_t ws_bytes, void *stream) {
+                         unsigned int *relu_mask, float *save_mean, float *save_rstd, float *running_mean,
+                         float *running_var, long long *num_batches_tracked, float momentum, float eps, int relu,
+                         int N, int C, int HW, void *ws, size_t ws_bytes, void *stream) {
     if (!x || !gamma || !beta || !y || !save_mean || !save_rstd) return ADDER_ERR_NULL_POINTER;
     if ((running_mean == nullptr) != (running_var == nullptr)) return ADDER_ERR_NULL_POINTER;
     if (int rc = check_bn(N, C, HW)) return rc;
+    if (int rc = check_mask(relu_mask, relu, N, C, HW)) return rc;
     if (!(eps > 0.f) || !(momentum >= 0.f && momentum <= 1.f)) return ADDER_ERR_BAD_SHAPE;
     if (!ws || ws_bytes < bn_workspace_bytes(N, C, HW) || (reinterpret_cast<uintptr_t>(ws) & 255))
         return ADDER_ERR_WORKSPACE;
-    return launch_bn_act_fwd(x, residual, gamma, beta, y, save_mean, save_rstd, running_mean, running_var,
+    return launch_bn_act_fwd(x, residual, gamma, beta, y, relu_mask, save_mean, save_rstd, running_mean, running_var,
                              num_batches_tracked, momentum, eps, relu != 0, N, C, HW, ws, nullptr, 0,
                              static_cast<hipStream_t>(stream));
 }
 
 int adder_bn_act_fwd_stats_f32(const float *x, const float *residual, const float *gamma, const float *beta, float *y,
-                               float *save_mean, float *save_rstd, float *running_mean, float *running_var,
-                               long long *num_batches_tracked, float momentum, float eps, int relu, int N, int C,
-                               int HW, const double *stats, int stats_slots, void *stream) {
+                               unsigned int *relu_mask, float *save_mean, float *save_rstd, float *running_mean,
+                               float *running_var, long long *num_batches_tracked, float momentum, float eps, int relu,
+                               int N, int C, int HW, const double *stats, int stats_slots, void *stream) {
     if (!x || !gamma || !beta || !y || !save_mean || !save_rstd || !stats) return ADDER_ERR_NULL_POINTER;
     if ((running_mean == nullptr) != (running_var == nullptr)) return ADDER_ERR_NULL_POINTER;
     if (int rc = check_bn(N, C, HW)) return rc;
+    if (int rc = check_mask(relu_mask, relu, N, C, HW)) return rc;
     if (stats_slots <= 0) return ADDER_ERR_BAD_SHAPE;
     if (!(eps > 0.f) || !(momentum >= 0.f && momentum <= 1.f)) return ADDER_ERR_BAD_SHAPE;
-    return launch_bn_act_fwd(x, residual, gamma, beta, y, save_mean, save_rstd, running_mean, running_var,
+    return launch_bn_act_fwd(x, residual, gamma, beta, y, relu_mask, save_mean, save_rstd, running_mean, running_var,
                              num_batches_tracked, momentum, eps, relu != 0, N, C, HW, nullptr, stats, stats_slots,
                              static_cast<hipStream_t>(stream));
 }
 
-int adder_bn_act_bwd_f32(const float *dy, const float *y, const float *x, const float *gamma, const float *save_mean,
-                         const float *save_rstd, float *dx, float *dresidual, float *dgamma, float *dbeta, int relu,
-                         int N, int C, int HW, void *ws, size_t ws_bytes, void *stream) {
+int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsigned int *relu_mask, const float *x,
+                         const float *gamma, const float *save_mean, const float *save_rstd, float *dx,
+                         float *dresidual, float *dgamma, float *dbeta, int relu, int N, int C, int HW, void *ws,
+                         size_t ws_bytes, void *stream) {
     if (!dy || !x || !gamma || !save_mean || !save_rstd || !dx || !dgamma || !dbeta) return ADDER_ERR_NULL_POINTER;
-    if (relu && !y) return ADDER_ERR_NULL_POINTER;
+    if (relu && !y && !relu_mask) return ADDER_ERR_NULL_POINTER;
     if (int rc = check_bn(N, C, HW)) return rc;
+    if (int rc = check_mask(relu_mask, relu, N, C, HW)) return rc;
     if (!ws || ws_bytes < bn_workspace_bytes(N, C, HW) || (reinterpret_cast<uintptr_t>(ws) & 255))
         return ADDER_ERR_WORKSPACE;
-    return launch_bn_act_bwd(dy, y, x, gamma, save_mean, save_rstd, dx, dresidual, dgamma, dbeta, relu != 0, N, C, HW,
-                             ws, static_cast<hipStream_t>(stream));
+    return launch_bn_act_bwd(dy, y, relu_mask, x, gamma, save_mean, save_rstd, dx, dresidual, dgamma, dbeta, relu != 0,
+                             N, C, HW, ws, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

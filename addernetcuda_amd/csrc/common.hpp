@@ -132,12 +132,14 @@ int launch_grad_w_1x1(const float *gy, const float *x, float *part, float *sgpar
 
 // fused BatchNorm + residual + ReLU (bn_act.hip)
 size_t bn_workspace_bytes(int N, int C, int HW);
+size_t bn_mask_words(int N, int C, int HW);
 int launch_bn_act_fwd(const float *x, const float *res, const float *gamma, const float *beta, float *y,
-                      float *mean, float *rstd, float *running_mean, float *running_var, long long *num_batches,
-                      float momentum, float eps, int relu, int N, int C, int HW, void *ws, const double *stats, int stats_slots, hipStream_t s);
-int launch_bn_act_bwd(const float *dy, const float *y, const float *x, const float *gamma, const float *mean,
-                      const float *rstd, float *dx, float *dres, float *dgamma, float *dbeta, int relu, int N,
-                      int C, int HW, void *ws, hipStream_t s);
+                      unsigned *mask, float *mean, float *rstd, float *running_mean, float *running_var,
+                      long long *num_batches, float momentum, float eps, int relu, int N, int C, int HW, void *ws,
+                      const double *stats, int stats_slots, hipStream_t s);
+int launch_bn_act_bwd(const float *dy, const float *y, const unsigned *mask, const float *x, const float *gamma,
+                      const float *mean, const float *rstd, float *dx, float *dres, float *dgamma, float *dbeta,
+                      int relu, int N, int C, int HW, void *ws, hipStream_t s);
 
 size_t norm_scale_workspace_bytes(long n);
 int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);

@@ -13,6 +13,7 @@ processes are needed.
 
     python -m addernetcuda_amd.train --synthetic 4096 --epochs 2
     python -m addernetcuda_amd.train --data cifar10.npz --epochs 400 --output-dir models/
+    python -m addernetcuda_amd.train --data cifar10.npz --resume models/addernet.pt --eval-only
     (npz keys: x_train (N,32,32,3) or (N,3,32,32) uint8, y_train (N,), x_test, y_test)
 """
 import argparse
@@ -124,6 +125,10 @@ def run(args):
     if args.resume:
         net.load_state_dict(torch.load(args.resume, map_location=dev, weights_only=True))
     opt = torch.optim.SGD(net.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4, fused=True)
+    if args.eval_only:   # the reference's test.py: load a checkpoint, one pass over the test split
+        test_loss, acc = evaluate(net, *data["test"], args.test_batch_size)
+        print(f"test loss {test_loss:.4f}  accuracy {acc:.4f}", flush=True)
+        return [{"epoch": 0, "test_loss": test_loss, "accuracy": acc}]
     os.makedirs(args.output_dir, exist_ok=True)
     gen = torch.Generator(device=dev).manual_seed(args.seed)
     best, history = 0.0, []
@@ -152,6 +157,7 @@ def parse_args(argv=None):
     p.add_argument("--synthetic", type=int, default=8192, help="training-set size when --data is not given")
     p.add_argument("--output-dir", type=str, default="./models/")
     p.add_argument("--resume", type=str, default=None, help="state_dict to start from")
+    p.add_argument("--eval-only", action="store_true", help="evaluate the --resume checkpoint and stop (test.py:74-80)")
     p.add_argument("--epochs", type=int, default=400)                 # main.py:135
     p.add_argument("--batch-size", type=int, default=256)
     p.add_argument("--test-batch-size", type=int, default=500)

@@ -142,22 +142,29 @@ ADDER_API int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps,
  *             (nullable, both or neither) are updated with `momentum` (unbiased variance);
  *             num_batches_tracked (nullable, one int64 on the device) is incremented by one.
  *   backward: dx, dgamma, dbeta; dresidual (nullable) receives the gradient of the residual input.
- *             y (the forward output) is needed only when relu != 0.
+ *             y (the forward output) is needed only when relu != 0, and only for its sign:
+ *   relu_mask (nullable, relu != 0 only): adder_bn_act_mask_words(N, C, HW) 32-bit words, one bit per
+ *             element of y (bit i % 32 of word i / 32 = [y_i > 0]), written by the forward and read by the
+ *             backward in place of y -- a quarter less HBM traffic in the backward.  Shapes whose planes
+ *             are not whole words (H*W % 32 != 0) report 0 words and take ADDER_ERR_UNSUPPORTED for a
+ *             non-null mask, as do tensors that are not 16-byte aligned.
  * ---------------------------------------------------------------------- */
 ADDER_API int adder_bn_act_workspace_bytes(int N, int C, int HW, size_t *bytes);
+ADDER_API int adder_bn_act_mask_words(int N, int C, int HW, size_t *words);
 ADDER_API int adder_bn_act_fwd_f32(const float *x, const float *residual, const float *gamma, const float *beta,
-                                   float *y, float *save_mean, float *save_rstd,
+                                   float *y, unsigned int *relu_mask, float *save_mean, float *save_rstd,
                                    float *running_mean, float *running_var, long long *num_batches_tracked,
                                    float momentum, float eps, int relu,
                                    int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);
 /* adder_bn_act_fwd_f32 with the statistics pass already done by the producer of x
  * (adder_conv2d_fwd_stats_f32): `stats` holds C x stats_slots pairs of partial sums; no workspace. */
 ADDER_API int adder_bn_act_fwd_stats_f32(const float *x, const float *residual, const float *gamma, const float *beta,
-                                         float *y, float *save_mean, float *save_rstd,
+                                         float *y, unsigned int *relu_mask, float *save_mean, float *save_rstd,
                                          float *running_mean, float *running_var, long long *num_batches_tracked,
                                          float momentum, float eps, int relu,
                                          int N, int C, int HW, const double *stats, int stats_slots, void *stream);
-ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const float *x, const float *gamma,
+ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsigned int *relu_mask,
+                                   const float *x, const float *gamma,
                                    const float *save_mean, const float *save_rstd,
                                    float *dx, float *dresidual, float *dgamma, float *dbeta, int relu,
                                    int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);

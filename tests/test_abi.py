@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_status_strings_and_version():
     from addernetcuda_amd._lib import lib
-    assert lib.adder_abi_version() == 1
+    assert lib.adder_abi_version() == 2
     assert lib.adder_strerror(0) == b"ok"
     seen = {lib.adder_strerror(c) for c in range(-7, 1)}
     assert len(seen) == 8 and b"unknown status" not in seen
@@ -133,6 +133,26 @@ def test_statistics_variants_validate_without_a_gpu():
     assert lib.adder_conv2d_fwd_stats_f32(fake, fake, ctypes.c_void_p(1 << 40), ctypes.c_void_p(1 << 41), 4,
                                           4, 8, 16, 16, 8, 1, 1, 1, 0, None) == -7
     bn = lib.adder_bn_act_fwd_stats_f32
-    args = [fake] * 10 + [0.1, 1e-5, 1, 4, 8, 64]
+    args = [fake] * 5 + [None] + [fake] * 5 + [0.1, 1e-5, 1, 4, 8, 64]
     assert bn(*args, None, 4, None) == -1
     assert bn(*args, fake, 0, None) == -2
+
+
+def test_relu_mask_is_offered_for_whole_word_planes_only():
+    """adder_bn_act_mask_words: one bit per element when H*W is a multiple of 32, otherwise no mask; a mask
+    passed for such a shape, or without ReLU, is refused before any HIP call."""
+    from addernetcuda_amd._lib import lib
+    words = ctypes.c_size_t(99)
+    assert lib.adder_bn_act_mask_words(256, 16, 1024, ctypes.byref(words)) == 0 and words.value == 256 * 16 * 32
+    assert lib.adder_bn_act_mask_words(4, 8, 64, ctypes.byref(words)) == 0 and words.value == 4 * 8 * 2
+    assert lib.adder_bn_act_mask_words(4, 8, 49, ctypes.byref(words)) == 0 and words.value == 0
+    assert lib.adder_bn_act_mask_words(4, 8, 64, None) == -1
+    fake = ctypes.c_void_p(4096)
+    ws = ctypes.c_void_p(1 << 20)
+    fwd_args = [fake] * 11 + [0.1, 1e-5]
+    assert lib.adder_bn_act_fwd_f32(*fwd_args, 1, 4, 8, 49, ws, 1 << 20, None) == -7    # no mask for 7x7 planes
+    assert lib.adder_bn_act_fwd_f32(*fwd_args, 0, 4, 8, 64, ws, 1 << 20, None) == -7    # no mask without ReLU
+    bwd_args = [fake] * 11
+    assert lib.adder_bn_act_bwd_f32(*bwd_args, 1, 4, 8, 49, ws, 1 << 20, None) == -7
+    no_y_no_mask = [fake, None, None] + [fake] * 8
+    assert lib.adder_bn_act_bwd_f32(*no_y_no_mask, 1, 4, 8, 64, ws, 1 << 20, None) == -1

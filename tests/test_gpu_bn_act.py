@@ -8,7 +8,8 @@ from tests.util import assert_close
 pytestmark = pytest.mark.gpu
 
 # (N, C, H, W)
-SHAPES = [(8, 16, 32, 32), (4, 64, 8, 8), (256, 16, 32, 32), (3, 5, 7, 7), (2, 10, 1, 1), (5, 33, 6, 10)]
+SHAPES = [(8, 16, 32, 32), (4, 64, 8, 8), (256, 16, 32, 32), (3, 5, 7, 7), (2, 10, 1, 1), (5, 33, 6, 10),
+          (2, 3, 4, 8), (3, 7, 16, 6)]   # the last two: the smallest planes that get a ReLU sign mask (32 and 96 elements)
 
 
 def _reference(x, res, gamma, beta, relu, dy, eps):

@@ -25,3 +25,8 @@ def test_two_epochs_learn_and_checkpoint(gpu, tmp_path):
     assert "layer1.0.conv1.adder" in state and "layer2.0.downsample.0.adder" in state and "bn2.running_mean" in state
     fresh = resnet20().to(gpu)
     fresh.load_state_dict(state)               # strict: same keys as the reference's resnet20.py
+    # the evaluation-only pass (test.py's job) reproduces the accuracy of the epoch that wrote the checkpoint
+    best = max(h["accuracy"] for h in hist)
+    ev = train.run(train.parse_args(["--synthetic", "2000", "--resume", ckpt, "--eval-only", "--test-batch-size", "50",
+                                     "--seed", "1"]))
+    assert abs(ev[0]["accuracy"] - best) < 1e-6
