@@ -144,3 +144,47 @@ def test_grad_x_does_not_degrade_with_the_scale_of_x(case, x_scale, gpu):
     xg = x.to(gpu).requires_grad_(True)
     adder.adder2d_function(xg, w.to(gpu), s, p, eta=0.0).backward(gy.to(gpu))
     assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p), f"grad_X x_scale={x_scale} {case}")
+
+
+def _random_cases(count, seed):
+    """Seeded random layer shapes around the kernels' switch points: channel counts on both sides of 64 and of
+    the tile sizes, map sizes that are and are not multiples of 4, kernels 1 / 3 / 5, strides 1..3."""
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    while len(cases) < count:
+        k = rnd.choice([1, 1, 3, 3, 3, 5])
+        s = rnd.choice([1, 1, 2, 3])
+        p = {1: 0, 3: rnd.choice([0, 1, 1]), 5: 2}[k]
+        ci = rnd.choice([1, 3, 7, 8, 16, 24, 63, 64, 65, 72, 130])
+        co = rnd.choice([1, 5, 8, 16, 33, 63, 64, 65, 96])
+        h, w = rnd.randint(k, 19), rnd.randint(k, 19)
+        n = rnd.randint(1, 5)
+        if ci * co * k * k * n * h * w > 6e7:     # keeps the C oracle at a fraction of a second per case
+            continue
+        cases.append((n, ci, h, w, co, k, s, p))
+    return cases
+
+
+def _random_1x1_cases(count, seed):
+    """1x1 layers with >= 64 channels on both sides (the tiled single-tap kernels and, with a stride, their
+    sampled-position variants), on planes of 4 .. 225 positions."""
+    import random
+    rnd = random.Random(seed)
+    return [(rnd.randint(1, 5), rnd.choice([64, 72, 80, 128, 136]), rnd.randint(2, 15), rnd.randint(2, 15),
+             rnd.choice([64, 65, 96, 130]), 1, rnd.choice([1, 2, 2, 3]), 0) for _ in range(count)]
+
+
+@pytest.mark.parametrize("case", _random_cases(40, 2024) + _random_1x1_cases(16, 7), ids=str)
+def test_random_shapes_match_oracle(case, gpu):
+    from addernetcuda_amd import adder
+    from oracle import c_oracle
+    s, p = case[6], case[7]
+    x, w, gy = make_case(*case, w_init="normal", seed=sum(case))
+    xg, wg = x.to(gpu).requires_grad_(True), w.to(gpu).requires_grad_(True)
+    y = adder.adder2d_function(xg, wg, s, p, eta=0.0)
+    y.backward(gy.to(gpu))
+    torch.cuda.synchronize()
+    assert_close(y, c_oracle.conv2d_fwd(x, w, s, p), f"forward {case}")
+    assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p), f"grad_X {case}")
+    assert_close(wg.grad, c_oracle.conv2d_grad_w(gy, x, w, s, p), f"grad_W {case}")
