@@ -27,6 +27,7 @@ _SIGNATURES = {
     "adder_conv2d_fwd_stats_f32": (_i, [_p, _p, _p, _p, _i] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_workspace_bytes": (_i, [_i] * 9 + [_szp]),
     "adder_conv2d_bwd_f32": (_i, [_p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
+    "adder_conv2d_bwd_add_f32": (_i, [_p, _p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
     "adder_col_fwd_f32": (_i, [_p, _p, _p, _i, _l, _i, _p]),
     "adder_col_bwd_workspace_bytes": (_i, [_i, _l, _i, _szp]),
     "adder_col_bwd_f32": (_i, [_p, _p, _p, _p, _p, _i, _l, _i, _p, _sz, _p]),

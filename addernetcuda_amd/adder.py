@@ -54,7 +54,7 @@ class _adder_nchw(Function):
     """Fused NCHW forward / backward (replaces adder.py:22-41 + 43-80 in one step each)."""
 
     @staticmethod
-    def forward(ctx, X, W, stride, padding, eta, with_stats=False):
+    def forward(ctx, X, W, stride, padding, eta, with_stats=False, with_shortcut=False):
         X, W = X.contiguous(), W.contiguous()
         require_gpu_f32(X, "X")
         require_gpu_f32(W, "W")
@@ -75,18 +75,27 @@ class _adder_nchw(Function):
                 check(lib.adder_conv2d_fwd_f32(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_f32")
         ctx.save_for_backward(X, W)  # the NCHW input, not the 9x larger X_col the reference keeps
         ctx.dims, ctx.eta = dims, eta
-        if not with_stats:
+        if not with_stats and not with_shortcut:
             return out
-        if stats is None:   # no statistics epilogue for this shape: an empty tensor stands for "none"
-            stats = torch.empty(0, device=dev, dtype=torch.float64)
-        ctx.mark_non_differentiable(stats)
-        ctx.set_materialize_grads(False)   # no zero-filled "gradient" of stats on the way back
-        return out, stats
+        ctx.set_materialize_grads(False)   # no zero-filled gradients for outputs nobody differentiates
+        outputs = [out]
+        if with_stats:
+            if stats is None:   # no statistics epilogue for this shape: an empty tensor stands for "none"
+                stats = torch.empty(0, device=dev, dtype=torch.float64)
+            ctx.mark_non_differentiable(stats)
+            outputs.append(stats)
+        if with_shortcut:
+            # X again, as an output of this node: what is back-propagated into it (a residual shortcut) reaches
+            # backward() together with grad_out and is added to grad_X by the kernel that computes grad_X
+            outputs.append(X.view_as(X))
+        return tuple(outputs)
 
     @staticmethod
-    def backward(ctx, grad_out, *unused):
+    def backward(ctx, grad_out, *more):
+        # more: the (absent) gradient of the statistics and / or the gradient of the shortcut output
+        grad_short = next((g for g in more if g is not None), None)
         if grad_out is None:
-            return None, None, None, None, None, None
+            return grad_short, None, None, None, None, None, None
         X, W = ctx.saved_tensors
         grad_out = grad_out.contiguous()
         require_gpu_f32(grad_out, "grad_output")
@@ -97,10 +106,22 @@ class _adder_nchw(Function):
         if need_x or need_w:
             with torch.cuda.device(dev):
                 ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev) if need_w else (None, 0)
-                check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw),
-                                               float(ctx.eta or 0.0), ptr(ws), nbytes, *ctx.dims, stream_ptr(dev)),
-                      "adder_conv2d_bwd_f32")
-        return gx, gw, None, None, None, None
+                fused = False
+                if need_x and grad_short is not None:
+                    grad_short = grad_short.contiguous()
+                    status = lib.adder_conv2d_bwd_add_f32(ptr(grad_out), ptr(X), ptr(W), ptr(grad_short), ptr(gx),
+                                                          ptr(gw), float(ctx.eta or 0.0), ptr(ws), nbytes, *ctx.dims,
+                                                          stream_ptr(dev))
+                    fused = status == 0
+                    if status not in (0, -7):   # -7: this layer's grad_X kernel has no fused add
+                        check(status, "adder_conv2d_bwd_add_f32")
+                if not fused:
+                    check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw),
+                                                   float(ctx.eta or 0.0), ptr(ws), nbytes, *ctx.dims, stream_ptr(dev)),
+                          "adder_conv2d_bwd_f32")
+                    if need_x and grad_short is not None:
+                        gx += grad_short
+        return gx, gw, None, None, None, None, None
 
 
 def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
@@ -111,13 +132,17 @@ def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
     return _adder_nchw.apply(X, W, int(stride), int(padding), eta)
 
 
-def adder2d_function_with_stats(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
+def adder2d_function_with_stats(X, W, stride=1, padding=0, eta=DEFAULT_ETA, with_shortcut=False):
     """``adder2d_function`` that also returns the BatchNorm partial sums of its output, a float64 tensor
-    (Co, slots, 2) for ``BatchNormAct2d(..., stats=)``, or None where the kernel has no such epilogue."""
+    (Co, slots, 2) for ``BatchNormAct2d(..., stats=)``, or None where the kernel has no such epilogue.
+    ``with_shortcut``: a third result, X itself as an output of the layer's autograd node; use it as the
+    residual shortcut and the shortcut's gradient is added to grad_X inside the grad_X kernel instead of
+    by a separate autograd accumulation."""
     if W.size(2) != W.size(3):
         raise RuntimeError("adder2d_function expects a square kernel")
-    out, stats = _adder_nchw.apply(X, W, int(stride), int(padding), eta, True)
-    return out, (stats if stats.numel() else None)
+    res = _adder_nchw.apply(X, W, int(stride), int(padding), eta, True, bool(with_shortcut))
+    out, stats = res[0], (res[1] if res[1].numel() else None)
+    return (out, stats, res[2]) if with_shortcut else (out, stats)
 
 
 class adder2d(nn.Module):
@@ -149,12 +174,14 @@ class adder2d(nn.Module):
             output = output + self.b.unsqueeze(0).unsqueeze(2).unsqueeze(3)
         return output
 
-    def forward_with_stats(self, x):
+    def forward_with_stats(self, x, with_shortcut=False):
         """(output, stats): ``stats`` are the BatchNorm partial sums of the output for
-        ``BatchNormAct2d.forward(..., stats=stats)``, or None (bias layers, shapes without the epilogue)."""
+        ``BatchNormAct2d.forward(..., stats=stats)``, or None (bias layers, shapes without the epilogue).
+        ``with_shortcut``: (output, stats, shortcut) with ``shortcut`` = x routed through this layer's
+        autograd node (see ``adder2d_function_with_stats``)."""
         if self.bias:
-            return self.forward(x), None
-        return adder2d_function_with_stats(x, self.adder, self.stride, self.padding, self.eta)
+            return (self.forward(x), None, x) if with_shortcut else (self.forward(x), None)
+        return adder2d_function_with_stats(x, self.adder, self.stride, self.padding, self.eta, with_shortcut)
 
     def extra_repr(self):
         return (f"{self.input_channel}, {self.output_channel}, kernel_size={self.kernel_size}, "

@@ -113,9 +113,26 @@ int adder_conv2d_bwd_workspace_bytes(int N, int Ci, int H, int W, int Co, int kh
     return ADDER_OK;
 }
 
+static int conv2d_bwd(const float *gy, const float *x, const float *w, const float *gx_add, float *gx, float *gw,
+                      float eta, void *ws, size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw,
+                      int stride, int pad, void *stream);
+
 int adder_conv2d_bwd_f32(const float *gy, const float *x, const float *w, float *gx, float *gw, float eta,
                          void *ws, size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw,
                          int stride, int pad, void *stream) {
+    return conv2d_bwd(gy, x, w, nullptr, gx, gw, eta, ws, ws_bytes, N, Ci, H, W, Co, kh, kw, stride, pad, stream);
+}
+
+int adder_conv2d_bwd_add_f32(const float *gy, const float *x, const float *w, const float *gx_add, float *gx,
+                             float *gw, float eta, void *ws, size_t ws_bytes, int N, int Ci, int H, int W, int Co,
+                             int kh, int kw, int stride, int pad, void *stream) {
+    if (!gx_add || !gx) return ADDER_ERR_NULL_POINTER;
+    return conv2d_bwd(gy, x, w, gx_add, gx, gw, eta, ws, ws_bytes, N, Ci, H, W, Co, kh, kw, stride, pad, stream);
+}
+
+static int conv2d_bwd(const float *gy, const float *x, const float *w, const float *gx_add, float *gx, float *gw,
+                      float eta, void *ws, size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw,
+                      int stride, int pad, void *stream) {
     if (!gy || !x || !w) return ADDER_ERR_NULL_POINTER;
     if (!gx && !gw) return ADDER_ERR_NULL_POINTER;
     if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
@@ -125,18 +142,18 @@ int adder_conv2d_bwd_f32(const float *gy, const float *x, const float *w, float 
                  ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo;
     if (overlaps(gx, nx, x, nx) || overlaps(gx, nx, w, nw) || overlaps(gx, nx, gy, ny) ||
         overlaps(gw, nw, x, nx) || overlaps(gw, nw, w, nw) || overlaps(gw, nw, gy, ny) ||
-        overlaps(gw, nw, gx, nx))
+        overlaps(gw, nw, gx, nx) || overlaps(gx, nx, gx_add, nx) || overlaps(gw, nw, gx_add, nx))
         return ADDER_ERR_ALIAS;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (gw) {
         const size_t need = grad_w_workspace_bytes(d);
         if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
         if (overlaps(ws, need, x, nx) || overlaps(ws, need, w, nw) || overlaps(ws, need, gy, ny) ||
-            overlaps(ws, need, gx, nx) || overlaps(ws, need, gw, nw))
+            overlaps(ws, need, gx, nx) || overlaps(ws, need, gw, nw) || overlaps(ws, need, gx_add, nx))
             return ADDER_ERR_ALIAS;
     }
     if (gx)
-        if (int rc = launch_grad_x(gy, x, w, gx, d, s)) return rc;
+        if (int rc = launch_grad_x(gy, x, w, gx, d, s, gx_add)) return rc;
     if (gw)
         if (int rc = launch_grad_w(gy, x, w, gw, eta, ws, ws_bytes, d, s)) return rc;
     return ADDER_OK;

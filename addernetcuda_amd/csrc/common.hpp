@@ -110,7 +110,7 @@ int check_launch();                  // hipGetLastError -> status
 int launch_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s);
 int fwd_stats_slots(const ConvDims &d);   // 0: no statistics epilogue for these dimensions
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
-                  hipStream_t s);
+                  hipStream_t s, const float *gadd = nullptr);
 size_t grad_w_workspace_bytes(const ConvDims &d);
 int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta,
                   void *ws, size_t ws_bytes, const ConvDims &d, hipStream_t s);

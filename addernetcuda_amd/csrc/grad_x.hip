@@ -101,7 +101,8 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
                                                                    const float *__restrict__ w,
                                                                    float *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int tilesH,
-                                                                   int tilesW, const Subsample sub) {
+                                                                   int tilesW, const Subsample sub,
+                                                                   const float *__restrict__ gadd) {
     static_assert(!SUB || C::KS == 1, "sampling is for single-tap layers");
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
@@ -307,16 +308,22 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
                     }
                     continue;
                 }
-                float *dst = gx + (((size_t)n * Ci + ci) * H + hi) * W + wi0;
+                const size_t o = (((size_t)n * Ci + ci) * H + hi) * W + wi0;
+                float *dst = gx + o;
                 if (TN % 4 == 0 && (W & 3) == 0 && wi0 + TN <= W) {
 #pragma unroll
-                    for (int t = 0; t < TN; t += 4)
-                        *reinterpret_cast<float4 *>(dst + t) =
-                            make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]);
+                    for (int t = 0; t < TN; t += 4) {
+                        float4 v = make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]);
+                        if (gadd) {   // a second gradient of the same tensor (a residual shortcut), added on the way out
+                            const float4 a = *reinterpret_cast<const float4 *>(gadd + o + t);
+                            v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+                        }
+                        *reinterpret_cast<float4 *>(dst + t) = v;
+                    }
                 } else {
 #pragma unroll
                     for (int t = 0; t < TN; ++t)
-                        if (wi0 + t < W) dst[t] = tot[m][t];
+                        if (wi0 + t < W) dst[t] = gadd ? tot[m][t] + gadd[o + t] : tot[m][t];
                 }
             }
         }
@@ -331,7 +338,8 @@ static constexpr int kSatMaxTerms = 2304;
 
 template <class C, bool VEC, bool SAT, bool SUB = false>
 static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
+                               const ConvDims &d, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0},
+                               const float *gadd = nullptr) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
@@ -345,22 +353,22 @@ static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w
         attr_set = true;
     }
     hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
-                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW, sub);
+                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW, sub, gadd);
     return check_launch();
 }
 
 template <class C>
 static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s) {
+                               const ConvDims &d, hipStream_t s, const float *gadd = nullptr) {
     // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
     const bool vec = d.W % 4 == 0;
     if constexpr (C::KS == 3) {   // (a single tap never has that many terms per output)
         if (d.Co * C::KK > kSatMaxTerms)
-            return vec ? launch_grad_x_3x3s1_v<C, true, false>(gy, x, w, gx, d, s)
-                       : launch_grad_x_3x3s1_v<C, false, false>(gy, x, w, gx, d, s);
+            return vec ? launch_grad_x_3x3s1_v<C, true, false>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd)
+                       : launch_grad_x_3x3s1_v<C, false, false>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd);
     }
-    return vec ? launch_grad_x_3x3s1_v<C, true, true>(gy, x, w, gx, d, s)
-               : launch_grad_x_3x3s1_v<C, false, true>(gy, x, w, gx, d, s);
+    return vec ? launch_grad_x_3x3s1_v<C, true, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd)
+               : launch_grad_x_3x3s1_v<C, false, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd);
 }
 
 // ---------------------------------------------------------------------------
@@ -634,15 +642,19 @@ using Gx1x1s = Tile3x3Cfg<4, 16, 1, 4, 8, 8, 16, 1, 1, 1>;    // planes of <= 64
 static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
               "the launcher checks Ci against one TM per stride");
 
+// gadd (nullable): a tensor shaped like gx that is added to the result (3x3 / stride 1 / pad 1 tiled kernels
+// only; ADDER_ERR_UNSUPPORTED elsewhere)
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
-                  hipStream_t s) {
+                  hipStream_t s, const float *gadd) {
     const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
     if (k3s1p1 && d.Ci >= GxW32::TM &&
-        (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0)) {
-        if (d.W > 16) return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s);
-        if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s);
-        return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s);
+        (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx) |
+                           reinterpret_cast<uintptr_t>(gadd)) & 15) == 0)) {
+        if (d.W > 16) return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s, gadd);
+        if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s, gadd);
+        return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s, gadd);
     }
+    if (gadd) return ADDER_ERR_UNSUPPORTED;
     if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.W % 2 == 0 && d.Ci >= GxS2W32::TM &&
         (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
         if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);

@@ -93,6 +93,17 @@ ADDER_API int adder_conv2d_bwd_f32(const float *gy, const float *x, const float 
                          int N, int Ci, int H, int W, int Co, int kh, int kw,
                          int stride, int pad, void *stream);
 
+/* adder_conv2d_bwd_f32 with gx = grad_X + gx_add.  Where the layer's input also feeds a residual
+ * shortcut (resnet20.py:28-39, out += residual) autograd adds the shortcut's gradient to grad_X in a
+ * launch of its own; here the kernel adds it on the way out.  gx_add (N, Ci, H, W) and gx must both be
+ * given and must not overlap.  ADDER_ERR_UNSUPPORTED (nothing launched) where the layer's grad_X kernel
+ * has no such epilogue: only the tiled 3x3 / stride 1 / pad 1 kernels do. */
+ADDER_API int adder_conv2d_bwd_add_f32(const float *gy, const float *x, const float *w, const float *gx_add,
+                         float *gx, float *gw, float eta,
+                         void *ws, size_t ws_bytes,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream);
+
 /* ------------------------------------------------------------------------
  * Column-matrix path: the literal signatures of the reference extension.
  *   Xcol (K, NL)   Wcol (Co, K)   out, gy (Co, NL)   gW (Co, K)   gX (K, NL)

@@ -188,3 +188,30 @@ def test_random_shapes_match_oracle(case, gpu):
     assert_close(y, c_oracle.conv2d_fwd(x, w, s, p), f"forward {case}")
     assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p), f"grad_X {case}")
     assert_close(wg.grad, c_oracle.conv2d_grad_w(gy, x, w, s, p), f"grad_W {case}")
+
+
+@pytest.mark.parametrize("case", [(3, 16, 32, 32, 16, 3, 1, 1), (2, 32, 16, 16, 32, 3, 1, 1), (5, 64, 8, 8, 64, 3, 1, 1),
+                                  (2, 9, 10, 18, 8, 3, 1, 1), (2, 16, 14, 14, 24, 1, 1, 0), (2, 6, 14, 24, 10, 3, 2, 1)],
+                         ids=str)
+def test_shortcut_gradient_is_added_to_grad_x(case, gpu):
+    """with_shortcut: x leaves the layer's autograd node a second time; what is back-propagated into that output
+    must come out added to grad_X (inside the grad_X kernel for the tiled 3x3 stride-1 layers, by a plain add
+    elsewhere), exactly as if the caller had used x itself."""
+    from addernetcuda_amd import adder
+    from oracle import c_oracle
+    s, p = case[6], case[7]
+    x, w, gy = make_case(*case)
+    gs = torch.randn(x.shape, generator=torch.Generator().manual_seed(99))
+    xg, wg = x.to(gpu).requires_grad_(True), w.to(gpu).requires_grad_(True)
+    y, stats, shortcut = adder.adder2d_function_with_stats(xg, wg, s, p, eta=0.0, with_shortcut=True)
+    assert shortcut.data_ptr() == xg.data_ptr() and torch.equal(shortcut, xg)
+    torch.autograd.backward([y, shortcut], [gy.to(gpu), gs.to(gpu)])
+    torch.cuda.synchronize()
+    assert_close(y, c_oracle.conv2d_fwd(x, w, s, p), f"forward {case}")
+    assert_close(xg.grad, c_oracle.conv2d_grad_x(gy, x, w, s, p) + gs.double(), f"grad_X + shortcut {case}")
+    assert_close(wg.grad, c_oracle.conv2d_grad_w(gy, x, w, s, p), f"grad_W {case}")
+    # only the shortcut is used downstream: its gradient passes through unchanged
+    x2 = x.to(gpu).requires_grad_(True)
+    _, _, sc2 = adder.adder2d_function_with_stats(x2, w.to(gpu), s, p, eta=0.0, with_shortcut=True)
+    sc2.backward(gs.to(gpu))
+    assert torch.equal(x2.grad.cpu(), gs)
