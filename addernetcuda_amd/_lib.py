@@ -35,6 +35,8 @@ _SIGNATURES = {
     "adder_col_gradx_f32": (_i, [_p, _p, _p, _p, _i, _l, _i, _p]),
     "adder_norm_scale_workspace_bytes": (_i, [_l, _szp]),
     "adder_grad_norm_scale_f32": (_i, [_p, _l, _f, _f, _p, _sz, _p]),
+    "adder_norm_scale_batched_workspace_bytes": (_i, [_i, _szp]),
+    "adder_grad_norm_scale_batched_f32": (_i, [_i, _p, _p, _p, _f, _p, _sz, _p]),
     "adder_bn_act_workspace_bytes": (_i, [_i, _i, _i, _szp]),
     "adder_bn_act_mask_words": (_i, [_i, _i, _i, _szp]),
     "adder_bn_act_fwd_f32": (_i, [_p] * 11 + [_f, _f, _i, _i, _i, _i, _p, _sz, _p]),

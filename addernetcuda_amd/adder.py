@@ -50,11 +50,60 @@ class adder(Function):
         return grad_W_col, grad_X_col, None
 
 
+_eta_batch = None   # while a batched_eta_scaling() block is open: the (weight, eta) pairs whose scaling is pending
+
+
+class batched_eta_scaling:
+    """``with batched_eta_scaling(): loss.backward()`` -- inside the block the adder layers leave the *raw*
+    weight gradient in ``weight.grad`` and the block's exit applies adder.py:78 to all of them in two kernel
+    launches instead of one per layer.  After the block ``.grad`` holds what it would hold without it.
+
+    It only takes over layers whose weight is a leaf with ``grad is None`` when their backward runs (the usual
+    ``zero_grad(set_to_none=True)`` loop); all others are scaled on the spot as always.  Not for code that
+    looks at weight gradients from hooks during the backward pass, nor for ``torch.autograd.grad``."""
+
+    def __enter__(self):
+        global _eta_batch
+        if _eta_batch is not None:
+            raise RuntimeError("batched_eta_scaling blocks do not nest")
+        _eta_batch = []
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        global _eta_batch
+        pending, _eta_batch = _eta_batch, None
+        if exc_type is not None:
+            return False
+        by_device = {}
+        for W, eta in pending:
+            g = W.grad
+            if g is None or g.dtype != torch.float32 or not g.is_contiguous():
+                raise RuntimeError("batched_eta_scaling: a weight's .grad is missing or not a contiguous float32 "
+                                   "tensor at the end of the block")
+            by_device.setdefault(g.device, []).append((g, eta))
+        for dev, items in by_device.items():
+            with torch.cuda.device(dev):
+                for i in range(0, len(items), 64):
+                    chunk = items[i:i + 64]
+                    count = len(chunk)
+                    ptrs = (ctypes.c_void_p * count)(*[g.data_ptr() for g, _ in chunk])
+                    sizes = (ctypes.c_long * count)(*[g.numel() for g, _ in chunk])
+                    etas = (ctypes.c_float * count)(*[float(eta) for _, eta in chunk])
+                    need = ctypes.c_size_t(0)
+                    check(lib.adder_norm_scale_batched_workspace_bytes(count, ctypes.byref(need)),
+                          "adder_norm_scale_batched_workspace_bytes")
+                    ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=dev)
+                    check(lib.adder_grad_norm_scale_batched_f32(count, ptrs, sizes, etas, 1e-12, ptr(ws), need.value,
+                                                                stream_ptr(dev)), "adder_grad_norm_scale_batched_f32")
+        return False
+
+
 class _adder_nchw(Function):
     """Fused NCHW forward / backward (replaces adder.py:22-41 + 43-80 in one step each)."""
 
     @staticmethod
     def forward(ctx, X, W, stride, padding, eta, with_stats=False, with_shortcut=False):
+        ctx.w_is_given = W.is_contiguous()   # then the saved W is the caller's own tensor (its .grad is visible)
         X, W = X.contiguous(), W.contiguous()
         require_gpu_f32(X, "X")
         require_gpu_f32(W, "W")
@@ -103,6 +152,12 @@ class _adder_nchw(Function):
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         gx = torch.empty_like(X) if need_x else None
         gw = torch.empty_like(W) if need_w else None
+        eta = float(ctx.eta or 0.0)
+        if (_eta_batch is not None and need_w and eta > 0.0 and ctx.w_is_given and W.is_leaf and W.grad is None):
+            if any(W is seen for seen, _ in _eta_batch):
+                raise RuntimeError("batched_eta_scaling: a weight that is used by two layers cannot be deferred")
+            _eta_batch.append((W, eta))   # raw gradient now, scaled with all the others when the block ends
+            eta = 0.0
         if need_x or need_w:
             with torch.cuda.device(dev):
                 ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev) if need_w else (None, 0)
@@ -110,15 +165,13 @@ class _adder_nchw(Function):
                 if need_x and grad_short is not None:
                     grad_short = grad_short.contiguous()
                     status = lib.adder_conv2d_bwd_add_f32(ptr(grad_out), ptr(X), ptr(W), ptr(grad_short), ptr(gx),
-                                                          ptr(gw), float(ctx.eta or 0.0), ptr(ws), nbytes, *ctx.dims,
-                                                          stream_ptr(dev))
+                                                          ptr(gw), eta, ptr(ws), nbytes, *ctx.dims, stream_ptr(dev))
                     fused = status == 0
                     if status not in (0, -7):   # -7: this layer's grad_X kernel has no fused add
                         check(status, "adder_conv2d_bwd_add_f32")
                 if not fused:
-                    check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw),
-                                                   float(ctx.eta or 0.0), ptr(ws), nbytes, *ctx.dims, stream_ptr(dev)),
-                          "adder_conv2d_bwd_f32")
+                    check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw), eta, ptr(ws), nbytes,
+                                                   *ctx.dims, stream_ptr(dev)), "adder_conv2d_bwd_f32")
                     if need_x and grad_short is not None:
                         gx += grad_short
         return gx, gw, None, None, None, None, None

@@ -236,6 +236,27 @@ int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps, void *ws, 
     return launch_norm_scale(g, n, eta, eps, ws, static_cast<hipStream_t>(stream));
 }
 
+int adder_norm_scale_batched_workspace_bytes(int count, size_t *bytes) {
+    if (!bytes) return ADDER_ERR_NULL_POINTER;
+    if (count <= 0 || count > ADDER_NORM_BATCH_MAX) return ADDER_ERR_BAD_SHAPE;
+    *bytes = norm_scale_batched_workspace_bytes(count);
+    return ADDER_OK;
+}
+
+int adder_grad_norm_scale_batched_f32(int count, float *const *g, const long *n, const float *eta, float eps,
+                                      void *ws, size_t ws_bytes, void *stream) {
+    if (!g || !n || !eta) return ADDER_ERR_NULL_POINTER;
+    if (count <= 0 || count > ADDER_NORM_BATCH_MAX || !(eps > 0.f)) return ADDER_ERR_BAD_SHAPE;
+    for (int t = 0; t < count; ++t) {
+        if (!g[t]) return ADDER_ERR_NULL_POINTER;
+        if (n[t] <= 0 || !(eta[t] > 0.f)) return ADDER_ERR_BAD_SHAPE;
+        if (n[t] > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    }
+    if (!ws || ws_bytes < norm_scale_batched_workspace_bytes(count) || (reinterpret_cast<uintptr_t>(ws) & 255))
+        return ADDER_ERR_WORKSPACE;
+    return launch_norm_scale_batched(count, g, n, eta, eps, ws, static_cast<hipStream_t>(stream));
+}
+
 static int check_bn(int N, int C, int HW) {
     if (N <= 0 || C <= 0 || HW <= 0) return ADDER_ERR_BAD_SHAPE;
     if ((long)N * C * HW > kMaxElems) return ADDER_ERR_TOO_LARGE;

@@ -143,6 +143,10 @@ int launch_bn_act_bwd(const float *dy, const float *y, const unsigned *mask, con
 
 size_t norm_scale_workspace_bytes(long n);
 int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);
+static constexpr int kNormBatchMax = ADDER_NORM_BATCH_MAX;
+size_t norm_scale_batched_workspace_bytes(int count);
+int launch_norm_scale_batched(int count, float *const *g, const long *n, const float *eta, float eps, void *ws,
+                              hipStream_t s);
 
 int launch_col_fwd(const float *X, const float *W, float *out, int K, long NL, int Co, hipStream_t s);
 size_t col_grad_w_workspace_bytes(int K, long NL, int Co);

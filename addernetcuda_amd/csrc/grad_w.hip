@@ -165,6 +165,73 @@ __global__ __launch_bounds__(256) void norm_scale_kernel(float *__restrict__ g, 
 
 size_t norm_scale_workspace_bytes(long) { return sizeof(double) * kNormBlocksMax; }
 
+// ---------------------------------------------------------------------------
+// The same scaling for up to kNormBatchMax tensors at once (every adder layer of a network after its
+// backward pass): two launches in all instead of one or two per layer.  grid = (P, count); block (p, t)
+// handles a slice of tensor t.  The tensor table travels by value in the kernel arguments.
+// ---------------------------------------------------------------------------
+struct NormBatch {
+    float *g[kNormBatchMax];
+    long n[kNormBatchMax];
+    float eta[kNormBatchMax];
+};
+
+__global__ __launch_bounds__(256) void batch_sumsq_kernel(const NormBatch b, double *__restrict__ ss) {
+    const int t = blockIdx.y;
+    const float *g = b.g[t];
+    const long n = b.n[t];
+    double v = 0.0;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const double e = g[i];
+        v += e * e;
+    }
+    __shared__ double red[4];
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) ss[(size_t)t * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ __launch_bounds__(256) void batch_norm_scale_kernel(const NormBatch b, const double *__restrict__ ss,
+                                                               float eps) {
+    const int t = blockIdx.y, P = gridDim.x;
+    __shared__ double red[4];
+    double v = 0.0;
+    for (int i = threadIdx.x; i < P; i += 256) v += ss[(size_t)t * P + i];
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const double total = (red[0] + red[1]) + (red[2] + red[3]);
+    float *g = b.g[t];
+    const long n = b.n[t];
+    const float eta = b.eta[t];
+    float nrm = (float)sqrt(total);   // same fp32 steps as norm_scale_kernel
+    nrm = fmaxf(nrm, eps);
+    const float rt = sqrtf((float)n);
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+        g[i] = g[i] / nrm * rt * eta;
+}
+
+static int batch_blocks(int count, const long *n) {
+    long most = 1;
+    for (int t = 0; t < count; ++t) most = n[t] > most ? n[t] : most;
+    const long p = ceil_div_l(most, 2048);   // ~8 elements per thread for the largest tensor
+    return (int)(p < 1 ? 1 : (p > 256 ? 256 : p));
+}
+
+size_t norm_scale_batched_workspace_bytes(int count) { return sizeof(double) * 256 * (size_t)count; }
+
+int launch_norm_scale_batched(int count, float *const *g, const long *n, const float *eta, float eps, void *ws,
+                              hipStream_t s) {
+    NormBatch b{};
+    for (int t = 0; t < count; ++t) { b.g[t] = g[t]; b.n[t] = n[t]; b.eta[t] = eta[t]; }
+    const int P = batch_blocks(count, n);
+    double *ss = reinterpret_cast<double *>(ws);
+    hipLaunchKernelGGL(batch_sumsq_kernel, dim3(P, count), dim3(256), 0, s, b, ss);
+    hipLaunchKernelGGL(batch_norm_scale_kernel, dim3(P, count), dim3(256), 0, s, b, ss, eps);
+    return check_launch();
+}
+
 static int norm_blocks(long n) {
     long b = ceil_div_l(n, 1024);
     return (int)(b < 1 ? 1 : (b > kNormBlocksMax ? kNormBlocksMax : b));

@@ -97,6 +97,7 @@ def evaluate(net, x_u8, y, batch):
 
 
 def train_one_epoch(net, opt, x_u8, y, batch, generator=None):
+    from addernetcuda_amd.adder import batched_eta_scaling
     net.train()
     n = x_u8.shape[0]
     perm = torch.randperm(n, device=x_u8.device, generator=generator)
@@ -108,7 +109,8 @@ def train_one_epoch(net, opt, x_u8, y, batch, generator=None):
         images = augment(normalise(x_u8[idx]), generator)
         opt.zero_grad(set_to_none=True)
         loss = F.cross_entropy(net(images), y[idx])
-        loss.backward()
+        with batched_eta_scaling():   # the adaptive scaling of all adder layers in two launches
+            loss.backward()
         opt.step()
         losses.append(loss.detach())
     return torch.stack(losses).mean().item()

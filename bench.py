@@ -175,10 +175,13 @@ def issue_probe():
 
 
 def make_step(model, opt, x, y):
+    from addernetcuda_amd.adder import batched_eta_scaling
+
     def step():
         opt.zero_grad(set_to_none=True)
         loss = torch.nn.functional.cross_entropy(model(x), y)
-        loss.backward()
+        with batched_eta_scaling():   # adder.py:78 for all adder layers in two launches after the backward pass
+            loss.backward()
         opt.step()
         return loss
     return step
@@ -208,9 +211,11 @@ def capture_step(model, opt, x, y):
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     opt.zero_grad(set_to_none=True)
+    from addernetcuda_amd.adder import batched_eta_scaling
     with torch.cuda.graph(graph):
         loss = torch.nn.functional.cross_entropy(model(x), y)
-        loss.backward()
+        with batched_eta_scaling():
+            loss.backward()
         opt.step()
     return graph, loss
 

@@ -143,6 +143,16 @@ ADDER_API int adder_norm_scale_workspace_bytes(long n, size_t *bytes);
 ADDER_API int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps,
                               void *ws, size_t ws_bytes, void *stream);
 
+/* The same scaling (adder.py:78) for `count` <= ADDER_NORM_BATCH_MAX tensors in two launches in all, for
+ * callers that take the raw gradients of all their adder layers (adder_conv2d_bwd_f32 with eta = 0) and
+ * scale them together after the backward pass.  g, n, eta are host arrays of `count` entries (device
+ * pointers, element counts, eta > 0 per tensor); each tensor is scaled by its own norm.
+ * ws must hold adder_norm_scale_batched_workspace_bytes(count) bytes. */
+#define ADDER_NORM_BATCH_MAX 64
+ADDER_API int adder_norm_scale_batched_workspace_bytes(int count, size_t *bytes);
+ADDER_API int adder_grad_norm_scale_batched_f32(int count, float *const *g, const long *n, const float *eta,
+                              float eps, void *ws, size_t ws_bytes, void *stream);
+
 /* ------------------------------------------------------------------------
  * The element-wise neighbours of every adder layer: training-mode BatchNorm2d fused with the
  * residual add and ReLU that follow it.  The reference runs these as separate PyTorch ops

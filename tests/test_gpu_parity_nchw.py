@@ -215,3 +215,42 @@ def test_shortcut_gradient_is_added_to_grad_x(case, gpu):
     _, _, sc2 = adder.adder2d_function_with_stats(x2, w.to(gpu), s, p, eta=0.0, with_shortcut=True)
     sc2.backward(gs.to(gpu))
     assert torch.equal(x2.grad.cpu(), gs)
+
+
+def test_batched_eta_scaling_leaves_the_same_gradients(gpu):
+    """Inside batched_eta_scaling() the layers leave raw weight gradients and the block's exit scales them all
+    at once: .grad afterwards must equal what the layers produce on their own, for every layer, bit for bit
+    in the norm's fp64 sum order or to rounding (two different reduction trees): compare to 1e-6 relative."""
+    from addernetcuda_amd import adder
+    shapes = [(16, 16, 3, 1, 1), (16, 32, 1, 2, 0), (32, 32, 3, 1, 1), (32, 24, 3, 2, 1), (24, 8, 5, 1, 2)]
+    g = torch.Generator().manual_seed(3)
+    x0 = torch.randn(4, 16, 16, 16, generator=g).to(gpu)
+
+    def run(batched):
+        torch.manual_seed(0)
+        layers = [adder.adder2d(ci, co, k, stride=s, padding=p, eta=0.1 * (i + 1)).to(gpu)
+                  for i, (ci, co, k, s, p) in enumerate(shapes)]
+        h = x0
+        for layer in layers:
+            h = layer(h)
+        loss = h.square().mean()
+        if batched:
+            with adder.batched_eta_scaling():
+                loss.backward()
+        else:
+            loss.backward()
+        torch.cuda.synchronize()
+        return [layer.adder.grad.clone() for layer in layers]
+
+    plain, batched = run(False), run(True)
+    for a, b, shp in zip(plain, batched, shapes):
+        assert torch.allclose(a, b, rtol=1e-6, atol=0.0), shp
+        n = a.numel()
+    # a second backward into existing .grad inside the block is scaled on the spot and accumulated, as without it
+    layer = adder.adder2d(8, 8, 3, padding=1).to(gpu)
+    xin = torch.randn(2, 8, 6, 6, generator=g).to(gpu)
+    layer(xin).sum().backward()
+    first = layer.adder.grad.clone()
+    with adder.batched_eta_scaling():
+        layer(xin).sum().backward()
+    assert torch.allclose(layer.adder.grad, 2 * first, rtol=1e-6, atol=0.0)
