@@ -35,6 +35,9 @@ _SIGNATURES = {
     "adder_col_gradx_f32": (_i, [_p, _p, _p, _p, _i, _l, _i, _p]),
     "adder_norm_scale_workspace_bytes": (_i, [_l, _szp]),
     "adder_grad_norm_scale_f32": (_i, [_p, _l, _f, _f, _p, _sz, _p]),
+    "adder_conv2d_grad_w_staged_f32": (_i, [_p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p, _p]),
+    "adder_grad_w_finish_workspace_bytes": (_i, [_i, _p, _szp]),
+    "adder_grad_w_finish_f32": (_i, [_i, _p, _p, _sz, _p]),
     "adder_norm_scale_batched_workspace_bytes": (_i, [_i, _szp]),
     "adder_grad_norm_scale_batched_f32": (_i, [_i, _p, _p, _p, _f, _p, _sz, _p]),
     "adder_bn_act_workspace_bytes": (_i, [_i, _i, _i, _szp]),
@@ -48,6 +51,13 @@ for _name, (_res, _args) in _SIGNATURES.items():
     _fn.restype, _fn.argtypes = _res, _args
 
 EXPORTED = tuple(_SIGNATURES)
+
+
+class GradWStage(ctypes.Structure):
+    """adder_grad_w_stage of include/addernet_hip.h."""
+    _fields_ = [("part", ctypes.c_void_p), ("sgpart", ctypes.c_void_p), ("w", ctypes.c_void_p),
+                ("gw", ctypes.c_void_p), ("slots", ctypes.c_int), ("Co", ctypes.c_int), ("K", ctypes.c_int),
+                ("fp64", ctypes.c_int), ("eta", ctypes.c_float)]
 
 
 def check(status, what):

@@ -14,7 +14,8 @@ import torch.nn as nn
 from torch.autograd import Function
 
 from . import adder_cuda
-from ._lib import lib, check, ptr, require_gpu_f32, same_device, stream_ptr, conv_dims, conv2d_bwd_workspace
+from ._lib import (lib, check, ptr, require_gpu_f32, same_device, stream_ptr, conv_dims, conv2d_bwd_workspace,
+                   GradWStage)
 
 DEFAULT_ETA = 0.2  # adder.py:78 divides by 5
 
@@ -50,13 +51,17 @@ class adder(Function):
         return grad_W_col, grad_X_col, None
 
 
-_eta_batch = None   # while a batched_eta_scaling() block is open: the (weight, eta) pairs whose scaling is pending
+# while a batched_eta_scaling() block is open: one entry per layer whose weight gradient is pending,
+# (weight, eta, stage, workspace) -- stage / workspace are None where only the scaling is pending
+_eta_batch = None
 
 
 class batched_eta_scaling:
-    """``with batched_eta_scaling(): loss.backward()`` -- inside the block the adder layers leave the *raw*
-    weight gradient in ``weight.grad`` and the block's exit applies adder.py:78 to all of them in two kernel
-    launches instead of one per layer.  After the block ``.grad`` holds what it would hold without it.
+    """``with batched_eta_scaling(): loss.backward()`` -- inside the block the adder layers only reduce their
+    weight gradient to partial slabs (or, for layers without such a kernel, to the raw gradient), and the block's
+    exit finishes all of them -- slab sums, ``- w * sum gy``, and the scaling of adder.py:78 -- in a few kernel
+    launches in all instead of two or three per layer.  Until then ``weight.grad`` is allocated but not
+    meaningful; after the block it holds what it would hold without it.
 
     It only takes over layers whose weight is a leaf with ``grad is None`` when their backward runs (the usual
     ``zero_grad(set_to_none=True)`` loop); all others are scaled on the spot as always.  Not for code that
@@ -74,13 +79,28 @@ class batched_eta_scaling:
         pending, _eta_batch = _eta_batch, None
         if exc_type is not None:
             return False
-        by_device = {}
-        for W, eta in pending:
+        by_device, staged = {}, {}
+        for W, eta, stage, ws in pending:
             g = W.grad
             if g is None or g.dtype != torch.float32 or not g.is_contiguous():
                 raise RuntimeError("batched_eta_scaling: a weight's .grad is missing or not a contiguous float32 "
                                    "tensor at the end of the block")
-            by_device.setdefault(g.device, []).append((g, eta))
+            if stage is None:
+                by_device.setdefault(g.device, []).append((g, eta))
+            else:
+                stage.gw = g.data_ptr()   # autograd may have handed the gradient over in another tensor
+                staged.setdefault(g.device, []).append(stage)
+        for dev, stages in staged.items():
+            with torch.cuda.device(dev):
+                for i in range(0, len(stages), 32):
+                    chunk = stages[i:i + 32]
+                    arr = (GradWStage * len(chunk))(*chunk)
+                    need = ctypes.c_size_t(0)
+                    check(lib.adder_grad_w_finish_workspace_bytes(len(chunk), arr, ctypes.byref(need)),
+                          "adder_grad_w_finish_workspace_bytes")
+                    ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=dev)
+                    check(lib.adder_grad_w_finish_f32(len(chunk), arr, ptr(ws), need.value, stream_ptr(dev)),
+                          "adder_grad_w_finish_f32")
         for dev, items in by_device.items():
             with torch.cuda.device(dev):
                 for i in range(0, len(items), 64):
@@ -153,11 +173,25 @@ class _adder_nchw(Function):
         gx = torch.empty_like(X) if need_x else None
         gw = torch.empty_like(W) if need_w else None
         eta = float(ctx.eta or 0.0)
-        if (_eta_batch is not None and need_w and eta > 0.0 and ctx.w_is_given and W.is_leaf and W.grad is None):
-            if any(W is seen for seen, _ in _eta_batch):
+        if (_eta_batch is not None and need_w and ctx.w_is_given and W.is_leaf and W.grad is None):
+            if any(W is entry[0] for entry in _eta_batch):
                 raise RuntimeError("batched_eta_scaling: a weight that is used by two layers cannot be deferred")
-            _eta_batch.append((W, eta))   # raw gradient now, scaled with all the others when the block ends
-            eta = 0.0
+            with torch.cuda.device(dev):
+                ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev)
+                stage = GradWStage()
+                status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gw), eta, ptr(ws), nbytes,
+                                                            *ctx.dims, ctypes.byref(stage), stream_ptr(dev))
+            if status == 0:      # slabs only; finished with all the others when the block ends
+                _eta_batch.append((W, eta, stage, ws))
+                need_w = False
+            elif status != -7:
+                check(status, "adder_conv2d_grad_w_staged_f32")
+            elif eta > 0.0:      # no slab kernel for this layer: raw gradient now, scaled when the block ends
+                _eta_batch.append((W, eta, None, None))
+                eta = 0.0
+        gw_out = gw
+        if not need_w:
+            gw = None
         if need_x or need_w:
             with torch.cuda.device(dev):
                 ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev) if need_w else (None, 0)
@@ -174,7 +208,7 @@ class _adder_nchw(Function):
                                                    *ctx.dims, stream_ptr(dev)), "adder_conv2d_bwd_f32")
                     if need_x and grad_short is not None:
                         gx += grad_short
-        return gx, gw, None, None, None, None, None
+        return gx, gw_out, None, None, None, None, None
 
 
 def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):

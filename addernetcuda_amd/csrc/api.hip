@@ -236,6 +236,48 @@ int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps, void *ws, 
     return launch_norm_scale(g, n, eta, eps, ws, static_cast<hipStream_t>(stream));
 }
 
+int adder_conv2d_grad_w_staged_f32(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
+                                   size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
+                                   int pad, adder_grad_w_stage *stage, void *stream) {
+    if (!gy || !x || !w || !gw || !stage) return ADDER_ERR_NULL_POINTER;
+    if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo;
+    const size_t need = grad_w_workspace_bytes(d);
+    if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
+    if (overlaps(ws, need, x, nx) || overlaps(ws, need, w, nw) || overlaps(ws, need, gy, ny) ||
+        overlaps(ws, need, gw, nw) || overlaps(gw, nw, x, nx) || overlaps(gw, nw, w, nw) || overlaps(gw, nw, gy, ny))
+        return ADDER_ERR_ALIAS;
+    return launch_grad_w_staged(gy, x, w, gw, eta, ws, ws_bytes, d, stage, static_cast<hipStream_t>(stream));
+}
+
+static int check_stages(int count, const adder_grad_w_stage *st) {
+    if (!st) return ADDER_ERR_NULL_POINTER;
+    if (count <= 0 || count > ADDER_GRAD_W_FINISH_MAX) return ADDER_ERR_BAD_SHAPE;
+    for (int t = 0; t < count; ++t) {
+        if (!st[t].part || !st[t].sgpart || !st[t].w || !st[t].gw) return ADDER_ERR_NULL_POINTER;
+        if (st[t].slots <= 0 || st[t].Co <= 0 || st[t].K <= 0 || !(st[t].eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
+        if ((long)st[t].Co * st[t].K > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    }
+    return ADDER_OK;
+}
+
+int adder_grad_w_finish_workspace_bytes(int count, const adder_grad_w_stage *stages, size_t *bytes) {
+    if (!bytes) return ADDER_ERR_NULL_POINTER;
+    if (int rc = check_stages(count, stages)) return rc;
+    *bytes = grad_w_finish_workspace_bytes(count, stages);
+    return ADDER_OK;
+}
+
+int adder_grad_w_finish_f32(int count, const adder_grad_w_stage *stages, void *ws, size_t ws_bytes, void *stream) {
+    if (int rc = check_stages(count, stages)) return rc;
+    if (!ws || ws_bytes < grad_w_finish_workspace_bytes(count, stages) || (reinterpret_cast<uintptr_t>(ws) & 255))
+        return ADDER_ERR_WORKSPACE;
+    return launch_grad_w_finish(count, stages, ws, static_cast<hipStream_t>(stream));
+}
+
 int adder_norm_scale_batched_workspace_bytes(int count, size_t *bytes) {
     if (!bytes) return ADDER_ERR_NULL_POINTER;
     if (count <= 0 || count > ADDER_NORM_BATCH_MAX) return ADDER_ERR_BAD_SHAPE;

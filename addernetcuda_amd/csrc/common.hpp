@@ -144,6 +144,11 @@ int launch_bn_act_bwd(const float *dy, const float *y, const unsigned *mask, con
 size_t norm_scale_workspace_bytes(long n);
 int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);
 static constexpr int kNormBatchMax = ADDER_NORM_BATCH_MAX;
+static constexpr int kGwFinishMax = ADDER_GRAD_W_FINISH_MAX;
+int launch_grad_w_staged(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
+                         size_t ws_bytes, const ConvDims &d, adder_grad_w_stage *stage, hipStream_t s);
+size_t grad_w_finish_workspace_bytes(int count, const adder_grad_w_stage *st);
+int launch_grad_w_finish(int count, const adder_grad_w_stage *st, void *ws, hipStream_t s);
 size_t norm_scale_batched_workspace_bytes(int count);
 int launch_norm_scale_batched(int count, float *const *g, const long *n, const float *eta, float eps, void *ws,
                               hipStream_t s);

@@ -90,15 +90,12 @@ __global__ __launch_bounds__(256) void grad_w_generic_kernel(const float *__rest
 // ---------------------------------------------------------------------------
 static constexpr int kFinOut = 16, kFinLanes = 16;   // a wave reads four full 64-byte runs per slot row
 template <typename PT>
-__global__ __launch_bounds__(kFinOut * kFinLanes) void grad_w_finalize_kernel(const PT *__restrict__ part,
-                                                                              const PT *__restrict__ sgpart,
-                                                                              const float *__restrict__ w,
-                                                                              float *__restrict__ gw,
-                                                                              double *__restrict__ ss, int slots,
-                                                                              int Co, int K) {
+__device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ part, const PT *__restrict__ sgpart,
+                                                      const float *__restrict__ w, float *__restrict__ gw,
+                                                      double *__restrict__ ss, int slots, int Co, int K, int block) {
     const int o = threadIdx.x % kFinOut, sl = threadIdx.x / kFinOut;
     const int total = Co * K;
-    const int idx = blockIdx.x * kFinOut + o;
+    const int idx = block * kFinOut + o;
     const int idc = idx < total ? idx : total - 1;
     const int co = idc / K;
     double a = 0.0, sgs = 0.0;
@@ -122,8 +119,60 @@ __global__ __launch_bounds__(kFinOut * kFinLanes) void grad_w_finalize_kernel(co
         }
 #pragma unroll
         for (int off = kFinOut / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-        if (threadIdx.x == 0 && ss) ss[blockIdx.x] = v;
+        if (threadIdx.x == 0 && ss) ss[block] = v;
     }
+}
+
+template <typename PT>
+__global__ __launch_bounds__(kFinOut * kFinLanes) void grad_w_finalize_kernel(const PT *__restrict__ part,
+                                                                              const PT *__restrict__ sgpart,
+                                                                              const float *__restrict__ w,
+                                                                              float *__restrict__ gw,
+                                                                              double *__restrict__ ss, int slots,
+                                                                              int Co, int K) {
+    grad_w_finalize_block<PT>(part, sgpart, w, gw, ss, slots, Co, K, blockIdx.x);
+}
+
+// The finalize of up to kGwFinishMax layers in one launch (grid = (most blocks of any layer, layers)) and
+// their scaling in a second: for callers that leave the partial slabs of every layer in its workspace
+// during the backward pass and finish all weight gradients together at its end.
+struct GwStageBatch {
+    adder_grad_w_stage it[kGwFinishMax];
+};
+
+__global__ __launch_bounds__(kFinOut * kFinLanes) void batch_finalize_kernel(const GwStageBatch b,
+                                                                             double *__restrict__ ss, int nbmax) {
+    const adder_grad_w_stage &it = b.it[blockIdx.y];
+    const int nb = ceil_div(it.Co * it.K, kFinOut);
+    if ((int)blockIdx.x >= nb) return;
+    double *mine = ss + (size_t)blockIdx.y * nbmax;
+    if (it.fp64)
+        grad_w_finalize_block<double>(static_cast<const double *>(it.part), static_cast<const double *>(it.sgpart), it.w,
+                                      it.gw, mine, it.slots, it.Co, it.K, blockIdx.x);
+    else
+        grad_w_finalize_block<float>(static_cast<const float *>(it.part), static_cast<const float *>(it.sgpart), it.w,
+                                     it.gw, mine, it.slots, it.Co, it.K, blockIdx.x);
+}
+
+__global__ __launch_bounds__(256) void batch_finish_scale_kernel(const GwStageBatch b, const double *__restrict__ ss,
+                                                                 int nbmax, float eps) {
+    const adder_grad_w_stage &it = b.it[blockIdx.y];
+    if (!(it.eta > 0.f)) return;   // left raw
+    const long n = (long)it.Co * it.K;
+    const int nb = ceil_div(it.Co * it.K, kFinOut);
+    __shared__ double red[4];
+    double v = 0.0;
+    for (int i = threadIdx.x; i < nb; i += 256) v += ss[(size_t)blockIdx.y * nbmax + i];
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const double total = (red[0] + red[1]) + (red[2] + red[3]);
+    float nrm = (float)sqrt(total);   // same fp32 steps as norm_scale_kernel
+    nrm = fmaxf(nrm, eps);
+    const float rt = sqrtf((float)n);
+    float *g = it.gw;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+        g[i] = g[i] / nrm * rt * it.eta;
 }
 
 // ---------------------------------------------------------------------------
@@ -330,6 +379,73 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
     if (rc) return rc;
     if (eta > 0.f) return launch_norm_scale(gw, n, eta, 1e-12f, ws, s);
     return ADDER_OK;
+}
+
+// ---- staged weight gradient: partial slabs now, finalize + scaling for many layers later --------------
+int launch_grad_w_staged(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
+                         size_t ws_bytes, const ConvDims &d, adder_grad_w_stage *stage, hipStream_t s) {
+    if (ws_bytes < grad_w_workspace_bytes(d)) return ADDER_ERR_WORKSPACE;
+    GradWPlan p = plan_grad_w(d);
+    const bool rows_1x1 = p.variant == 2 && d.kh == 1;
+    const bool need_x16 = p.variant == 2 && !(rows_1x1 && d.stride > 1) && (rows_1x1 ? d.H * d.W : d.W) % 4 == 0;
+    const bool need_g16 = p.variant == 2 && (rows_1x1 ? d.Ho * d.Wo : d.Wo) % 4 == 0;
+    if (!p.variant || (need_x16 && (reinterpret_cast<uintptr_t>(x) & 15)) ||
+        (need_g16 && (reinterpret_cast<uintptr_t>(gy) & 15)))
+        return ADDER_ERR_UNSUPPORTED;   // no slab-based kernel for this layer: nothing to stage
+    double *ss = reinterpret_cast<double *>(ws);
+    const int K = d.K();
+    int rc;
+    if (p.variant == 2) {
+        double *part = reinterpret_cast<double *>(ss + kNormBlocksMax);
+        double *sgpart = part + (size_t)p.slots * d.Co * K;
+        rc = launch_grad_w_mfma(gy, x, part, sgpart, d, p.mfma, s);
+        stage->part = part;
+        stage->sgpart = sgpart;
+    } else {
+        float *part = reinterpret_cast<float *>(ss + kNormBlocksMax);
+        float *sgpart = part + (size_t)p.slots * d.Co * K;
+        rc = launch_grad_w_1x1(gy, x, part, sgpart, p.slots, d, s);
+        stage->part = part;
+        stage->sgpart = sgpart;
+    }
+    stage->w = w;
+    stage->gw = gw;
+    stage->slots = p.slots;
+    stage->Co = d.Co;
+    stage->K = K;
+    stage->fp64 = p.variant == 2;
+    stage->eta = eta;
+    return rc;
+}
+
+static int finish_blocks(int count, const adder_grad_w_stage *st) {
+    int most = 1;
+    for (int t = 0; t < count; ++t) {
+        const int nb = ceil_div(st[t].Co * st[t].K, kFinOut);
+        most = nb > most ? nb : most;
+    }
+    return most;
+}
+
+size_t grad_w_finish_workspace_bytes(int count, const adder_grad_w_stage *st) {
+    return ((size_t)count * finish_blocks(count, st) * sizeof(double) + 255) & ~(size_t)255;
+}
+
+int launch_grad_w_finish(int count, const adder_grad_w_stage *st, void *ws, hipStream_t s) {
+    GwStageBatch b{};
+    long most_n = 1;
+    for (int t = 0; t < count; ++t) {
+        b.it[t] = st[t];
+        const long n = (long)st[t].Co * st[t].K;
+        most_n = n > most_n ? n : most_n;
+    }
+    const int nbmax = finish_blocks(count, st);
+    double *ss = reinterpret_cast<double *>(ws);
+    hipLaunchKernelGGL(batch_finalize_kernel, dim3(nbmax, count), dim3(kFinOut * kFinLanes), 0, s, b, ss, nbmax);
+    long P = ceil_div_l(most_n, 2048);
+    P = P < 1 ? 1 : (P > 256 ? 256 : P);
+    hipLaunchKernelGGL(batch_finish_scale_kernel, dim3((unsigned)P, count), dim3(256), 0, s, b, ss, nbmax, 1e-12f);
+    return check_launch();
 }
 
 }  // namespace adder

@@ -154,6 +154,36 @@ ADDER_API int adder_grad_norm_scale_batched_f32(int count, float *const *g, cons
                               float eps, void *ws, size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
+ * grad_W in two stages, for callers that finish the weight gradients of all their layers together after
+ * the backward pass (two launches in all instead of two per layer; adder.py:62-80 has no counterpart, it
+ * finishes every layer on the spot).
+ *   adder_conv2d_grad_w_staged_f32: the position reduction of grad_W into partial slabs inside ws (same size
+ *     as for adder_conv2d_bwd_f32), described by *stage; gw and eta are only recorded there.  ws and w must
+ *     stay untouched until the stage is finished.  ADDER_ERR_UNSUPPORTED (nothing launched) for layers whose
+ *     grad_W kernel has no partial slabs (kernel sizes other than 1x1 and 3x3 / pad 1).
+ *   adder_grad_w_finish_f32: for each of `count` <= ADDER_GRAD_W_FINISH_MAX stages (a host array)
+ *     gw = sum of the slabs - w * sum gy, then the scaling of adder.py:78 where eta > 0.  stage.gw may be
+ *     redirected by the caller before this call.
+ * ---------------------------------------------------------------------- */
+typedef struct adder_grad_w_stage {
+    const void *part;      /* partial slabs of sum x * gy   (inside the layer's workspace) */
+    const void *sgpart;    /* partial sums of gy per output channel */
+    const float *w;        /* the layer's weights (Co, K) */
+    float *gw;             /* where the finished gradient goes (Co, K) */
+    int slots, Co, K;      /* slabs, output channels, Ci * kh * kw */
+    int fp64;              /* slabs are double (matrix-core kernels) or float */
+    float eta;             /* 0: leave gw raw */
+} adder_grad_w_stage;
+#define ADDER_GRAD_W_FINISH_MAX 32
+ADDER_API int adder_conv2d_grad_w_staged_f32(const float *gy, const float *x, const float *w, float *gw, float eta,
+                         void *ws, size_t ws_bytes,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, adder_grad_w_stage *stage, void *stream);
+ADDER_API int adder_grad_w_finish_workspace_bytes(int count, const adder_grad_w_stage *stages, size_t *bytes);
+ADDER_API int adder_grad_w_finish_f32(int count, const adder_grad_w_stage *stages, void *ws, size_t ws_bytes,
+                         void *stream);
+
+/* ------------------------------------------------------------------------
  * The element-wise neighbours of every adder layer: training-mode BatchNorm2d fused with the
  * residual add and ReLU that follow it.  The reference runs these as separate PyTorch ops
  * (resnet20.py:28-39: bn -> relu, bn -> += residual -> relu); here each direction is one

@@ -156,3 +156,31 @@ def test_relu_mask_is_offered_for_whole_word_planes_only():
     assert lib.adder_bn_act_bwd_f32(*bwd_args, 1, 4, 8, 49, ws, 1 << 20, None) == -7
     no_y_no_mask = [fake, None, None] + [fake] * 8
     assert lib.adder_bn_act_bwd_f32(*no_y_no_mask, 1, 4, 8, 64, ws, 1 << 20, None) == -1
+
+
+def test_staged_grad_w_and_batched_scaling_validate_without_a_gpu():
+    """The entry points that finish many layers at once refuse bad arguments before any HIP call."""
+    from addernetcuda_amd._lib import lib, GradWStage
+    fake = ctypes.c_void_p(1 << 20)
+    need = ctypes.c_size_t(0)
+    # batched scaling
+    assert lib.adder_norm_scale_batched_workspace_bytes(20, ctypes.byref(need)) == 0 and need.value > 0
+    assert lib.adder_norm_scale_batched_workspace_bytes(65, ctypes.byref(need)) == -2
+    ptrs = (ctypes.c_void_p * 2)(4096, 8192)
+    sizes = (ctypes.c_long * 2)(100, 0)
+    etas = (ctypes.c_float * 2)(0.1, 0.1)
+    assert lib.adder_grad_norm_scale_batched_f32(2, ptrs, sizes, etas, 1e-12, fake, 1 << 20, None) == -2   # n = 0
+    assert lib.adder_grad_norm_scale_batched_f32(2, None, sizes, etas, 1e-12, fake, 1 << 20, None) == -1
+    # staged grad_W
+    stage = GradWStage()
+    dims = (4, 16, 8, 8, 16, 3, 3, 1, 1)
+    assert lib.adder_conv2d_grad_w_staged_f32(fake, fake, fake, None, 0.1, fake, 1 << 30, *dims, ctypes.byref(stage),
+                                              None) == -1
+    assert lib.adder_conv2d_grad_w_staged_f32(fake, fake, fake, ctypes.c_void_p(1 << 40), 0.1, fake, 16, *dims,
+                                              ctypes.byref(stage), None) == -4                              # workspace
+    stages = (GradWStage * 1)(GradWStage(4096, 4096, 4096, 4096, 0, 16, 144, 1, 0.1))
+    assert lib.adder_grad_w_finish_workspace_bytes(1, stages, ctypes.byref(need)) == -2                    # slots = 0
+    stages[0].slots = 8
+    assert lib.adder_grad_w_finish_workspace_bytes(1, stages, ctypes.byref(need)) == 0 and need.value >= 144 * 8
+    assert lib.adder_grad_w_finish_f32(33, stages, fake, 1 << 20, None) == -2
+    assert lib.adder_grad_w_finish_f32(1, stages, fake, 16, None) == -4
