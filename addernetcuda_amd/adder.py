@@ -211,6 +211,37 @@ class _adder_nchw(Function):
         return gx, gw_out, None, None, None, None, None
 
 
+def conv2d_weight_grad(grad_out, X, W, stride, padding):
+    """Weight gradient of an *ordinary* convolution ``F.conv2d(X, W, None, stride, padding)``, i.e. the
+    ``sum x * gy`` half of the adder layer's weight gradient, from the same fp64 matrix-core kernel (the slab
+    finalize leaves the ``- w * sum gy`` term out).  Inside a ``batched_eta_scaling()`` block it is finished
+    together with the adder layers' gradients.  Returns None where the geometry has no such kernel."""
+    grad_out, X = grad_out.contiguous(), X.contiguous()
+    require_gpu_f32(grad_out, "grad_output")
+    require_gpu_f32(X, "X")
+    dev = X.device
+    dims, _, _ = conv_dims(X.shape, W.shape, stride, padding)
+    gw = torch.empty(W.shape, device=dev, dtype=torch.float32)
+    with torch.cuda.device(dev):
+        ws, nbytes = conv2d_bwd_workspace(dims, dev)
+        stage = GradWStage()
+        status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), None, ptr(gw), 0.0, ptr(ws), nbytes, *dims,
+                                                    ctypes.byref(stage), stream_ptr(dev))
+        if status == -7:
+            return None
+        check(status, "adder_conv2d_grad_w_staged_f32")
+        if (_eta_batch is not None and W.is_leaf and W.grad is None and W.is_contiguous()
+                and not any(W is entry[0] for entry in _eta_batch)):
+            _eta_batch.append((W, 0.0, stage, ws))
+            return gw
+        arr = (GradWStage * 1)(stage)
+        need = ctypes.c_size_t(0)
+        check(lib.adder_grad_w_finish_workspace_bytes(1, arr, ctypes.byref(need)), "adder_grad_w_finish_workspace_bytes")
+        fws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=dev)
+        check(lib.adder_grad_w_finish_f32(1, arr, ptr(fws), need.value, stream_ptr(dev)), "adder_grad_w_finish_f32")
+    return gw
+
+
 def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
     """Same call as adder.py:22; ``eta`` (default 0.2 = the reference's /5) is the only addition."""
     if W.size(2) != W.size(3):

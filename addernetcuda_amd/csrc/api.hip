@@ -239,7 +239,7 @@ int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps, void *ws, 
 int adder_conv2d_grad_w_staged_f32(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
                                    size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
                                    int pad, adder_grad_w_stage *stage, void *stream) {
-    if (!gy || !x || !w || !gw || !stage) return ADDER_ERR_NULL_POINTER;
+    if (!gy || !x || !gw || !stage) return ADDER_ERR_NULL_POINTER;
     if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
     ConvDims d;
     if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
@@ -257,7 +257,7 @@ static int check_stages(int count, const adder_grad_w_stage *st) {
     if (!st) return ADDER_ERR_NULL_POINTER;
     if (count <= 0 || count > ADDER_GRAD_W_FINISH_MAX) return ADDER_ERR_BAD_SHAPE;
     for (int t = 0; t < count; ++t) {
-        if (!st[t].part || !st[t].sgpart || !st[t].w || !st[t].gw) return ADDER_ERR_NULL_POINTER;
+        if (!st[t].part || !st[t].sgpart || !st[t].gw) return ADDER_ERR_NULL_POINTER;
         if (st[t].slots <= 0 || st[t].Co <= 0 || st[t].K <= 0 || !(st[t].eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
         if ((long)st[t].Co * st[t].K > kMaxElems) return ADDER_ERR_TOO_LARGE;
     }

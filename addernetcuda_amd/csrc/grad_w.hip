@@ -113,7 +113,7 @@ __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ par
         for (int k = 0; k < kFinLanes; ++k) { ta += ra[k][o]; ts += rs[k][o]; }
         double v = 0.0;
         if (idx < total) {
-            const float r = (float)(ta - (double)w[idx] * ts);
+            const float r = (float)(w ? ta - (double)w[idx] * ts : ta);   // no weights: the plain sum of x * gy
             gw[idx] = r;
             v = (double)r * (double)r;
         }

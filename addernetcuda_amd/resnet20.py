@@ -15,7 +15,9 @@ The BatchNorm layers are ``BatchNormAct2d``: the same module as nn.BatchNorm2d
 (parameters, buffers, state_dict keys) with the ReLU, and in the second half
 of a block the residual add, folded into its GPU kernels.
 """
+import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import adder as _adder
 from .bn_act import BatchNormAct2d
@@ -56,13 +58,52 @@ class BasicBlock(nn.Module):
         return self._conv_bn(self.conv2, self.bn2, out, shortcut)       # bn + residual + relu
 
 
+class _conv2d_matrix_grad(torch.autograd.Function):
+    """An ordinary convolution whose weight gradient comes from the adder library's matrix-core kernel."""
+
+    @staticmethod
+    def forward(ctx, x, w, stride, padding):
+        ctx.save_for_backward(x, w)
+        ctx.conf = (stride, padding)
+        return F.conv2d(x, w, None, stride, padding)
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, w = ctx.saved_tensors
+        stride, padding = ctx.conf
+        gx = gw = None
+        if ctx.needs_input_grad[0]:
+            gx = torch.nn.grad.conv2d_input(x.shape, w, gy, stride, padding)
+        if ctx.needs_input_grad[1]:
+            gw = _adder.conv2d_weight_grad(gy, x, w, stride, padding)
+            if gw is None:
+                gw = torch.nn.grad.conv2d_weight(x, w.shape, gy, stride, padding)
+        return gx, gw, None, None
+
+
+class StemConv2d(nn.Conv2d):
+    """``nn.Conv2d`` (resnet20.py:49) with the same parameters and state_dict; on the GPU in training its
+    weight gradient -- a sum over N*H*W positions into 16 x 27 values, which the vendor library spends six
+    launches and three layout changes on -- runs through the kernel that does the same reduction for the
+    adder layers."""
+
+    def forward(self, x):
+        plain = (x.is_cuda and x.dtype == torch.float32 and self.bias is None and self.groups == 1
+                 and self.dilation == (1, 1) and self.padding_mode == "zeros" and torch.is_grad_enabled()
+                 and self.stride[0] == self.stride[1] and self.padding[0] == self.padding[1]
+                 and isinstance(self.padding[0], int))
+        if not plain:
+            return super().forward(x)
+        return _conv2d_matrix_grad.apply(x, self.weight, self.stride[0], self.padding[0])
+
+
 class ResNet(nn.Module):
     def __init__(self, block, layers, num_classes=10, adder2d_cls=None, **adder_kw):
         super().__init__()
         self._make = adder2d_cls or _adder.adder2d
         self._adder_kw = adder_kw
         self.inplanes = 16
-        self.conv1 = nn.Conv2d(3, 16, kernel_size=3, stride=1, padding=1, bias=False)
+        self.conv1 = StemConv2d(3, 16, kernel_size=3, stride=1, padding=1, bias=False)
         self.bn1 = BatchNormAct2d(16, relu=True)
         self.relu = nn.ReLU(inplace=True)
         self.layer1 = self._make_layer(block, 16, layers[0])

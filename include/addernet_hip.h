@@ -161,6 +161,8 @@ ADDER_API int adder_grad_norm_scale_batched_f32(int count, float *const *g, cons
  *     as for adder_conv2d_bwd_f32), described by *stage; gw and eta are only recorded there.  ws and w must
  *     stay untouched until the stage is finished.  ADDER_ERR_UNSUPPORTED (nothing launched) for layers whose
  *     grad_W kernel has no partial slabs (kernel sizes other than 1x1 and 3x3 / pad 1).
+ *     w == NULL: the stage finishes to the plain sum of x * gy, which is the weight gradient of an ordinary
+ *     convolution of the same geometry (the stem of resnet20.py:49 runs through the same kernel that way).
  *   adder_grad_w_finish_f32: for each of `count` <= ADDER_GRAD_W_FINISH_MAX stages (a host array)
  *     gw = sum of the slabs - w * sum gy, then the scaling of adder.py:78 where eta > 0.  stage.gw may be
  *     redirected by the caller before this call.
@@ -168,7 +170,7 @@ ADDER_API int adder_grad_norm_scale_batched_f32(int count, float *const *g, cons
 typedef struct adder_grad_w_stage {
     const void *part;      /* partial slabs of sum x * gy   (inside the layer's workspace) */
     const void *sgpart;    /* partial sums of gy per output channel */
-    const float *w;        /* the layer's weights (Co, K) */
+    const float *w;        /* the layer's weights (Co, K), or NULL (see above) */
     float *gw;             /* where the finished gradient goes (Co, K) */
     int slots, Co, K;      /* slabs, output channels, Ci * kh * kw */
     int fp64;              /* slabs are double (matrix-core kernels) or float */

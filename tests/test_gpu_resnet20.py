@@ -116,3 +116,36 @@ def test_state_dict_round_trip_and_eval_forward(gpu):
     x = torch.randn(8, 3, 32, 32, device=gpu)
     with torch.no_grad():
         assert torch.equal(a(x), b(x))
+
+
+def test_stem_convolution_weight_gradient_matches_torch(gpu):
+    """StemConv2d: an ordinary convolution; its weight gradient comes from the adder library's matrix-core
+    kernel (sum x * gy, no weight term) and must be the float64 gradient of F.conv2d to the parity bar, alone
+    and inside a batched_eta_scaling() block; its input gradient and its state_dict are nn.Conv2d's."""
+    from addernetcuda_amd import adder
+    from addernetcuda_amd.resnet20 import StemConv2d
+    from tests.util import assert_close
+    g = torch.Generator().manual_seed(11)
+    for shape, co, stride in (((6, 3, 32, 32), 16, 1), ((3, 5, 14, 10), 7, 1), ((4, 8, 16, 16), 12, 2)):
+        x = torch.randn(shape, generator=g)
+        gy_shape = None
+        conv = StemConv2d(shape[1], co, 3, stride=stride, padding=1, bias=False).to(gpu)
+        assert list(conv.state_dict()) == ["weight"]
+        w = conv.weight.detach().cpu()
+        xd = x.double().requires_grad_(True)
+        wd = w.double().requires_grad_(True)
+        yd = torch.nn.functional.conv2d(xd, wd, None, stride, 1)
+        gy = torch.randn(yd.shape, generator=g)
+        yd.backward(gy.double())
+        for batched in (False, True):
+            conv.weight.grad = None
+            xg = x.to(gpu).requires_grad_(True)
+            y = conv(xg)
+            if batched:
+                with adder.batched_eta_scaling():
+                    y.backward(gy.to(gpu))
+            else:
+                y.backward(gy.to(gpu))
+            torch.cuda.synchronize()
+            assert_close(conv.weight.grad, wd.grad, f"stem grad_W {shape} batched={batched}", rtol=1e-5, atol=1e-4)
+            assert_close(xg.grad, xd.grad, f"stem grad_X {shape}", rtol=1e-4, atol=1e-4)
