@@ -123,7 +123,8 @@ int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sg
 
 // 1x1 / pad 0 / stride 1-2 kernels (conv1x1.hip)
 bool conv1x1_supported(const ConvDims &d, const void *a, const void *b);
-int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s);
+int fwd_1x1_stats_slots(const ConvDims &d);
+int launch_fwd_1x1(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s);
 int launch_grad_x_1x1(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                       hipStream_t s);
 int grad_w_1x1_slots(const ConvDims &d);

@@ -73,8 +73,8 @@ __device__ __forceinline__ void st2(float *p, const float2 v, int valid) {
 
 template <int S, int TM, bool VEC = true>
 __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ x, const float *__restrict__ w,
-                                                      float *__restrict__ y, int N, int Ci, int H, int W,
-                                                      int Co, int Ho, int Wo, int gpr, int groups) {
+                                                      float *__restrict__ y, double *__restrict__ stats, int N, int Ci,
+                                                      int H, int W, int Co, int Ho, int Wo, int gpr, int groups) {
     constexpr int TN = 4 / S;
     const Lane1x1<S> L(blockIdx.x * 256 + threadIdx.x, groups, gpr, Ho);
     const int co0 = blockIdx.y * TM;
@@ -128,6 +128,32 @@ __global__ __launch_bounds__(256) void fwd_1x1_kernel(const float *__restrict__ 
     for (int m = 0; m < TM; ++m)
 #pragma unroll
         for (int t = 0; t < TN; ++t) tot[m][t] += acc[m][t];
+    if (stats) {
+        // BatchNorm statistics of the output on the way out, as in the tiled forward kernels: per wave and output
+        // channel the sums of y and y*y over the wave's valid outputs (deviations from a pivot in fp32, moved
+        // back to the origin in fp64), slot = wave of this launch
+        const int lane = threadIdx.x & 63;
+        const int slots = gridDim.x * 4, slot = blockIdx.x * 4 + (threadIdx.x >> 6);
+        const int nvalid = L.ok ? min(TN, Wo - L.wo0) : 0;
+        const double count = (double)wave_sum_dpp((float)nvalid);
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const float pivot = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(tot[m][0])));
+            float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int t = 0; t < TN; ++t)
+                if (t < nvalid) {
+                    const float dv = tot[m][t] - pivot;
+                    s1 += dv;
+                    s2 = fmaf(dv, dv, s2);
+                }
+            const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2), c = (double)pivot;
+            if (lane == 0 && co0 + m < Co) {
+                stats[((size_t)(co0 + m) * slots + slot) * 2] = d1 + count * c;
+                stats[((size_t)(co0 + m) * slots + slot) * 2 + 1] = d2 + 2.0 * c * d1 + count * c * c;
+            }
+        }
+    }
     if (L.ok) {
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
@@ -348,23 +374,32 @@ static void lane_space(const ConvDims &f, int &gpr, int &groups) {
     groups = f.N * f.Ho * gpr;
 }
 
-int launch_fwd_1x1(const float *x, const float *w, float *y, const ConvDims &d, hipStream_t s) {
+// partial-sum slots per channel of the statistics epilogue (one per wave of the launch)
+int fwd_1x1_stats_slots(const ConvDims &d) {
+    const ConvDims f = lane_dims(d);
+    int gpr, groups;
+    lane_space(f, gpr, groups);
+    return ceil_div(groups, 256) * 4;
+}
+
+// stats (nullable): per-channel partial sums of y and y*y, fwd_1x1_stats_slots(d) slots per channel
+int launch_fwd_1x1(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s) {
     constexpr int TM = 8;
     const ConvDims f = lane_dims(d);
     int gpr, groups;
     lane_space(f, gpr, groups);
     const dim3 grid(ceil_div(groups, 256), ceil_div(f.Co, TM));
     if (f.stride == 2 && vec_ok(f, x, y, nullptr))
-        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM, true>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM, true>), grid, dim3(256), 0, s, x, w, y, stats, f.N, f.Ci, f.H, f.W, f.Co,
                            f.Ho, f.Wo, gpr, groups);
     else if (f.stride == 2)
-        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM, false>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+        hipLaunchKernelGGL((fwd_1x1_kernel<2, TM, false>), grid, dim3(256), 0, s, x, w, y, stats, f.N, f.Ci, f.H, f.W, f.Co,
                            f.Ho, f.Wo, gpr, groups);
     else if (vec_ok(f, x, y, nullptr))
-        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM, true>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM, true>), grid, dim3(256), 0, s, x, w, y, stats, f.N, f.Ci, f.H, f.W, f.Co,
                            f.Ho, f.Wo, gpr, groups);
     else
-        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM, false>), grid, dim3(256), 0, s, x, w, y, f.N, f.Ci, f.H, f.W, f.Co,
+        hipLaunchKernelGGL((fwd_1x1_kernel<1, TM, false>), grid, dim3(256), 0, s, x, w, y, stats, f.N, f.Ci, f.H, f.W, f.Co,
                            f.Ho, f.Wo, gpr, groups);
     return check_launch();
 }

@@ -347,7 +347,7 @@ int fwd_stats_slots(const ConvDims &d) {
         case 7: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
         case 8: return stats_slots_3x3<Fwd1x1>(as_one_row(d));
         case 9: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
-        default: return 0;
+        default: return conv1x1_supported(d, nullptr, nullptr) ? fwd_1x1_stats_slots(d) : 0;
     }
 }
 
@@ -379,8 +379,12 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
             default: break;
         }
     }
-    if (stats) return ADDER_ERR_UNSUPPORTED;   // only the tiled kernels have the statistics epilogue
-    if (conv1x1_supported(d, x, y)) return launch_fwd_1x1(x, w, y, d, s);
+    if (conv1x1_supported(d, x, y)) {
+        // (a tiled variant that was turned down for its alignment counted its statistics slots differently)
+        if (stats && variant != 0) return ADDER_ERR_UNSUPPORTED;
+        return launch_fwd_1x1(x, w, y, stats, d, s);
+    }
+    if (stats) return ADDER_ERR_UNSUPPORTED;   // the generic kernel has no statistics epilogue
     constexpr int TM = 8;
     const long total = (long)d.N * d.Ho * d.Wo;
     hipLaunchKernelGGL(fwd_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Co, TM)),

@@ -402,7 +402,8 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
                                                                    const float *__restrict__ w,
                                                                    float *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int Ho, int Wo,
-                                                                   int tilesH, int tilesW) {
+                                                                   int tilesH, int tilesW,
+                                                                   const float *__restrict__ gadd) {
     constexpr int TNW = C::TNW, TM = C::TM, GSTRIP = C::GSTRIP;
     extern __shared__ __align__(16) float smem[];
 
@@ -585,15 +586,22 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
             for (int rp = 0; rp < 2; ++rp) {
                 const int hi = hi0 + rp;
                 if (hi >= H) continue;
-                float *dst = gx + (((size_t)n * Ci + ci) * H + hi) * W + wi0;
+                const size_t o = (((size_t)n * Ci + ci) * H + hi) * W + wi0;
+                float *dst = gx + o;
                 if ((W & 1) == 0 && wi0 + TNW <= W) {
 #pragma unroll
-                    for (int t = 0; t < TNW; t += 2)
-                        *reinterpret_cast<float2 *>(dst + t) = make_float2(tot[m][rp][t], tot[m][rp][t + 1]);
+                    for (int t = 0; t < TNW; t += 2) {
+                        float2 v = make_float2(tot[m][rp][t], tot[m][rp][t + 1]);
+                        if (gadd) {   // a second gradient of the same tensor, added on the way out
+                            const float2 a = *reinterpret_cast<const float2 *>(gadd + o + t);
+                            v.x += a.x; v.y += a.y;
+                        }
+                        *reinterpret_cast<float2 *>(dst + t) = v;
+                    }
                 } else {
 #pragma unroll
                     for (int t = 0; t < TNW; ++t)
-                        if (wi0 + t < W) dst[t] = tot[m][rp][t];
+                        if (wi0 + t < W) dst[t] = gadd ? tot[m][rp][t] + gadd[o + t] : tot[m][rp][t];
                 }
             }
         }
@@ -602,7 +610,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 
 template <class C, bool VEC, bool SAT>
 static int launch_grad_x_3x3s2_v(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s) {
+                               const ConvDims &d, hipStream_t s, const float *gadd) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
@@ -610,20 +618,20 @@ static int launch_grad_x_3x3s2_v(const float *gy, const float *x, const float *w
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
     hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
-                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW);
+                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, gadd);
     return check_launch();
 }
 
 template <class C>
 static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s) {
+                               const ConvDims &d, hipStream_t s, const float *gadd) {
     // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
     const bool vec = d.Wo % 4 == 0;
     if (d.Co * 4 > kSatMaxTerms)   // an input position meets at most four of the nine taps per output channel
-        return vec ? launch_grad_x_3x3s2_v<C, true, false>(gy, x, w, gx, d, s)
-                   : launch_grad_x_3x3s2_v<C, false, false>(gy, x, w, gx, d, s);
-    return vec ? launch_grad_x_3x3s2_v<C, true, true>(gy, x, w, gx, d, s)
-               : launch_grad_x_3x3s2_v<C, false, true>(gy, x, w, gx, d, s);
+        return vec ? launch_grad_x_3x3s2_v<C, true, false>(gy, x, w, gx, d, s, gadd)
+                   : launch_grad_x_3x3s2_v<C, false, false>(gy, x, w, gx, d, s, gadd);
+    return vec ? launch_grad_x_3x3s2_v<C, true, true>(gy, x, w, gx, d, s, gadd)
+               : launch_grad_x_3x3s2_v<C, false, true>(gy, x, w, gx, d, s, gadd);
 }
 
 //                              TNW BPR TH NIMG TM CIW CC
@@ -642,8 +650,8 @@ using Gx1x1s = Tile3x3Cfg<4, 16, 1, 4, 8, 8, 16, 1, 1, 1>;    // planes of <= 64
 static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
               "the launcher checks Ci against one TM per stride");
 
-// gadd (nullable): a tensor shaped like gx that is added to the result (3x3 / stride 1 / pad 1 tiled kernels
-// only; ADDER_ERR_UNSUPPORTED elsewhere)
+// gadd (nullable): a tensor shaped like gx that is added to the result (tiled 3x3 / pad 1 kernels only;
+// ADDER_ERR_UNSUPPORTED elsewhere)
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s, const float *gadd) {
     const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
@@ -654,12 +662,13 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s, gadd);
         return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s, gadd);
     }
-    if (gadd) return ADDER_ERR_UNSUPPORTED;
     if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.W % 2 == 0 && d.Ci >= GxS2W32::TM &&
-        (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0) {
-        if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s);
-        return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s);
+        (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) &&
+        ((reinterpret_cast<uintptr_t>(gx) | reinterpret_cast<uintptr_t>(gadd)) & 7) == 0) {
+        if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s, gadd);
+        return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s, gadd);
     }
+    if (gadd) return ADDER_ERR_UNSUPPORTED;
     if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 64) {
         ConvDims f = d;   // every (H, W) plane as one row of H*W positions
         f.H = f.Ho = 1;

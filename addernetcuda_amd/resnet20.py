@@ -46,12 +46,18 @@ class BasicBlock(nn.Module):
         return bn(conv(x), residual=residual)
 
     def forward(self, x):
-        if (self.downsample is None and self.bn1.training and x.is_cuda and x.requires_grad
-                and hasattr(self.conv1, "forward_with_stats")):
-            # identity shortcut: x leaves conv1's autograd node a second time, so that the shortcut's gradient
-            # is added to conv1's input gradient by the kernel that computes it, not by a launch of its own
+        if self.bn1.training and x.is_cuda and x.requires_grad and hasattr(self.conv1, "forward_with_stats"):
+            # x leaves conv1's autograd node a second time and feeds the shortcut from there, so that the
+            # shortcut's gradient is added to conv1's input gradient by the kernel that computes it, not by
+            # a launch of its own
             out, stats, shortcut = self.conv1.forward_with_stats(x, with_shortcut=True)
             out = self.bn1(out, stats=stats)
+            if self.downsample is not None:
+                ds = self.downsample
+                if isinstance(ds, nn.Sequential) and len(ds) == 2 and isinstance(ds[1], BatchNormAct2d):
+                    shortcut = self._conv_bn(ds[0], ds[1], shortcut)   # statistics from the 1x1 kernel's epilogue
+                else:
+                    shortcut = ds(shortcut)
             return self._conv_bn(self.conv2, self.bn2, out, shortcut)
         out = self._conv_bn(self.conv1, self.bn1, x)                    # bn + relu
         shortcut = x if self.downsample is None else self.downsample(x)

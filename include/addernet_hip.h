@@ -97,7 +97,7 @@ ADDER_API int adder_conv2d_bwd_f32(const float *gy, const float *x, const float 
  * shortcut (resnet20.py:28-39, out += residual) autograd adds the shortcut's gradient to grad_X in a
  * launch of its own; here the kernel adds it on the way out.  gx_add (N, Ci, H, W) and gx must both be
  * given and must not overlap.  ADDER_ERR_UNSUPPORTED (nothing launched) where the layer's grad_X kernel
- * has no such epilogue: only the tiled 3x3 / stride 1 / pad 1 kernels do. */
+ * has no such epilogue: only the tiled 3x3 / pad 1 kernels (stride 1 or 2) do. */
 ADDER_API int adder_conv2d_bwd_add_f32(const float *gy, const float *x, const float *w, const float *gx_add,
                          float *gx, float *gw, float eta,
                          void *ws, size_t ws_bytes,

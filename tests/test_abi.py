@@ -122,7 +122,10 @@ def test_statistics_variants_validate_without_a_gpu():
     n32 = slots.value
     assert lib.adder_conv2d_fwd_stats_slots(128, 16, 32, 32, 16, 3, 3, 1, 1, ctypes.byref(slots)) == 0
     assert slots.value * 2 == n32                                  # slots follow the number of position waves
-    for k, s, p in ((1, 1, 0), (1, 2, 0), (5, 1, 2), (3, 3, 1)):
+    for k, s, p in ((1, 1, 0), (1, 2, 0)):
+        assert lib.adder_conv2d_fwd_stats_slots(4, 8, 16, 16, 8, k, k, s, p, ctypes.byref(slots)) == 0
+        assert slots.value > 0                                     # the 1x1 kernels have the epilogue too
+    for k, s, p in ((5, 1, 2), (3, 3, 1), (1, 3, 0)):
         assert lib.adder_conv2d_fwd_stats_slots(4, 8, 16, 16, 8, k, k, s, p, ctypes.byref(slots)) == 0
         assert slots.value == 0                                    # no statistics epilogue for these kernels
     assert lib.adder_conv2d_fwd_stats_slots(*dims32, None) == -1
@@ -131,7 +134,7 @@ def test_statistics_variants_validate_without_a_gpu():
     assert lib.adder_conv2d_fwd_stats_f32(fake, fake, ctypes.c_void_p(1 << 40), ctypes.c_void_p(1 << 41), n32 + 1,
                                           *dims32, None) == -2     # slot count must be the one reported
     assert lib.adder_conv2d_fwd_stats_f32(fake, fake, ctypes.c_void_p(1 << 40), ctypes.c_void_p(1 << 41), 4,
-                                          4, 8, 16, 16, 8, 1, 1, 1, 0, None) == -7
+                                          4, 8, 16, 16, 8, 5, 5, 1, 2, None) == -7
     bn = lib.adder_bn_act_fwd_stats_f32
     args = [fake] * 5 + [None] + [fake] * 5 + [0.1, 1e-5, 1, 4, 8, 64]
     assert bn(*args, None, 4, None) == -1

@@ -78,6 +78,8 @@ STATS_CASES = [
     (3, 16, 32, 32, 16, 3, 1, 1), (2, 32, 16, 16, 32, 3, 1, 1), (5, 64, 8, 8, 64, 3, 1, 1),
     (2, 5, 12, 20, 7, 3, 1, 1), (2, 16, 32, 32, 32, 3, 2, 1), (3, 32, 16, 16, 64, 3, 2, 1),
     (2, 16, 14, 14, 20, 3, 1, 1), (2, 9, 10, 18, 8, 3, 1, 1),
+    (2, 16, 32, 32, 32, 1, 2, 0), (3, 32, 16, 16, 64, 1, 2, 0), (2, 8, 8, 8, 4, 1, 1, 0), (3, 12, 7, 7, 20, 1, 1, 0),
+    (2, 6, 9, 9, 10, 1, 2, 0), (3, 64, 14, 14, 72, 1, 1, 0), (2, 64, 28, 28, 72, 1, 2, 0),   # 1x1 kernels, element-wise and tiled
 ]
 
 
@@ -104,7 +106,7 @@ def test_forward_statistics_epilogue_sums_the_output(case, gpu):
 def test_layers_without_the_epilogue_report_none(gpu):
     from addernetcuda_amd import adder
     x = torch.randn(2, 8, 8, 8, device=gpu)
-    for k, s, p in ((1, 1, 0), (1, 2, 0), (5, 1, 2)):
+    for k, s, p in ((5, 1, 2), (1, 3, 0), (3, 1, 0)):
         w = torch.randn(4, 8, k, k, device=gpu)
         y, stats = adder.adder2d_function_with_stats(x, w, s, p)
         assert stats is None and torch.equal(y, adder.adder2d_function(x, w, s, p))
