@@ -25,6 +25,7 @@ _SIGNATURES = {
     "adder_conv2d_fwd_f32": (_i, [_p, _p, _p] + [_i] * 9 + [_p]),
     "adder_conv2d_fwd_stats_slots": (_i, [_i] * 9 + [ctypes.POINTER(ctypes.c_int)]),
     "adder_conv2d_fwd_stats_f32": (_i, [_p, _p, _p, _p, _i] + [_i] * 9 + [_p]),
+    "adder_plain_conv2d_fwd_f32": (_i, [_p, _p, _p, _p, _i] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_workspace_bytes": (_i, [_i] * 9 + [_szp]),
     "adder_conv2d_bwd_f32": (_i, [_p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_add_f32": (_i, [_p, _p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),

@@ -211,6 +211,26 @@ class _adder_nchw(Function):
         return gx, gw_out, None, None, None, None, None
 
 
+def plain_conv2d_forward(X, W, stride, padding):
+    """An *ordinary* convolution ``F.conv2d(X, W, None, stride, padding)`` through the adder forward's tiled
+    kernel (3x3 / stride 1 / pad 1), with the BatchNorm partial sums of its output: (y, stats), or (None, None)
+    where the geometry has no such kernel."""
+    require_gpu_f32(X, "X")
+    require_gpu_f32(W, "W")
+    dev = same_device(X, W)
+    dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
+    with torch.cuda.device(dev):
+        slots = ctypes.c_int(0)
+        check(lib.adder_conv2d_fwd_stats_slots(*dims, ctypes.byref(slots)), "adder_conv2d_fwd_stats_slots")
+        y = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
+        stats = torch.empty((W.size(0), slots.value, 2), device=dev, dtype=torch.float64) if slots.value else None
+        status = lib.adder_plain_conv2d_fwd_f32(ptr(X), ptr(W), ptr(y), ptr(stats), slots.value, *dims, stream_ptr(dev))
+    if status == -7:
+        return None, None
+    check(status, "adder_plain_conv2d_fwd_f32")
+    return y, stats
+
+
 def conv2d_weight_grad(grad_out, X, W, stride, padding):
     """Weight gradient of an *ordinary* convolution ``F.conv2d(X, W, None, stride, padding)``, i.e. the
     ``sum x * gy`` half of the adder layer's weight gradient, from the same fp64 matrix-core kernel (the slab

@@ -104,6 +104,25 @@ int adder_conv2d_fwd_stats_f32(const float *x, const float *w, float *y, double 
     return launch_fwd(x, w, y, stats, d, static_cast<hipStream_t>(stream));
 }
 
+int adder_plain_conv2d_fwd_f32(const float *x, const float *w, float *y, double *stats, int stats_slots, int N,
+                               int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, void *stream) {
+    if (!x || !w || !y) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo;
+    if (overlaps(y, ny, x, nx) || overlaps(y, ny, w, nw)) return ADDER_ERR_ALIAS;
+    if (stats) {
+        const int slots = fwd_stats_slots(d);
+        if (slots == 0) return ADDER_ERR_UNSUPPORTED;
+        if (stats_slots != slots) return ADDER_ERR_BAD_SHAPE;
+        const size_t ns = sizeof(double) * 2 * (size_t)Co * slots;
+        if (overlaps(stats, ns, x, nx) || overlaps(stats, ns, w, nw) || overlaps(stats, ns, y, ny))
+            return ADDER_ERR_ALIAS;
+    }
+    return launch_mulconv_fwd(x, w, y, stats, d, static_cast<hipStream_t>(stream));
+}
+
 int adder_conv2d_bwd_workspace_bytes(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
                                      int pad, size_t *bytes) {
     if (!bytes) return ADDER_ERR_NULL_POINTER;

@@ -108,7 +108,8 @@ int check_launch();                  // hipGetLastError -> status
 
 // Launchers implemented in the kernel translation units.
 int launch_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s);
-int fwd_stats_slots(const ConvDims &d);   // 0: no statistics epilogue for these dimensions
+int fwd_stats_slots(const ConvDims &d);
+int launch_mulconv_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s);   // 0: no statistics epilogue for these dimensions
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s, const float *gadd = nullptr);
 size_t grad_w_workspace_bytes(const ConvDims &d);

@@ -84,7 +84,9 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 // input channels.  Column 0 of a row is input column w0*S-1, so a lane's strip
 // starts at column strip*TN*S, which is 16-byte aligned when TN*S is a multiple of 4.
 // ---------------------------------------------------------------------------
-template <class C, bool VEC = true, bool SUB = false>
+// MUL: the same kernel as an ordinary convolution, y = sum w * x (one v_fmac per term), for the regular
+// stem layer that precedes the adder layers of a network.
+template <class C, bool VEC = true, bool SUB = false, bool MUL = false>
 __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__restrict__ x,
                                                                 const float *__restrict__ w,
                                                                 float *__restrict__ y,
@@ -168,7 +170,10 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
 #pragma unroll
                 for (int idx = 0; idx < CQ * KK * TN; ++idx) {
                     const int t = idx % TN, j = (idx / TN) % KS, i = (idx / TN / KS) % KS, q = idx / TN / KK;
-                    acc[m][t] -= fabsf(wv[m & 1][q * KK + i * KS + j] - xr[cur][q][i][t * S + j]);
+                    if constexpr (MUL)
+                        acc[m][t] = fmaf(wv[m & 1][q * KK + i * KS + j], xr[cur][q][i][t * S + j], acc[m][t]);
+                    else
+                        acc[m][t] -= fabsf(wv[m & 1][q * KK + i * KS + j] - xr[cur][q][i][t * S + j]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
                         if (m + 1 < TM) {
@@ -261,7 +266,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     }
 }
 
-template <class C, bool VEC, bool SUB = false>
+template <class C, bool VEC, bool SUB = false, bool MUL = false>
 static int launch_fwd_3x3_v(const float *x, const float *w, float *y, double *stats, const ConvDims &d,
                             hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
     const int tilesH = ceil_div(d.Ho, C::TH), tilesW = ceil_div(d.Wo, C::TW);
@@ -270,12 +275,12 @@ static int launch_fwd_3x3_v(const float *x, const float *w, float *y, double *st
     if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     static bool attr_set = false;
     if (!attr_set && C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C, VEC, SUB>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C, VEC, SUB, MUL>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return record_hip_error(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC, SUB>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
+    hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC, SUB, MUL>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
                        stats, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, sub);
     return check_launch();
 }
@@ -286,6 +291,14 @@ static int launch_fwd_3x3(const float *x, const float *w, float *y, double *stat
     // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
     if (d.W % 4 == 0) return launch_fwd_3x3_v<C, true>(x, w, y, stats, d, s);
     return launch_fwd_3x3_v<C, false>(x, w, y, stats, d, s);
+}
+
+// the same tile shapes as an ordinary convolution (3x3 / stride 1 / pad 1 only)
+template <class C>
+static int launch_mulconv_3x3(const float *x, const float *w, float *y, double *stats, const ConvDims &d,
+                              hipStream_t s) {
+    if (d.W % 4 == 0) return launch_fwd_3x3_v<C, true, false, true>(x, w, y, stats, d, s);
+    return launch_fwd_3x3_v<C, false, false, true>(x, w, y, stats, d, s);
 }
 
 // partial-sum slots per channel the statistics epilogue of this tile shape writes
@@ -390,6 +403,20 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
     hipLaunchKernelGGL(fwd_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Co, TM)),
                        dim3(256), 0, s, x, w, y, d);
     return check_launch();
+}
+
+// An ordinary convolution y = sum w * x through the tiled forward kernels: 3x3 / stride 1 / pad 1 only
+// (ADDER_ERR_UNSUPPORTED elsewhere).  stats as in launch_fwd; the slot count is fwd_stats_slots(d).
+int launch_mulconv_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s) {
+    const bool ok = d.kh == 3 && d.kw == 3 && d.pad == 1 && d.stride == 1 &&
+                    (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0);
+    if (!ok) return ADDER_ERR_UNSUPPORTED;
+    switch (fwd_tiled_variant(d)) {
+        case 1: return launch_mulconv_3x3<FwdW32>(x, w, y, stats, d, s);
+        case 2: return launch_mulconv_3x3<FwdW16>(x, w, y, stats, d, s);
+        case 3: return launch_mulconv_3x3<FwdW8>(x, w, y, stats, d, s);
+        default: return ADDER_ERR_UNSUPPORTED;
+    }
 }
 
 }  // namespace adder

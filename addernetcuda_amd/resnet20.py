@@ -69,12 +69,22 @@ class _conv2d_matrix_grad(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w, stride, padding):
+        x, w = x.contiguous(), w.contiguous()
         ctx.save_for_backward(x, w)
         ctx.conf = (stride, padding)
-        return F.conv2d(x, w, None, stride, padding)
+        ctx.set_materialize_grads(False)
+        y, stats = _adder.plain_conv2d_forward(x, w, stride, padding)
+        if y is None:   # no tiled kernel for this geometry
+            y, stats = F.conv2d(x, w, None, stride, padding), None
+        if stats is None:
+            stats = torch.empty(0, device=x.device, dtype=torch.float64)
+        ctx.mark_non_differentiable(stats)
+        return y, stats
 
     @staticmethod
-    def backward(ctx, gy):
+    def backward(ctx, gy, _unused=None):
+        if gy is None:
+            return None, None, None, None
         x, w = ctx.saved_tensors
         stride, padding = ctx.conf
         gx = gw = None
@@ -100,7 +110,18 @@ class StemConv2d(nn.Conv2d):
                  and isinstance(self.padding[0], int))
         if not plain:
             return super().forward(x)
-        return _conv2d_matrix_grad.apply(x, self.weight, self.stride[0], self.padding[0])
+        return _conv2d_matrix_grad.apply(x, self.weight, self.stride[0], self.padding[0])[0]
+
+    def forward_with_stats(self, x):
+        """(output, stats) like ``adder2d.forward_with_stats``: the BatchNorm partial sums of the output from the
+        kernel's epilogue, or None."""
+        if not (x.is_cuda and x.dtype == torch.float32 and self.bias is None and self.groups == 1
+                and self.dilation == (1, 1) and self.padding_mode == "zeros" and torch.is_grad_enabled()
+                and self.stride[0] == self.stride[1] and isinstance(self.padding[0], int)
+                and self.padding[0] == self.padding[1]):
+            return super().forward(x), None
+        y, stats = _conv2d_matrix_grad.apply(x, self.weight, self.stride[0], self.padding[0])
+        return y, (stats if stats.numel() else None)
 
 
 class ResNet(nn.Module):
@@ -136,7 +157,11 @@ class ResNet(nn.Module):
         return nn.Sequential(*stage)
 
     def forward(self, x):
-        x = self.bn1(self.conv1(x))
+        if self.bn1.training and x.is_cuda and hasattr(self.conv1, "forward_with_stats"):
+            x, stats = self.conv1.forward_with_stats(x)
+            x = self.bn1(x, stats=stats)
+        else:
+            x = self.bn1(self.conv1(x))
         x = self.layer3(self.layer2(self.layer1(x)))
         if x.shape[2] == 8 and x.shape[3] == 8:
             x = x.mean(dim=(2, 3), keepdim=True)   # AvgPool2d(8) of an 8x8 map, as one reduction kernel

@@ -75,6 +75,15 @@ ADDER_API int adder_conv2d_fwd_stats_f32(const float *x, const float *w, float *
                                          int N, int Ci, int H, int W, int Co, int kh, int kw,
                                          int stride, int pad, void *stream);
 
+/* An ordinary convolution y = sum w * x (no bias) through the tiled kernel of the adder forward, for the
+ * regular stem layer in front of the adder layers (resnet20.py:49 uses nn.Conv2d there): 3x3 / stride 1 /
+ * pad 1 only, ADDER_ERR_UNSUPPORTED (nothing launched) elsewhere.  stats (nullable) / stats_slots as in
+ * adder_conv2d_fwd_stats_f32, with the slot count of adder_conv2d_fwd_stats_slots for the same dimensions.
+ * Its weight gradient: adder_conv2d_grad_w_staged_f32 with w = NULL. */
+ADDER_API int adder_plain_conv2d_fwd_f32(const float *x, const float *w, float *y, double *stats, int stats_slots,
+                                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                                         int stride, int pad, void *stream);
+
 /* Bytes of scratch adder_conv2d_bwd_f32 needs for these dimensions. */
 ADDER_API int adder_conv2d_bwd_workspace_bytes(int N, int Ci, int H, int W, int Co, int kh, int kw,
                                      int stride, int pad, size_t *bytes);

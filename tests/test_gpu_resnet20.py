@@ -141,6 +141,7 @@ def test_stem_convolution_weight_gradient_matches_torch(gpu):
             conv.weight.grad = None
             xg = x.to(gpu).requires_grad_(True)
             y = conv(xg)
+            assert_close(y, yd.detach(), f"stem forward {shape}", rtol=1e-5, atol=1e-5)
             if batched:
                 with adder.batched_eta_scaling():
                     y.backward(gy.to(gpu))
@@ -149,3 +150,12 @@ def test_stem_convolution_weight_gradient_matches_torch(gpu):
             torch.cuda.synchronize()
             assert_close(conv.weight.grad, wd.grad, f"stem grad_W {shape} batched={batched}", rtol=1e-5, atol=1e-4)
             assert_close(xg.grad, xd.grad, f"stem grad_X {shape}", rtol=1e-4, atol=1e-4)
+        y2, stats = conv.forward_with_stats(x.to(gpu))
+        if stride == 1:     # the tiled kernel: statistics of the output from its epilogue
+            assert stats is not None
+            tot = stats.sum(dim=1).cpu()
+            assert torch.allclose(tot[:, 0], yd.detach().sum(dim=(0, 2, 3)), rtol=1e-5, atol=1e-4)
+            assert torch.allclose(tot[:, 1], (yd.detach() ** 2).sum(dim=(0, 2, 3)), rtol=1e-5, atol=1e-4)
+        else:
+            assert stats is None
+        assert_close(y2, yd.detach(), f"stem forward_with_stats {shape}", rtol=1e-5, atol=1e-5)
