@@ -98,11 +98,24 @@ __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ par
     const int idx = block * kFinOut + o;
     const int idc = idx < total ? idx : total - 1;
     const int co = idc / K;
-    double a = 0.0, sgs = 0.0;
-    for (int p = sl; p < slots; p += kFinLanes) {
-        a += (double)part[(size_t)p * total + idc];
-        sgs += (double)sgpart[(size_t)p * Co + co];
+    // four slots per round, so that eight loads are in flight per thread (the loop is latency-bound)
+    double a4[4] = {0.0, 0.0, 0.0, 0.0}, s4[4] = {0.0, 0.0, 0.0, 0.0};
+    int p = sl;
+    for (; p + 3 * kFinLanes < slots; p += 4 * kFinLanes) {
+        PT va[4], vs[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            va[u] = part[(size_t)(p + u * kFinLanes) * total + idc];
+            vs[u] = sgpart[(size_t)(p + u * kFinLanes) * Co + co];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { a4[u] += (double)va[u]; s4[u] += (double)vs[u]; }
     }
+    for (; p < slots; p += kFinLanes) {
+        a4[0] += (double)part[(size_t)p * total + idc];
+        s4[0] += (double)sgpart[(size_t)p * Co + co];
+    }
+    const double a = (a4[0] + a4[1]) + (a4[2] + a4[3]), sgs = (s4[0] + s4[1]) + (s4[2] + s4[3]);
     __shared__ double ra[kFinLanes][kFinOut + 1], rs[kFinLanes][kFinOut + 1];
     ra[sl][o] = a;
     rs[sl][o] = sgs;
@@ -133,36 +146,40 @@ __global__ __launch_bounds__(kFinOut * kFinLanes) void grad_w_finalize_kernel(co
     grad_w_finalize_block<PT>(part, sgpart, w, gw, ss, slots, Co, K, blockIdx.x);
 }
 
-// The finalize of up to kGwFinishMax layers in one launch (grid = (most blocks of any layer, layers)) and
-// their scaling in a second: for callers that leave the partial slabs of every layer in its workspace
-// during the backward pass and finish all weight gradients together at its end.
+// The finalize of up to kGwFinishMax layers in one launch and their scaling in a second: for callers that
+// leave the partial slabs of every layer in its workspace during the backward pass and finish all weight
+// gradients together at its end.  The finalize grid is the concatenation of the layers' own grids
+// (first[t] = first workgroup of layer t); the scaling grid is (P, layers).
 struct GwStageBatch {
     adder_grad_w_stage it[kGwFinishMax];
+    int first[kGwFinishMax + 1];
+    int count;
 };
 
 __global__ __launch_bounds__(kFinOut * kFinLanes) void batch_finalize_kernel(const GwStageBatch b,
-                                                                             double *__restrict__ ss, int nbmax) {
-    const adder_grad_w_stage &it = b.it[blockIdx.y];
-    const int nb = ceil_div(it.Co * it.K, kFinOut);
-    if ((int)blockIdx.x >= nb) return;
-    double *mine = ss + (size_t)blockIdx.y * nbmax;
+                                                                             double *__restrict__ ss) {
+    int t = 0;
+    while (t + 1 < b.count && (int)blockIdx.x >= b.first[t + 1]) ++t;   // wave-uniform, at most 31 steps
+    const adder_grad_w_stage &it = b.it[t];
+    const int block = blockIdx.x - b.first[t];
+    double *mine = ss + b.first[t];
     if (it.fp64)
         grad_w_finalize_block<double>(static_cast<const double *>(it.part), static_cast<const double *>(it.sgpart), it.w,
-                                      it.gw, mine, it.slots, it.Co, it.K, blockIdx.x);
+                                      it.gw, mine, it.slots, it.Co, it.K, block);
     else
         grad_w_finalize_block<float>(static_cast<const float *>(it.part), static_cast<const float *>(it.sgpart), it.w,
-                                     it.gw, mine, it.slots, it.Co, it.K, blockIdx.x);
+                                     it.gw, mine, it.slots, it.Co, it.K, block);
 }
 
 __global__ __launch_bounds__(256) void batch_finish_scale_kernel(const GwStageBatch b, const double *__restrict__ ss,
-                                                                 int nbmax, float eps) {
-    const adder_grad_w_stage &it = b.it[blockIdx.y];
+                                                                 float eps) {
+    const int t = blockIdx.y;
+    const adder_grad_w_stage &it = b.it[t];
     if (!(it.eta > 0.f)) return;   // left raw
     const long n = (long)it.Co * it.K;
-    const int nb = ceil_div(it.Co * it.K, kFinOut);
     __shared__ double red[4];
     double v = 0.0;
-    for (int i = threadIdx.x; i < nb; i += 256) v += ss[(size_t)blockIdx.y * nbmax + i];
+    for (int i = b.first[t] + threadIdx.x; i < b.first[t + 1]; i += 256) v += ss[i];
     v = wave_sum(v);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
     __syncthreads();
@@ -418,33 +435,32 @@ int launch_grad_w_staged(const float *gy, const float *x, const float *w, float 
     return rc;
 }
 
-static int finish_blocks(int count, const adder_grad_w_stage *st) {
-    int most = 1;
-    for (int t = 0; t < count; ++t) {
-        const int nb = ceil_div(st[t].Co * st[t].K, kFinOut);
-        most = nb > most ? nb : most;
-    }
-    return most;
+static long finish_blocks(int count, const adder_grad_w_stage *st) {
+    long total = 0;
+    for (int t = 0; t < count; ++t) total += ceil_div(st[t].Co * st[t].K, kFinOut);
+    return total;
 }
 
 size_t grad_w_finish_workspace_bytes(int count, const adder_grad_w_stage *st) {
-    return ((size_t)count * finish_blocks(count, st) * sizeof(double) + 255) & ~(size_t)255;
+    return ((size_t)finish_blocks(count, st) * sizeof(double) + 255) & ~(size_t)255;
 }
 
 int launch_grad_w_finish(int count, const adder_grad_w_stage *st, void *ws, hipStream_t s) {
     GwStageBatch b{};
     long most_n = 1;
+    b.count = count;
     for (int t = 0; t < count; ++t) {
         b.it[t] = st[t];
+        b.first[t + 1] = b.first[t] + ceil_div(st[t].Co * st[t].K, kFinOut);
         const long n = (long)st[t].Co * st[t].K;
         most_n = n > most_n ? n : most_n;
     }
-    const int nbmax = finish_blocks(count, st);
+    if (finish_blocks(count, st) > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     double *ss = reinterpret_cast<double *>(ws);
-    hipLaunchKernelGGL(batch_finalize_kernel, dim3(nbmax, count), dim3(kFinOut * kFinLanes), 0, s, b, ss, nbmax);
+    hipLaunchKernelGGL(batch_finalize_kernel, dim3((unsigned)b.first[count]), dim3(kFinOut * kFinLanes), 0, s, b, ss);
     long P = ceil_div_l(most_n, 2048);
     P = P < 1 ? 1 : (P > 256 ? 256 : P);
-    hipLaunchKernelGGL(batch_finish_scale_kernel, dim3((unsigned)P, count), dim3(256), 0, s, b, ss, nbmax, 1e-12f);
+    hipLaunchKernelGGL(batch_finish_scale_kernel, dim3((unsigned)P, count), dim3(256), 0, s, b, ss, 1e-12f);
     return check_launch();
 }
 
