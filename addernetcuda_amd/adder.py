@@ -64,8 +64,9 @@ class batched_eta_scaling:
     meaningful; after the block it holds what it would hold without it.
 
     It only takes over layers whose weight is a leaf with ``grad is None`` when their backward runs (the usual
-    ``zero_grad(set_to_none=True)`` loop); all others are scaled on the spot as always.  Not for code that
-    looks at weight gradients from hooks during the backward pass, nor for ``torch.autograd.grad``."""
+    ``zero_grad(set_to_none=True)`` loop); all others are finished on the spot as always.  One backward pass
+    per block.  Not for code that looks at weight gradients from hooks during the backward pass, nor for
+    ``torch.autograd.grad``."""
 
     def __enter__(self):
         global _eta_batch
@@ -173,9 +174,10 @@ class _adder_nchw(Function):
         gx = torch.empty_like(X) if need_x else None
         gw = torch.empty_like(W) if need_w else None
         eta = float(ctx.eta or 0.0)
+        if _eta_batch is not None and need_w and any(W is entry[0] for entry in _eta_batch):
+            raise RuntimeError("batched_eta_scaling: this weight already has a pending gradient in the block "
+                               "(one backward pass per block, no weight shared between layers)")
         if (_eta_batch is not None and need_w and ctx.w_is_given and W.is_leaf and W.grad is None):
-            if any(W is entry[0] for entry in _eta_batch):
-                raise RuntimeError("batched_eta_scaling: a weight that is used by two layers cannot be deferred")
             with torch.cuda.device(dev):
                 ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev)
                 stage = GradWStage()
