@@ -25,6 +25,7 @@ SHAPES = [
     (3, 24, 32, 32, 48, 1, 1, 0),      # DenseNet-BC bottleneck 1x1 (densenet.py:12-14)
     (3, 48, 32, 32, 12, 3, 1, 1),      # DenseNet-BC growth conv, Co = 12
     (1, 32, 16, 16, 640, 3, 2, 1),     # strided 3x3 with > 2304 terms per input position (three-instruction grad_X form)
+    (64, 1024, 7, 7, 64, 1, 1, 0),     # 1x1 on 49-position planes with many images x channel blocks (the larger small-plane grad_X tile)
 ]
 
 
