@@ -9,7 +9,8 @@ reference's (`adder`, `b`, BatchNorm names), so checkpoints move between the two
 What it drops: the CIFAR download and wandb (no network here; data comes from an ``.npz`` file or is
 synthetic), and the guards that skip batches whose size is not a multiple of 12 (main.py:83,114) — the
 kernels take any batch size.  Augmentation runs on the GPU on uint8-derived tensors, so no worker
-processes are needed.
+processes are needed.  What it adds: the training step of a full batch runs as one captured HIP graph
+(``--no-graph`` keeps it eager): 2.3 instead of 3.5 ms per batch of 256.
 
     python -m addernetcuda_amd.train --synthetic 4096 --epochs 2
     python -m addernetcuda_amd.train --data cifar10.npz --epochs 400 --output-dir models/
@@ -96,8 +97,48 @@ def evaluate(net, x_u8, y, batch):
     return loss_sum / n, correct / n
 
 
-def train_one_epoch(net, opt, x_u8, y, batch, generator=None):
+def train_step(net, opt, images, labels):
     from addernetcuda_amd.adder import batched_eta_scaling
+    opt.zero_grad(set_to_none=True)
+    loss = F.cross_entropy(net(images), labels)
+    with batched_eta_scaling():   # the adaptive scaling of all adder layers in two launches
+        loss.backward()
+    opt.step()
+    return loss.detach()
+
+
+class GraphedStep:
+    """``train_step`` for one fixed batch shape as a captured HIP graph: the eager step spends more time in
+    Python and launch calls than the GPU spends on the kernels.  The first ``warmup`` calls run eagerly (they are
+    real training steps), the next one is captured, all later ones replay the capture on fresh data copied into
+    the graph's input buffers.  The learning rate must be a device tensor of the optimizer (a float would be
+    frozen into the graph); BatchNorm's running statistics and the optimizer state are updated by the graph's
+    own kernels.  All calls must come from the same (non-default) stream."""
+
+    def __init__(self, net, opt, warmup=3):
+        self.net, self.opt, self.warmup = net, opt, warmup
+        self.graph = self.images = self.labels = self.loss = None
+        self.calls = 0
+
+    def __call__(self, images, labels):
+        self.calls += 1
+        if self.graph is None and self.calls <= self.warmup:
+            return train_step(self.net, self.opt, images, labels)
+        if self.graph is None:
+            self.images, self.labels = images.clone(), labels.clone()
+            self.opt.zero_grad(set_to_none=True)
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, stream=torch.cuda.current_stream()):
+                self.loss = train_step(self.net, self.opt, self.images, self.labels)
+        else:
+            self.images.copy_(images)
+            self.labels.copy_(labels)
+        self.graph.replay()
+        return self.loss.clone()
+
+
+def train_one_epoch(net, opt, x_u8, y, batch, generator=None, graphed=None):
+    """``graphed``: a GraphedStep for batches of exactly ``batch`` images (the tail batch runs eagerly)."""
     net.train()
     n = x_u8.shape[0]
     perm = torch.randperm(n, device=x_u8.device, generator=generator)
@@ -107,12 +148,8 @@ def train_one_epoch(net, opt, x_u8, y, batch, generator=None):
         if idx.numel() < 2:     # BatchNorm needs more than one value per channel
             break
         images = augment(normalise(x_u8[idx]), generator)
-        opt.zero_grad(set_to_none=True)
-        loss = F.cross_entropy(net(images), y[idx])
-        with batched_eta_scaling():   # the adaptive scaling of all adder layers in two launches
-            loss.backward()
-        opt.step()
-        losses.append(loss.detach())
+        step = graphed if graphed is not None and idx.numel() == batch else None
+        losses.append(step(images, y[idx]) if step else train_step(net, opt, images, y[idx]))
     return torch.stack(losses).mean().item()
 
 
@@ -126,20 +163,26 @@ def run(args):
     net = resnet20(eta=args.eta).to(dev)
     if args.resume:
         net.load_state_dict(torch.load(args.resume, map_location=dev, weights_only=True))
-    opt = torch.optim.SGD(net.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4, fused=True)
+    # the learning rate lives on the device so that the captured step sees each epoch's value
+    lr_now = torch.tensor(float(args.lr), device=dev)
+    opt = torch.optim.SGD(net.parameters(), lr=lr_now, momentum=0.9, weight_decay=5e-4, fused=True)
     if args.eval_only:   # the reference's test.py: load a checkpoint, one pass over the test split
         test_loss, acc = evaluate(net, *data["test"], args.test_batch_size)
         print(f"test loss {test_loss:.4f}  accuracy {acc:.4f}", flush=True)
         return [{"epoch": 0, "test_loss": test_loss, "accuracy": acc}]
     os.makedirs(args.output_dir, exist_ok=True)
     gen = torch.Generator(device=dev).manual_seed(args.seed)
+    graphed = None if args.no_graph else GraphedStep(net, opt)
+    stream = torch.cuda.Stream()   # graph capture needs a stream of its own; the eager steps share it
     best, history = 0.0, []
     for epoch in range(1, args.epochs + 1):
         lr = cosine_lr(epoch, args.epochs, args.lr)
-        for group in opt.param_groups:
-            group["lr"] = lr
+        torch.cuda.synchronize()
+        lr_now.fill_(lr)
         t0 = time.time()
-        train_loss = train_one_epoch(net, opt, *data["train"], args.batch_size, gen)
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            train_loss = train_one_epoch(net, opt, *data["train"], args.batch_size, gen, graphed)
         torch.cuda.synchronize()
         dt = time.time() - t0
         test_loss, acc = evaluate(net, *data["test"], args.test_batch_size)
@@ -165,6 +208,7 @@ def parse_args(argv=None):
     p.add_argument("--test-batch-size", type=int, default=500)
     p.add_argument("--lr", type=float, default=0.05, help="peak of the cosine schedule (main.py:71: 2 x 0.025)")
     p.add_argument("--eta", type=float, default=0.2, help="adaptive grad_W scale, adder.py:78 uses 1/5")
+    p.add_argument("--no-graph", action="store_true", help="run every training step eagerly instead of as a HIP graph")
     p.add_argument("--seed", type=int, default=0)
     return p.parse_args(argv)
 
