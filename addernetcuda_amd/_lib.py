@@ -1,5 +1,6 @@
 """ctypes binding of libaddernet_hip.so (the C ABI declared in include/addernet_hip.h)."""
 import ctypes
+import functools
 import os
 
 import torch
@@ -90,15 +91,46 @@ def same_device(*tensors):
     return dev
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    """The current HIP stream of ``device`` as the integer handle the C ABI takes."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def ptr(t):
-    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+    """Device address of a tensor (None -> NULL) for a ``void *`` / ``float *`` argument."""
+    return t.data_ptr() if t is not None else None
 
 
-def conv_dims(x_shape, w_shape, stride, padding):
+class on_device:
+    """``with on_device(dev):`` makes ``dev`` the current HIP device for the launches inside, like
+    ``torch.cuda.device`` but without touching the runtime when it already is (the usual case)."""
+    __slots__ = ("index", "previous")
+
+    def __init__(self, device):
+        self.index = device.index
+
+    def __enter__(self):
+        self.previous = None
+        if self.index is not None:
+            current = torch.cuda.current_device()
+            if current != self.index:
+                self.previous = current
+                torch.cuda.set_device(self.index)
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if self.previous is not None:
+            torch.cuda.set_device(self.previous)
+        return False
+
+
+@functools.lru_cache(maxsize=4096)
+def _conv_dims(x_shape, w_shape, stride, padding):
     N, Ci, H, W = x_shape
     Co, Ciw, kh, kw = w_shape
     if Ci != Ciw:
@@ -110,8 +142,36 @@ def conv_dims(x_shape, w_shape, stride, padding):
     return (N, Ci, H, W, Co, kh, kw, stride, padding), Ho, Wo
 
 
-def conv2d_bwd_workspace(dims, device):
+def conv_dims(x_shape, w_shape, stride, padding):
+    """(N, Ci, H, W, Co, kh, kw, stride, padding), Ho, Wo of a layer; the answers are cached per geometry."""
+    return _conv_dims(tuple(x_shape), tuple(w_shape), stride, padding)
+
+
+@functools.lru_cache(maxsize=4096)
+def fwd_stats_slots(dims):
+    """Slots of the forward's BatchNorm partial sums for this geometry (0: the kernel has no such epilogue)."""
+    slots = ctypes.c_int(0)
+    check(lib.adder_conv2d_fwd_stats_slots(*dims, ctypes.byref(slots)), "adder_conv2d_fwd_stats_slots")
+    return slots.value
+
+
+@functools.lru_cache(maxsize=4096)
+def conv2d_bwd_workspace_bytes(dims):
     need = ctypes.c_size_t(0)
     check(lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)), "adder_conv2d_bwd_workspace_bytes")
+    return need.value
+
+
+def conv2d_bwd_workspace(dims, device):
+    need = conv2d_bwd_workspace_bytes(dims)
     # torch's caching allocator hands out >=512-byte aligned blocks and is graph-capture safe
-    return torch.empty(max(need.value, 256), dtype=torch.uint8, device=device), need.value
+    return torch.empty(max(need, 256), dtype=torch.uint8, device=device), need
+
+
+@functools.lru_cache(maxsize=4096)
+def bn_act_sizes(N, C, HW):
+    """(workspace bytes, sign-mask words) of the fused BatchNorm kernels for an (N, C, HW) tensor."""
+    need, words = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    check(lib.adder_bn_act_workspace_bytes(N, C, HW, ctypes.byref(need)), "adder_bn_act_workspace_bytes")
+    check(lib.adder_bn_act_mask_words(N, C, HW, ctypes.byref(words)), "adder_bn_act_mask_words")
+    return need.value, words.value

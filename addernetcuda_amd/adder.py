@@ -15,7 +15,7 @@ from torch.autograd import Function
 
 from . import adder_cuda
 from ._lib import (lib, check, ptr, require_gpu_f32, same_device, stream_ptr, conv_dims, conv2d_bwd_workspace,
-                   GradWStage)
+                   fwd_stats_slots, on_device, GradWStage)
 
 DEFAULT_ETA = 0.2  # adder.py:78 divides by 5
 
@@ -45,7 +45,7 @@ class adder(Function):
             need = ctypes.c_size_t(0)
             check(lib.adder_norm_scale_workspace_bytes(n, ctypes.byref(need)), "adder_norm_scale_workspace_bytes")
             ws = torch.empty(need.value, dtype=torch.uint8, device=dev)
-            with torch.cuda.device(dev):
+            with on_device(dev):
                 check(lib.adder_grad_norm_scale_f32(ptr(grad_W_col), n, float(ctx.eta), 1e-12, ptr(ws), need.value,
                                                     stream_ptr(dev)), "adder_grad_norm_scale_f32")
         return grad_W_col, grad_X_col, None
@@ -92,7 +92,7 @@ class batched_eta_scaling:
                 stage.gw = g.data_ptr()   # autograd may have handed the gradient over in another tensor
                 staged.setdefault(g.device, []).append(stage)
         for dev, stages in staged.items():
-            with torch.cuda.device(dev):
+            with on_device(dev):
                 for i in range(0, len(stages), 32):
                     chunk = stages[i:i + 32]
                     arr = (GradWStage * len(chunk))(*chunk)
@@ -103,7 +103,7 @@ class batched_eta_scaling:
                     check(lib.adder_grad_w_finish_f32(len(chunk), arr, ptr(ws), need.value, stream_ptr(dev)),
                           "adder_grad_w_finish_f32")
         for dev, items in by_device.items():
-            with torch.cuda.device(dev):
+            with on_device(dev):
                 for i in range(0, len(items), 64):
                     chunk = items[i:i + 64]
                     count = len(chunk)
@@ -132,14 +132,12 @@ class _adder_nchw(Function):
         dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
         out = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
         stats = None
-        with torch.cuda.device(dev):
-            slots = ctypes.c_int(0)
-            if with_stats:
-                check(lib.adder_conv2d_fwd_stats_slots(*dims, ctypes.byref(slots)), "adder_conv2d_fwd_stats_slots")
-            if slots.value > 0:
+        with on_device(dev):
+            slots = fwd_stats_slots(dims) if with_stats else 0
+            if slots > 0:
                 # partial sums of out and out**2 per channel for the BatchNorm that follows (bn_act.py)
-                stats = torch.empty((W.size(0), slots.value, 2), device=dev, dtype=torch.float64)
-                check(lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots.value, *dims,
+                stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64)
+                check(lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots, *dims,
                                                      stream_ptr(dev)), "adder_conv2d_fwd_stats_f32")
             else:
                 check(lib.adder_conv2d_fwd_f32(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_f32")
@@ -178,7 +176,7 @@ class _adder_nchw(Function):
             raise RuntimeError("batched_eta_scaling: this weight already has a pending gradient in the block "
                                "(one backward pass per block, no weight shared between layers)")
         if (_eta_batch is not None and need_w and ctx.w_is_given and W.is_leaf and W.grad is None):
-            with torch.cuda.device(dev):
+            with on_device(dev):
                 ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev)
                 stage = GradWStage()
                 status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gw), eta, ptr(ws), nbytes,
@@ -195,7 +193,7 @@ class _adder_nchw(Function):
         if not need_w:
             gw = None
         if need_x or need_w:
-            with torch.cuda.device(dev):
+            with on_device(dev):
                 ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev) if need_w else (None, 0)
                 fused = False
                 if need_x and grad_short is not None:
@@ -221,12 +219,11 @@ def plain_conv2d_forward(X, W, stride, padding):
     require_gpu_f32(W, "W")
     dev = same_device(X, W)
     dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
-    with torch.cuda.device(dev):
-        slots = ctypes.c_int(0)
-        check(lib.adder_conv2d_fwd_stats_slots(*dims, ctypes.byref(slots)), "adder_conv2d_fwd_stats_slots")
+    with on_device(dev):
+        slots = fwd_stats_slots(dims)
         y = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
-        stats = torch.empty((W.size(0), slots.value, 2), device=dev, dtype=torch.float64) if slots.value else None
-        status = lib.adder_plain_conv2d_fwd_f32(ptr(X), ptr(W), ptr(y), ptr(stats), slots.value, *dims, stream_ptr(dev))
+        stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64) if slots else None
+        status = lib.adder_plain_conv2d_fwd_f32(ptr(X), ptr(W), ptr(y), ptr(stats), slots, *dims, stream_ptr(dev))
     if status == -7:
         return None, None
     check(status, "adder_plain_conv2d_fwd_f32")
@@ -244,7 +241,7 @@ def conv2d_weight_grad(grad_out, X, W, stride, padding):
     dev = X.device
     dims, _, _ = conv_dims(X.shape, W.shape, stride, padding)
     gw = torch.empty(W.shape, device=dev, dtype=torch.float32)
-    with torch.cuda.device(dev):
+    with on_device(dev):
         ws, nbytes = conv2d_bwd_workspace(dims, dev)
         stage = GradWStage()
         status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), None, ptr(gw), 0.0, ptr(ws), nbytes, *dims,

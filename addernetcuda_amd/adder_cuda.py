@@ -13,7 +13,7 @@ import ctypes
 import torch
 
 from . import _lib
-from ._lib import lib, check, ptr, require_gpu_f32, same_device, stream_ptr
+from ._lib import lib, check, ptr, require_gpu_f32, same_device, stream_ptr, on_device
 
 
 def _col_shapes(x, w, **others):
@@ -44,7 +44,7 @@ def ADDER_CONV(x, w, y):
         require_gpu_f32(t, n)
     dev = same_device(x, w, y)
     K, NL, Co = _col_shapes(x, w, y=y)
-    with torch.cuda.device(dev):
+    with on_device(dev):
         check(lib.adder_col_fwd_f32(ptr(x), ptr(w), ptr(y), K, NL, Co, stream_ptr(dev)), "ADDER_CONV")
 
 
@@ -54,7 +54,7 @@ def ADDER_CONV_WEIGHT(grad_y, x, w, grad_w):
         require_gpu_f32(t, n)
     dev = same_device(grad_y, x, w, grad_w)
     K, NL, Co = _col_shapes(x, w, grad_y=grad_y, grad_w=grad_w)
-    with torch.cuda.device(dev):
+    with on_device(dev):
         ws, nbytes = _ws(K, NL, Co, dev)
         check(lib.adder_col_gradw_f32(ptr(grad_y), ptr(x), ptr(w), ptr(grad_w), K, NL, Co, ptr(ws), nbytes,
                                       stream_ptr(dev)), "ADDER_CONV_WEIGHT")
@@ -66,7 +66,7 @@ def ADDER_CONV_INPUT(grad_y, x, w, grad_i):
         require_gpu_f32(t, n)
     dev = same_device(grad_y, x, w, grad_i)
     K, NL, Co = _col_shapes(x, w, grad_y=grad_y, grad_i=grad_i)
-    with torch.cuda.device(dev):
+    with on_device(dev):
         check(lib.adder_col_gradx_f32(ptr(grad_y), ptr(x), ptr(w), ptr(grad_i), K, NL, Co, stream_ptr(dev)),
               "ADDER_CONV_INPUT")
 
@@ -77,7 +77,7 @@ def ADDER_BACKWARD(grad_y, x, w, grad_w, grad_i):
         require_gpu_f32(t, n)
     dev = same_device(grad_y, x, w, grad_w, grad_i)
     K, NL, Co = _col_shapes(x, w, grad_y=grad_y, grad_w=grad_w, grad_i=grad_i)
-    with torch.cuda.device(dev):
+    with on_device(dev):
         ws, nbytes = _ws(K, NL, Co, dev)
         check(lib.adder_col_bwd_f32(ptr(grad_y), ptr(x), ptr(w), ptr(grad_w), ptr(grad_i), K, NL, Co, ptr(ws),
                                     nbytes, stream_ptr(dev)), "ADDER_BACKWARD")

@@ -7,20 +7,17 @@ csrc/bn_act.hip.  It replaces the separate bn / += residual / relu ops of resnet
 Anything the fused kernels do not cover (eval mode, CPU tensors, non-fp32) goes through the
 ordinary torch ops with identical semantics.
 """
-import ctypes
-
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 from torch.autograd import Function
 
-from ._lib import lib, check, ptr, stream_ptr
+from ._lib import lib, check, ptr, stream_ptr, on_device, bn_act_sizes
 
 
 def _workspace(N, C, HW, device):
-    need = ctypes.c_size_t(0)
-    check(lib.adder_bn_act_workspace_bytes(N, C, HW, ctypes.byref(need)), "adder_bn_act_workspace_bytes")
-    return torch.empty(max(need.value, 256), dtype=torch.uint8, device=device), need.value
+    need = bn_act_sizes(N, C, HW)[0]
+    return torch.empty(max(need, 256), dtype=torch.uint8, device=device), need
 
 
 class _bn_act(Function):
@@ -39,11 +36,10 @@ class _bn_act(Function):
         # the backward needs y only for its sign: one bit per element where the kernels offer it
         mask = None
         if relu and all(t is None or t.data_ptr() % 16 == 0 for t in (x, y, residual)):
-            words = ctypes.c_size_t(0)
-            check(lib.adder_bn_act_mask_words(N, C, HW, ctypes.byref(words)), "adder_bn_act_mask_words")
-            if words.value:
-                mask = torch.empty(words.value, dtype=torch.int32, device=dev)
-        with torch.cuda.device(dev):
+            words = bn_act_sizes(N, C, HW)[1]
+            if words:
+                mask = torch.empty(words, dtype=torch.int32, device=dev)
+        with on_device(dev):
             if stats is not None:
                 # the layer that produced x already summed x and x*x per channel (adder.forward_with_stats)
                 if stats.dtype != torch.float64 or stats.dim() != 3 or stats.shape[0] != C or stats.shape[2] != 2 \
@@ -74,7 +70,7 @@ class _bn_act(Function):
         dgamma, dbeta = torch.empty_like(weight), torch.empty_like(weight)
         if mask is not None and dy.data_ptr() % 16:
             dy = dy.clone()   # the masked kernels move float4 groups
-        with torch.cuda.device(dev):
+        with on_device(dev):
             ws, nbytes = _workspace(N, C, HW, dev)
             check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(mask), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
                                            ptr(dres), ptr(dgamma), ptr(dbeta), int(ctx.relu), N, C, HW, ptr(ws), nbytes,
