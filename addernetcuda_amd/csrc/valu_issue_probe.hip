@@ -8,6 +8,7 @@
 //   fwd   pair    v_sub d, s_w, v_x ; v_sub acc, acc, |d|                   (forward)
 //   gradx pair    v_fma d, s_w, 0.5, v_c clamp ; v_fmac acc, d, g          (input gradient)
 //   sgpr  only    v_sub acc, s_w, acc    (every instruction reads a scalar register: one per slot)
+//   vgpr  pair    the gradx pair with the weight in a vector register (no scalar operand at all)
 // Output: one line per case, "<name> <waves per SIMD> <lane-instructions per second>".
 //
 // A second table is about the fp64 matrix instruction of the weight-gradient kernel,
@@ -32,7 +33,7 @@ constexpr int kChains = 16, kRepeat = 8;
 template <int MODE>
 __global__ __launch_bounds__(1024) void issue_kernel(float *out, int iters, float w) {
     float acc[kChains], tmp[kChains];
-    const float x = threadIdx.x * 0.5f, g = threadIdx.x * 0.25f;
+    const float x = threadIdx.x * 0.5f, g = threadIdx.x * 0.25f, wv = w + threadIdx.x * 0.125f;
 #pragma unroll
     for (int i = 0; i < kChains; ++i) { acc[i] = threadIdx.x * 0.001f + i; tmp[i] = 0.f; }
     for (int it = 0; it < iters; ++it) {
@@ -46,6 +47,9 @@ __global__ __launch_bounds__(1024) void issue_kernel(float *out, int iters, floa
                 else if (MODE == 1)
                     asm volatile("v_fma_f32 %1, %2, 0.5, %3 clamp\n v_fmac_f32_e32 %0, %1, %4"
                                  : "+v"(acc[i]), "+v"(tmp[i]) : "s"(w), "v"(x), "v"(g));
+                else if (MODE == 3)
+                    asm volatile("v_fma_f32 %1, %2, 0.5, %3 clamp\n v_fmac_f32_e32 %0, %1, %4"
+                                 : "+v"(acc[i]), "+v"(tmp[i]) : "v"(wv), "v"(x), "v"(g));
                 else
                     asm volatile("v_sub_f32_e32 %0, %1, %0\n v_sub_f32_e32 %0, %1, %0" : "+v"(acc[i]) : "s"(w));
             }
@@ -139,6 +143,7 @@ int main() {
     if (run<0>("fwd_pair", 2, out, cus)) return 1;
     if (run<1>("gradx_pair", 2, out, cus)) return 1;
     if (run<2>("sgpr_only", 2, out, cus)) return 1;
+    if (run<3>("vgpr_pair", 2, out, cus)) return 1;
     float *in = nullptr;
     CHECK(hipMalloc(&in, 4096));
     CHECK(hipMemset(in, 0, 4096));

@@ -169,7 +169,7 @@ def issue_probe():
     table = {}
     for line in out.splitlines():
         f = line.split()
-        if len(f) == 3 and f[0] in ("fwd_pair", "gradx_pair", "sgpr_only"):
+        if len(f) == 3 and f[0] in ("fwd_pair", "gradx_pair", "sgpr_only", "vgpr_pair"):
             table.setdefault(f[0], {})[f"{f[1]}_waves_per_simd"] = round(float(f[2]) / 1e12, 2)
     return table or None
 
