@@ -187,15 +187,25 @@ def make_step(model, opt, x, y):
     return step
 
 
-def build_training(dev, seed=0):
-    from addernetcuda_amd.resnet20 import resnet20
+# the reference's three model configurations: (batch, input size, classes)
+MODELS = {"resnet20": (BATCH, 32, 10), "vgg_small": (128, 32, 10), "resnet50": (64, 224, 1000)}
+
+
+def build_training(dev, seed=0, which="resnet20"):
     torch.manual_seed(seed)
-    model = resnet20(eta=ETA).to(dev)
+    batch, size, classes = MODELS[which]
+    if which == "resnet20":
+        from addernetcuda_amd.resnet20 import resnet20
+        model = resnet20(eta=ETA)
+    else:
+        from addernetcuda_amd import models
+        model = getattr(models, which)(num_classes=classes, eta=ETA)
+    model = model.to(dev)
     # fused=True: the same update as the default implementation, in one kernel per parameter group
     opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4, fused=True)
     g = torch.Generator(device=dev).manual_seed(seed + 1)
-    x = torch.randn(BATCH, 3, 32, 32, device=dev, generator=g)
-    y = torch.randint(0, 10, (BATCH,), device=dev, generator=g)
+    x = torch.randn(batch, 3, size, size, device=dev, generator=g)
+    y = torch.randint(0, classes, (batch,), device=dev, generator=g)
     return model, opt, x, y
 
 
@@ -220,14 +230,14 @@ def capture_step(model, opt, x, y):
     return graph, loss
 
 
-def graph_matches_eager(dev, replays=4):
+def graph_matches_eager(dev, replays=4, which="resnet20"):
     """Replay the captured step from a saved state and run the eager step from the same state, several times.
 
     Torch's own kernels are not run-to-run deterministic, so trajectories cannot be compared over many steps;
     one step from identical weights, momentum and BatchNorm statistics can.
     """
     import copy
-    model, opt, x, y = build_training(dev)
+    model, opt, x, y = build_training(dev, which=which)
     graph, loss = capture_step(model, opt, x, y)
     eager = make_step(model, opt, x, y)
     worst = 0.0
@@ -290,6 +300,10 @@ def main():
     ap.add_argument("--layers-only", action="store_true",
                     help="run only the per-layer table (7 ResNet-20 layer shapes x forward / grad_X / grad_W); "
                          "meant to run under rocprofv3 --pmc / --kernel-trace")
+    ap.add_argument("--model", choices=sorted(MODELS), default="resnet20",
+                    help="resnet20 (default) is the benchmark; vgg_small (batch 128) and resnet50 (batch 64, 224x224) "
+                         "time the training step of the reference's two other model configurations and print a "
+                         "shorter line")
     ap.add_argument("--layer-set", choices=sorted(LAYER_SETS), default="resnet20",
                     help="with --layers-only: the adder layers of ResNet-20 (batch 256), the VGG-small stack "
                          "(batch 128) or ResNet-50 at 224x224 (batch 64)")
@@ -318,9 +332,9 @@ def main():
 
     mode = "eager"
     graph_check = None
-    model, opt, x, y = build_training(dev)
+    model, opt, x, y = build_training(dev, which=args.model)
     if not args.no_graph:
-        ok, worst, losses = graph_matches_eager(dev)
+        ok, worst, losses = graph_matches_eager(dev, replays=4 if args.model == "resnet20" else 2, which=args.model)
         graph_check = {"ok": ok, "max_param_diff_vs_eager_step": worst,
                        "loss_graph_vs_eager": [[round(a, 6), round(b, 6)] for a, b in losses]}
         if ok:
@@ -339,6 +353,18 @@ def main():
         run()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    if args.model != "resnet20":
+        batch, size, classes = MODELS[args.model]
+        print(json.dumps({
+            "metric": f"{args.model} AdderNet train ms/batch (bs{batch})", "value": round(ms, 3), "unit": "ms/batch",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
+            "higher_is_better": False, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": f"{args.model} AdderNet, batch {batch}, 3x{size}x{size}, {classes} classes, SGD "
+                                   "momentum 0.9 lr 0.1 wd 5e-4, adaptive eta 0.1, fwd+bwd+optimizer",
+                       "step_mode": mode},
+            "images_per_s": round(batch / ms * 1e3, 1), "graph_check": graph_check}))
+        return
 
     out = {
         "metric": "ResNet-20 AdderNet train ms/batch (bs256)", "value": round(ms, 3), "unit": "ms/batch",

@@ -1,0 +1,131 @@
+"""The larger networks of the reference (models.py) as callers of the adder layer: module layout and
+state_dict keys on the CPU, one training step against the oracle-built network on the GPU."""
+import copy
+import statistics
+
+import pytest
+import torch
+
+
+def _oracle_layer():
+    from oracle import adder_oracle
+    return adder_oracle.adder2d
+
+
+def test_resnet50_keys_and_cpu_forward():
+    from addernetcuda_amd.models import resnet50
+    torch.manual_seed(0)
+    net = resnet50(num_classes=7, adder2d_cls=_oracle_layer())
+    keys = set(net.state_dict())
+    for k in ("conv1.weight", "bn1.running_var", "layer1.0.conv1.adder", "layer1.0.conv3.adder",
+              "layer1.0.downsample.0.adder", "layer1.0.downsample.1.weight", "layer2.3.conv2.adder",
+              "layer3.5.bn3.bias", "layer4.2.conv3.adder", "fc.weight", "fc.bias", "bn2.num_batches_tracked"):
+        assert k in keys, k
+    assert net.layer2[0].conv2.stride == 2 and net.layer2[0].downsample[0].stride == 2
+    assert tuple(net.layer4[2].conv3.adder.shape) == (2048, 512, 1, 1)
+    # the stock-module build has the same parameters and buffers
+    plain = resnet50(num_classes=7, adder2d_cls=_oracle_layer(), fused=False)
+    assert set(plain.state_dict()) == keys
+    plain.load_state_dict(net.state_dict())
+    x = torch.randn(2, 3, 32, 32)
+    a, b = net(x), plain(x)
+    assert a.shape == (2, 7) and torch.allclose(a, b, rtol=1e-4, atol=1e-4)
+
+
+def test_vgg_small_layout_and_cpu_forward():
+    from addernetcuda_amd.models import vgg_small
+    torch.manual_seed(0)
+    net = vgg_small(adder2d_cls=_oracle_layer())
+    adders = [k for k in net.state_dict() if k.endswith(".adder")]
+    assert len(adders) == 5 and "features.0.weight" in net.state_dict()
+    allad = vgg_small(adder2d_cls=_oracle_layer(), first_adder=True)
+    assert tuple(allad.state_dict()["features.0.adder"].shape) == (128, 3, 3, 3)
+    plain = vgg_small(adder2d_cls=_oracle_layer(), fused=False)
+    x = torch.randn(2, 3, 32, 32)
+    assert net(x).shape == (2, 10) and plain(x).shape == (2, 10)
+
+
+def _one_step(model, x, y):
+    for p in model.parameters():
+        p.grad = None
+    logits = model(x)
+    loss = torch.nn.functional.cross_entropy(logits, y)
+    loss.backward()
+    return logits.detach().double(), loss.item()
+
+
+def _grad_deviation(model, truth):
+    pm, pt = dict(model.named_parameters()), dict(truth.named_parameters())
+    # a classifier bias in front of a BatchNorm has a true gradient of zero up to rounding: such tensors (largest
+    # entry below 1e-6 of the largest gradient entry of the network) are left out
+    top = max(p.grad.abs().max().item() for p in pt.values())
+    return {n: (pm[n].grad.double() - pt[n].grad).abs().max().item() / pt[n].grad.abs().max().item()
+            for n in pm if pt[n].grad.abs().max().item() > 1e-6 * top}
+
+
+def _compare_with_oracle_build(hip, ref, x, y):
+    """One forward + backward of `hip` (the HIP layer) and of `ref` (the same network and weights on the oracle
+    layer), the latter in float32 and in float64.  Logits and loss must agree with the float64 run.  Gradients
+    behind tens of BatchNorm + ReLU stages cannot agree element-wise: a 1e-6 difference in an activation flips
+    the occasional ReLU gate and every gradient below it moves by percents (with a handful of samples per
+    BatchNorm channel in the last stages, by more).  The reference formulation's own float32 evaluation shows
+    how much; the HIP path may deviate from float64 by at most three times as much (plus 0.01 on the median
+    over all gradient tensors and 0.1 on the worst one), the kernels themselves being held to rtol 1e-5 /
+    atol 1e-4 per layer by the parity tests."""
+    ref.load_state_dict(hip.state_dict())
+    ref64 = copy.deepcopy(ref).double()
+    lh, losh = _one_step(hip, x, y)
+    l32, los32 = _one_step(ref, x, y)
+    l64, los64 = _one_step(ref64, x.double(), y)
+    noise = max((l32 - l64).abs().max().item(), 1e-4)
+    assert (lh - l64).abs().max().item() <= 5 * noise + 2e-3, ((lh - l64).abs().max().item(), noise)
+    assert abs(losh - los64) <= 5 * max(abs(los32 - los64), 1e-5) + 1e-3 * abs(los64), (losh, los32, los64)
+    dh, dr = _grad_deviation(hip, ref64), _grad_deviation(ref, ref64)
+    worst = max(dh, key=dh.get)
+    assert dh[worst] <= 3 * max(dr.values()) + 0.1, (worst, dh[worst], max(dr.values()))
+    mh, mr = statistics.median(dh.values()), statistics.median(dr.values())
+    assert mh <= 3 * mr + 0.01, (mh, mr, sorted(dh.items(), key=lambda kv: -kv[1])[:5])
+    return mh, dh[worst], worst
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [True, False])
+def test_resnet50_one_block_per_stage_matches_the_oracle_built_network(gpu, fused):
+    """Every kind of bottleneck block once (downsample, stride 1 and 2, 64 to 2048 channels), 13 adder layers
+    deep: shallow enough for absolute bounds as well (those of the ResNet-20 test)."""
+    from addernetcuda_amd.models import ResNet50
+    torch.manual_seed(3)
+    hip = ResNet50((1, 1, 1, 1), num_classes=10, eta=0.1, fused=fused).to(gpu)
+    ref = ResNet50((1, 1, 1, 1), num_classes=10, eta=0.1, adder2d_cls=_oracle_layer(), fused=fused).to(gpu)
+    g = torch.Generator(device=gpu).manual_seed(4)
+    x = torch.randn(8, 3, 64, 64, device=gpu, generator=g)
+    y = torch.randint(0, 10, (8,), device=gpu, generator=g)
+    median, worst, name = _compare_with_oracle_build(hip, ref, x, y)
+    assert median <= 0.02 and worst <= 0.15, (median, worst, name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [True, False])
+def test_resnet50_step_matches_the_oracle_built_network(gpu, fused):
+    """The full-depth ResNet-50 AdderNet (53 adder layers, 64x64 inputs, batch 4)."""
+    from addernetcuda_amd.models import resnet50
+    torch.manual_seed(5)
+    hip = resnet50(num_classes=10, eta=0.1, fused=fused).to(gpu)
+    ref = resnet50(num_classes=10, eta=0.1, adder2d_cls=_oracle_layer(), fused=fused).to(gpu)
+    g = torch.Generator(device=gpu).manual_seed(6)
+    x = torch.randn(4, 3, 64, 64, device=gpu, generator=g)
+    y = torch.randint(0, 10, (4,), device=gpu, generator=g)
+    _compare_with_oracle_build(hip, ref, x, y)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("first_adder", [False, True])
+def test_vgg_small_step_matches_the_oracle_built_network(gpu, first_adder):
+    from addernetcuda_amd.models import vgg_small
+    torch.manual_seed(7)
+    hip = vgg_small(eta=0.1, first_adder=first_adder).to(gpu)
+    ref = vgg_small(eta=0.1, adder2d_cls=_oracle_layer(), first_adder=first_adder).to(gpu)
+    g = torch.Generator(device=gpu).manual_seed(8)
+    x = torch.randn(8, 3, 32, 32, device=gpu, generator=g)
+    y = torch.randint(0, 10, (8,), device=gpu, generator=g)
+    _compare_with_oracle_build(hip, ref, x, y)
