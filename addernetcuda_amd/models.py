@@ -1,4 +1,4 @@
-"""The reference's two larger AdderNets as callers of ``adder2d``: ResNet-50 and a VGG-small stack.
+"""The reference's other AdderNets as callers of ``adder2d``: ResNet-50, a VGG-small stack and the CIFAR DenseNet.
 
 ``resnet50`` has the architecture, parameter names and state_dict keys of the reference's resnet50.py:19-119:
 a regular 7x7 stride-2 stem convolution, BatchNorm, ReLU and 3x3 max pooling (resnet50.py:63-67), four stages
@@ -11,13 +11,24 @@ with conv - BatchNorm - ReLU units as built by vgg.py:66-80; the layers are adde
 except, by default, the first one on the 3-channel image (``first_adder=True`` makes that one an adder layer
 too, as vgg.py does), and a linear classifier.
 
-Both take ``adder2d_cls`` to build the same network around another implementation of the layer (the tests do
+``densenet_cifar`` has the architecture and state_dict keys of the reference's densenet.py:9-109: a regular 3x3
+stem convolution (densenet.py:41), four dense stages of [6, 12, 24, 16] pre-activation bottlenecks (BatchNorm - ReLU
+- adder2d 1x1 to 4 x growth channels - BatchNorm - ReLU - adder2d 3x3 to ``growth_rate`` = 12 channels, output
+concatenated in front of the input, densenet.py:9-21), transitions of BatchNorm - ReLU - adder2d 1x1 halving the
+channels - 2x2 average pooling (densenet.py:24-33), BatchNorm - ReLU - 4x4 average pooling - linear classifier
+(densenet.py:67-68, 92-95).  Its layers have channel counts that are multiples of 12, not of 16.
+
+All take ``adder2d_cls`` to build the same network around another implementation of the layer (the tests do
 this with their CPU reference), and ``fused=False`` to build it from stock ``nn.BatchNorm2d`` / ``nn.ReLU``
 modules exactly as the reference's model files do -- the adder layers are then the only thing that differs
 from the reference.  With ``fused=True`` the BatchNorm layers are ``BatchNormAct2d`` (same parameters, buffers
 and keys) and take their statistics from the adder kernels' epilogue.
 """
+import math
+
+import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import adder as _adder
 from .bn_act import BatchNormAct2d
@@ -163,3 +174,78 @@ class VGGSmall(nn.Module):
 
 def vgg_small(**kwargs):
     return VGGSmall(**kwargs)
+
+
+class _PreAct:
+    """BatchNorm - ReLU in front of a layer: one fused module, or the stock BatchNorm followed by F.relu."""
+
+    @staticmethod
+    def make(channels, fused):
+        return BatchNormAct2d(channels, relu=True) if fused else nn.BatchNorm2d(channels)
+
+
+def _bn_relu(bn, x):
+    return bn(x) if isinstance(bn, BatchNormAct2d) else F.relu(bn(x))
+
+
+class DenseBottleneck(nn.Module):
+    def __init__(self, in_planes, growth_rate, adder2d_cls=None, fused=True, **adder_kw):
+        super().__init__()
+        make = adder2d_cls or _adder.adder2d
+        self.bn1 = _PreAct.make(in_planes, fused)
+        self.conv1 = make(in_planes, 4 * growth_rate, kernel_size=1, bias=False, **adder_kw)
+        self.bn2 = _PreAct.make(4 * growth_rate, fused)
+        self.conv2 = make(4 * growth_rate, growth_rate, kernel_size=3, padding=1, bias=False, **adder_kw)
+
+    def forward(self, x):
+        y = self.conv1(_bn_relu(self.bn1, x))
+        y = self.conv2(_bn_relu(self.bn2, y))
+        return torch.cat([y, x], 1)
+
+
+class Transition(nn.Module):
+    def __init__(self, in_planes, out_planes, adder2d_cls=None, fused=True, **adder_kw):
+        super().__init__()
+        make = adder2d_cls or _adder.adder2d
+        self.bn = _PreAct.make(in_planes, fused)
+        self.conv = make(in_planes, out_planes, kernel_size=1, bias=False, **adder_kw)
+
+    def forward(self, x):
+        return F.avg_pool2d(self.conv(_bn_relu(self.bn, x)), 2)
+
+
+class DenseNet(nn.Module):
+    def __init__(self, num_block=(6, 12, 24, 16), growth_rate=12, reduction=0.5, num_classes=10, adder2d_cls=None,
+                 fused=True, **adder_kw):
+        super().__init__()
+        self.growth_rate = growth_rate
+        kw = dict(adder2d_cls=adder2d_cls, fused=fused, **adder_kw)
+        planes = 2 * growth_rate
+        self.conv1 = nn.Conv2d(3, planes, kernel_size=3, padding=1, bias=False)
+        for i, blocks in enumerate(num_block, start=1):
+            stage = []
+            for _ in range(blocks):
+                stage.append(DenseBottleneck(planes, growth_rate, **kw))
+                planes += growth_rate
+            setattr(self, f"dense{i}", nn.Sequential(*stage))
+            if i < len(num_block):
+                out_planes = int(math.floor(planes * reduction))
+                setattr(self, f"trans{i}", Transition(planes, out_planes, **kw))
+                planes = out_planes
+        self.stages = len(num_block)
+        self.bn = _PreAct.make(planes, fused)
+        self.linear = nn.Linear(planes, num_classes)
+
+    def forward(self, x):
+        x = self.conv1(x)
+        for i in range(1, self.stages + 1):
+            x = getattr(self, f"dense{i}")(x)
+            if i < self.stages:
+                x = getattr(self, f"trans{i}")(x)
+        x = F.avg_pool2d(_bn_relu(self.bn, x), 4)
+        return self.linear(x.view(x.size(0), -1))
+
+
+def densenet_cifar(**kwargs):
+    """densenet.py:108-109."""
+    return DenseNet((6, 12, 24, 16), growth_rate=12, **kwargs)

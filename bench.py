@@ -188,10 +188,11 @@ def make_step(model, opt, x, y):
 
 
 # the reference's three model configurations: (batch, input size, classes)
-MODELS = {"resnet20": (BATCH, 32, 10), "vgg_small": (128, 32, 10), "resnet50": (64, 224, 1000)}
+MODELS = {"resnet20": (BATCH, 32, 10), "vgg_small": (128, 32, 10), "resnet50": (64, 224, 1000),
+          "densenet_cifar": (64, 32, 10)}
 
 
-def build_training(dev, seed=0, which="resnet20"):
+def build_training(dev, seed=0, which="resnet20", fused=True):
     torch.manual_seed(seed)
     batch, size, classes = MODELS[which]
     if which == "resnet20":
@@ -199,7 +200,7 @@ def build_training(dev, seed=0, which="resnet20"):
         model = resnet20(eta=ETA)
     else:
         from addernetcuda_amd import models
-        model = getattr(models, which)(num_classes=classes, eta=ETA)
+        model = getattr(models, which)(num_classes=classes, eta=ETA, fused=fused)
     model = model.to(dev)
     # fused=True: the same update as the default implementation, in one kernel per parameter group
     opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4, fused=True)
@@ -230,14 +231,14 @@ def capture_step(model, opt, x, y):
     return graph, loss
 
 
-def graph_matches_eager(dev, replays=4, which="resnet20"):
+def graph_matches_eager(dev, replays=4, which="resnet20", fused=True):
     """Replay the captured step from a saved state and run the eager step from the same state, several times.
 
     Torch's own kernels are not run-to-run deterministic, so trajectories cannot be compared over many steps;
     one step from identical weights, momentum and BatchNorm statistics can.
     """
     import copy
-    model, opt, x, y = build_training(dev, which=which)
+    model, opt, x, y = build_training(dev, which=which, fused=fused)
     graph, loss = capture_step(model, opt, x, y)
     eager = make_step(model, opt, x, y)
     worst = 0.0
@@ -304,6 +305,9 @@ def main():
                     help="resnet20 (default) is the benchmark; vgg_small (batch 128) and resnet50 (batch 64, 224x224) "
                          "time the training step of the reference's two other model configurations and print a "
                          "shorter line")
+    ap.add_argument("--stock-modules", action="store_true",
+                    help="with --model vgg_small / resnet50 / densenet_cifar: build the network from stock "
+                         "nn.BatchNorm2d / ReLU modules as the reference's model files do (only the adder layers differ)")
     ap.add_argument("--layer-set", choices=sorted(LAYER_SETS), default="resnet20",
                     help="with --layers-only: the adder layers of ResNet-20 (batch 256), the VGG-small stack "
                          "(batch 128) or ResNet-50 at 224x224 (batch 64)")
@@ -332,9 +336,11 @@ def main():
 
     mode = "eager"
     graph_check = None
-    model, opt, x, y = build_training(dev, which=args.model)
+    fused = not args.stock_modules
+    model, opt, x, y = build_training(dev, which=args.model, fused=fused)
     if not args.no_graph:
-        ok, worst, losses = graph_matches_eager(dev, replays=4 if args.model == "resnet20" else 2, which=args.model)
+        ok, worst, losses = graph_matches_eager(dev, replays=4 if args.model == "resnet20" else 2, which=args.model,
+                                                fused=fused)
         graph_check = {"ok": ok, "max_param_diff_vs_eager_step": worst,
                        "loss_graph_vs_eager": [[round(a, 6), round(b, 6)] for a, b in losses]}
         if ok:
@@ -362,7 +368,8 @@ def main():
             "higher_is_better": False, "dtype": "f32", "data": "synthetic",
             "config": {"workload": f"{args.model} AdderNet, batch {batch}, 3x{size}x{size}, {classes} classes, SGD "
                                    "momentum 0.9 lr 0.1 wd 5e-4, adaptive eta 0.1, fwd+bwd+optimizer",
-                       "step_mode": mode},
+                       "step_mode": mode,
+                       "modules": "fused BatchNorm+ReLU kernels" if fused else "stock nn.BatchNorm2d / ReLU"},
             "images_per_s": round(batch / ms * 1e3, 1), "graph_check": graph_check}))
         return
 

@@ -45,6 +45,23 @@ def test_vgg_small_layout_and_cpu_forward():
     assert net(x).shape == (2, 10) and plain(x).shape == (2, 10)
 
 
+def test_densenet_keys_and_cpu_forward():
+    from addernetcuda_amd.models import densenet_cifar
+    torch.manual_seed(0)
+    net = densenet_cifar(adder2d_cls=_oracle_layer())
+    sd = net.state_dict()
+    assert tuple(sd["dense1.0.conv1.adder"].shape) == (48, 24, 1, 1)
+    assert tuple(sd["dense1.5.conv2.adder"].shape) == (12, 48, 3, 3)
+    assert tuple(sd["trans1.conv.adder"].shape) == (48, 96, 1, 1)
+    assert tuple(sd["dense4.15.conv1.adder"].shape) == (48, 372, 1, 1) and sd["linear.weight"].shape == (10, 384)
+    plain = densenet_cifar(adder2d_cls=_oracle_layer(), fused=False)
+    assert set(plain.state_dict()) == set(sd)
+    plain.load_state_dict(sd)
+    x = torch.randn(2, 3, 32, 32)
+    a, b = net(x), plain(x)
+    assert a.shape == (2, 10) and torch.allclose(a, b, rtol=1e-4, atol=1e-4)
+
+
 def _one_step(model, x, y):
     for p in model.parameters():
         p.grad = None
@@ -128,4 +145,18 @@ def test_vgg_small_step_matches_the_oracle_built_network(gpu, first_adder):
     g = torch.Generator(device=gpu).manual_seed(8)
     x = torch.randn(8, 3, 32, 32, device=gpu, generator=g)
     y = torch.randint(0, 10, (8,), device=gpu, generator=g)
+    _compare_with_oracle_build(hip, ref, x, y)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [True, False])
+def test_densenet_step_matches_the_oracle_built_network(gpu, fused):
+    """The CIFAR DenseNet (119 adder layers with 12 to 372 input channels), batch 4."""
+    from addernetcuda_amd.models import densenet_cifar
+    torch.manual_seed(9)
+    hip = densenet_cifar(eta=0.1, fused=fused).to(gpu)
+    ref = densenet_cifar(eta=0.1, adder2d_cls=_oracle_layer(), fused=fused).to(gpu)
+    g = torch.Generator(device=gpu).manual_seed(10)
+    x = torch.randn(4, 3, 32, 32, device=gpu, generator=g)
+    y = torch.randint(0, 10, (4,), device=gpu, generator=g)
     _compare_with_oracle_build(hip, ref, x, y)
