@@ -324,14 +324,20 @@ using FwdW8S2  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 1, 2>;    // stride 2, outputs
 // channels (8 weights, 64 vector instructions), eight output-channel waves share the staged x tile.
 using Fwd1x1   = Tile3x3Cfg<4, 64, 1, 1, 4, 8, 16, 8, 1, 1>;   // 256 positions of one image x 32 channels
 using Fwd1x1s  = Tile3x3Cfg<4, 16, 1, 4, 4, 8, 16, 8, 1, 1>;   // planes of <= 64 positions: four images
+// the same two with units of four input channels, for channel counts that are multiples of 4 but not of 8
+// (DenseNet's multiples of 12)
+using Fwd1x1q  = Tile3x3Cfg<4, 64, 1, 1, 4, 8, 16, 4, 1, 1>;
+using Fwd1x1sq = Tile3x3Cfg<4, 16, 1, 4, 4, 8, 16, 4, 1, 1>;
 
 // which tiled kernel serves these dimensions (0 = none): 1..3 3x3 stride 1 by output width, 4..5 3x3 stride 2,
-// 6..7 1x1 stride 1 by plane size, 8..9 1x1 with a stride (the sampled positions walked like a stride-1 plane)
+// 6..7 1x1 stride 1 by plane size, 8..9 1x1 with a stride (the sampled positions walked like a stride-1 plane),
+// 10..13 = 6..9 with units of four input channels
 static int fwd_tiled_variant(const ConvDims &d) {
     // (below 64 input channels the plain 1x1 kernel of conv1x1.hip is as fast or faster)
-    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.Ci % Fwd1x1::CQ == 0 && d.Ci >= 64) {
-        if (d.stride == 1) return d.H * d.W > 64 ? 6 : 7;
-        return d.Ho * d.Wo > 64 ? 8 : 9;
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.Ci % Fwd1x1q::CQ == 0 && d.Ci >= 64) {
+        const int quad = d.Ci % Fwd1x1::CQ ? 4 : 0;
+        if (d.stride == 1) return (d.H * d.W > 64 ? 6 : 7) + quad;
+        return (d.Ho * d.Wo > 64 ? 8 : 9) + quad;
     }
     if (d.kh != 3 || d.kw != 3 || d.pad != 1) return 0;
     if (d.stride == 1) return d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
@@ -360,6 +366,10 @@ int fwd_stats_slots(const ConvDims &d) {
         case 7: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
         case 8: return stats_slots_3x3<Fwd1x1>(as_one_row(d));
         case 9: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
+        case 10: return stats_slots_3x3<Fwd1x1q>(as_one_row(d));
+        case 11: return stats_slots_3x3<Fwd1x1sq>(as_one_row(d));
+        case 12: return stats_slots_3x3<Fwd1x1q>(as_one_row(d));
+        case 13: return stats_slots_3x3<Fwd1x1sq>(as_one_row(d));
         default: return conv1x1_supported(d, nullptr, nullptr) ? fwd_1x1_stats_slots(d) : 0;
     }
 }
@@ -371,16 +381,23 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
                       (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                       (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0);
     const int variant = fwd_tiled_variant(d);
-    if (variant >= 8) {   // x is read element by element; y is a dense row per plane
+    const bool strided = variant == 8 || variant == 9 || variant == 12 || variant == 13;
+    if (strided) {   // x is read element by element; y is a dense row per plane
         const ConvDims f = as_one_row(d);
-        if (f.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0)
-            return variant == 8 ? launch_fwd_3x3_v<Fwd1x1, false, true>(x, w, y, stats, f, s, sampling_of(d))
-                                : launch_fwd_3x3_v<Fwd1x1s, false, true>(x, w, y, stats, f, s, sampling_of(d));
+        if (f.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0) switch (variant) {
+            case 8: return launch_fwd_3x3_v<Fwd1x1, false, true>(x, w, y, stats, f, s, sampling_of(d));
+            case 9: return launch_fwd_3x3_v<Fwd1x1s, false, true>(x, w, y, stats, f, s, sampling_of(d));
+            case 12: return launch_fwd_3x3_v<Fwd1x1q, false, true>(x, w, y, stats, f, s, sampling_of(d));
+            default: return launch_fwd_3x3_v<Fwd1x1sq, false, true>(x, w, y, stats, f, s, sampling_of(d));
+        }
     } else if (variant >= 6) {
         const ConvDims f = as_one_row(d);
-        if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0)
-            return variant == 6 ? launch_fwd_3x3<Fwd1x1>(x, w, y, stats, f, s)
-                                : launch_fwd_3x3<Fwd1x1s>(x, w, y, stats, f, s);
+        if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0) switch (variant) {
+            case 6: return launch_fwd_3x3<Fwd1x1>(x, w, y, stats, f, s);
+            case 7: return launch_fwd_3x3<Fwd1x1s>(x, w, y, stats, f, s);
+            case 10: return launch_fwd_3x3<Fwd1x1q>(x, w, y, stats, f, s);
+            default: return launch_fwd_3x3<Fwd1x1sq>(x, w, y, stats, f, s);
+        }
     }
     if (k3p1) {
         switch (variant) {

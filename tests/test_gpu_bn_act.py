@@ -80,6 +80,7 @@ STATS_CASES = [
     (2, 16, 14, 14, 20, 3, 1, 1), (2, 9, 10, 18, 8, 3, 1, 1),
     (2, 16, 32, 32, 32, 1, 2, 0), (3, 32, 16, 16, 64, 1, 2, 0), (2, 8, 8, 8, 4, 1, 1, 0), (3, 12, 7, 7, 20, 1, 1, 0),
     (2, 6, 9, 9, 10, 1, 2, 0), (3, 64, 14, 14, 72, 1, 1, 0), (2, 64, 28, 28, 72, 1, 2, 0),   # 1x1 kernels, element-wise and tiled
+    (3, 84, 16, 16, 48, 1, 1, 0), (5, 68, 8, 8, 20, 1, 1, 0), (2, 76, 20, 20, 24, 1, 2, 0),   # ... units of four input channels
 ]
 
 

@@ -26,6 +26,10 @@ SHAPES = [
     (3, 48, 32, 32, 12, 3, 1, 1),      # DenseNet-BC growth conv, Co = 12
     (1, 32, 16, 16, 640, 3, 2, 1),     # strided 3x3 with > 2304 terms per input position (three-instruction grad_X form)
     (64, 1024, 7, 7, 64, 1, 1, 0),     # 1x1 on 49-position planes with many images x channel blocks (the larger small-plane grad_X tile)
+    (3, 84, 32, 32, 48, 1, 1, 0),      # DenseNet 1x1 with >= 64 input channels, a multiple of 4 but not of 8
+    (5, 132, 8, 8, 48, 1, 1, 0),       # ... on 64-position planes
+    (6, 372, 4, 4, 48, 1, 1, 0),       # ... the last dense stage: 16-position planes
+    (2, 180, 16, 16, 96, 1, 2, 0),     # ... with a stride
 ]
 
 
@@ -45,7 +49,8 @@ def test_layer_matches_oracle(case, gpu):
 
 
 @pytest.mark.parametrize("case", [(2, 64, 28, 28, 96, 1, 2, 0), (2, 128, 14, 14, 64, 1, 2, 0), (1, 64, 9, 9, 64, 1, 3, 0),
-                                  (3, 64, 7, 7, 128, 1, 2, 0), (2, 72, 10, 6, 64, 1, 2, 0), (5, 64, 8, 8, 64, 1, 4, 0)], ids=str)
+                                  (3, 64, 7, 7, 128, 1, 2, 0), (2, 72, 10, 6, 64, 1, 2, 0), (5, 64, 8, 8, 64, 1, 4, 0),
+                                  (2, 68, 18, 18, 40, 1, 2, 0), (3, 76, 7, 9, 64, 1, 3, 0)], ids=str)
 def test_strided_1x1_with_many_channels_walks_the_sampled_positions(case, gpu):
     """From 64 channels on, the tiled kernels walk the sampled positions x[:, :, ::s, ::s] of a strided 1x1
     layer like a stride-1 plane; results and both gradients (the input gradient stored together with the
