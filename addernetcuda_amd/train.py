@@ -153,14 +153,28 @@ def train_one_epoch(net, opt, x_u8, y, batch, generator=None, graphed=None):
     return torch.stack(losses).mean().item()
 
 
+ARCHS = ("resnet20", "vgg_small", "densenet_cifar", "resnet50")
+
+
+def build_network(arch, eta, num_classes=10):
+    """The reference's networks for 32x32 inputs (main.py:66 builds resnet20; vgg.py, densenet.py and resnet50.py
+    are its other model files)."""
+    if arch == "resnet20":
+        from addernetcuda_amd.resnet20 import resnet20
+        return resnet20(eta=eta, num_classes=num_classes)
+    if arch not in ARCHS:
+        raise ValueError(f"unknown architecture {arch!r}: one of {ARCHS}")
+    from addernetcuda_amd import models
+    return getattr(models, arch)(eta=eta, num_classes=num_classes)
+
+
 def run(args):
     if not torch.cuda.is_available():
         raise RuntimeError("addernetcuda_amd.train needs an MI355X: the adder kernels have no CPU path")
-    from addernetcuda_amd.resnet20 import resnet20
     dev = torch.device("cuda:0")
     torch.manual_seed(args.seed)
     data = synthetic_arrays(args.synthetic, dev, seed=args.seed) if args.data is None else load_arrays(args.data, dev)
-    net = resnet20(eta=args.eta).to(dev)
+    net = build_network(args.arch, args.eta).to(dev)
     if args.resume:
         net.load_state_dict(torch.load(args.resume, map_location=dev, weights_only=True))
     # the learning rate lives on the device so that the captured step sees each epoch's value
@@ -197,7 +211,7 @@ def run(args):
 
 
 def parse_args(argv=None):
-    p = argparse.ArgumentParser(description="train the ResNet-20 AdderNet on an MI355X")
+    p = argparse.ArgumentParser(description="train an AdderNet (ResNet-20 by default) on an MI355X")
     p.add_argument("--data", type=str, default=None, help=".npz with x_train, y_train, x_test, y_test (uint8 images)")
     p.add_argument("--synthetic", type=int, default=8192, help="training-set size when --data is not given")
     p.add_argument("--output-dir", type=str, default="./models/")
@@ -210,6 +224,7 @@ def parse_args(argv=None):
     p.add_argument("--eta", type=float, default=0.2, help="adaptive grad_W scale, adder.py:78 uses 1/5")
     p.add_argument("--no-graph", action="store_true", help="run every training step eagerly instead of as a HIP graph")
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--arch", choices=ARCHS, default="resnet20", help="network (main.py:66 trains resnet20)")
     return p.parse_args(argv)
 
 

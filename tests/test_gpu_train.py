@@ -30,3 +30,15 @@ def test_two_epochs_learn_and_checkpoint(gpu, tmp_path):
     ev = train.run(train.parse_args(["--synthetic", "2000", "--resume", ckpt, "--eval-only", "--test-batch-size", "50",
                                      "--seed", "1"]))
     assert abs(ev[0]["accuracy"] - best) < 1e-6
+
+
+def test_other_architectures_train(gpu, tmp_path):
+    """--arch: the VGG-small stack through the same loop (graph capture included)."""
+    from addernetcuda_amd import train
+    hist = train.run(train.parse_args(["--arch", "vgg_small", "--synthetic", "2000", "--epochs", "6", "--batch-size", "100",
+                                       "--test-batch-size", "50", "--output-dir", str(tmp_path), "--seed", "2"]))
+    assert len(hist) == 6 and all(h["train_loss"] == h["train_loss"] for h in hist)      # finite, not NaN
+    assert hist[-1]["train_loss"] < hist[0]["train_loss"]
+    assert max(h["accuracy"] for h in hist) > 0.4          # 0.72 when written
+    state = torch.load(os.path.join(str(tmp_path), "addernet.pt"), map_location="cpu", weights_only=True)
+    assert "features.2.adder" in state and "classifier.weight" in state
