@@ -189,63 +189,110 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
-        // Software pipeline over the output channels of the chunk, in units of HM input channels
-        // (9*HM contiguous weights): right after the first instruction of a unit, i.e. after the
-        // wait for its operands, the weights of the next unit and (once per output channel) the
-        // gy strips of the next channel are requested.
-        static_assert(CQ == 1, "pipeline is written for one output channel per step");
-        // input channels per unit: keeps ~100 vector instructions per unit and both weight
-        // buffers (2 * 9 * HM SGPRs) well inside the scalar register file
-        constexpr int HM = KS == 1 ? TM : (TN >= 4 ? 1 : 2), NU = TM / HM, HW = HM * KK;
-        static_assert(TM % HM == 0 && (NU % 2 == 0 || NU == 1), "one unit or an even number of units per output channel");
-        float gr[2][KS][TN + KS - 1];
-        float wv[2][HW];
+        if constexpr (KS == 1 && CQ > 1) {
+            // Single tap: a unit of one output channel would be TM * TN terms, too few instructions to hide the wait
+            // for its operands behind -- a unit is CQ output channels here (CQ * TM weights, CQ gy strips).
+            constexpr int CU = CQ;
+            static_assert(C::CC % CU == 0, "a chunk holds whole units (planes past Co are staged as zeros)");
+            float gr[2][CU][TN];
+            float wv[2][CU * TM];
 #pragma unroll
-        for (int i = 0; i < KS; ++i) lds_read_strip<TN + KS - 1, C::STRIP_ALIGN>(lbase + i * C::PITCH, gr[0][i]);
+            for (int u = 0; u < CU; ++u) {
+                lds_read_strip<TN, C::STRIP_ALIGN>(lbase + u * C::PLANE, gr[0][u]);
+                const int wrow = min(co0 + u, Co - 1) * K;   // rows past Co meet gy = 0: any finite weight will do
 #pragma unroll
-        for (int e = 0; e < HW; ++e) wv[0][e] = wc[co0 * K + e];
-
-        auto one_channel = [&](const int cc, const int cur) {
-            const int kofs = (co0 + cc) * K;
-            const bool more = cc + 1 < ccnt;
-            const int knext = more ? kofs + K : kofs;
+                for (int e = 0; e < TM; ++e) wv[0][u * TM + e] = wc[wrow + e];
+            }
+            auto unit = [&](const int cc, const int cur) {
+                const bool more = cc + CU < ccnt;
+                const int cnext = more ? cc + CU : cc;
 #pragma unroll
-            for (int h = 0; h < NU; ++h) {
-                // weight buffer of this unit: the buffers alternate from unit to unit, also across channels
-                const int wb = (cur * (NU & 1) + h) & 1;
-#pragma unroll
-                for (int idx = 0; idx < HM * KK * TN; ++idx) {
-                    const int t = idx % TN, j = (idx / TN) % KS, i = (idx / TN / KS) % KS, mm = idx / TN / KK;
-                    const int m = h * HM + mm;
-                    const float wgt = wv[wb][mm * KK + i * KS + j];
-                    const float d = SAT ? sat01(fmaf(wgt, 0.5f, cr[m][t])) : hardtanh(wgt - cr[m][t]);
-                    acc[m][t] = fmaf(d, gr[cur][KS - 1 - i][t + KS - 1 - j], acc[m][t]);
+                for (int idx = 0; idx < CU * TM * TN; ++idx) {
+                    const int t = idx % TN, mm = (idx / TN) % TM, u = idx / (TN * TM);
+                    const float wgt = wv[cur][u * TM + mm];
+                    const float d = SAT ? sat01(fmaf(wgt, 0.5f, cr[mm][t])) : hardtanh(wgt - cr[mm][t]);
+                    acc[mm][t] = fmaf(d, gr[cur][u][t], acc[mm][t]);
                     if (idx == 0) {
                         __builtin_amdgcn_sched_barrier(0);
-                        if (h + 1 < NU) {
 #pragma unroll
-                            for (int e = 0; e < HW; ++e) wv[wb ^ 1][e] = wc[kofs + (h + 1) * HW + e];
-                        } else {
+                        for (int u2 = 0; u2 < CU; ++u2) {
+                            const int wrow = min(co0 + cnext + u2, Co - 1) * K;
 #pragma unroll
-                            for (int e = 0; e < HW; ++e) wv[wb ^ 1][e] = wc[knext + e];
+                            for (int e = 0; e < TM; ++e) wv[cur ^ 1][u2 * TM + e] = wc[wrow + e];
                         }
-                        if (h == 0 && more) {
+                        if (more) {
 #pragma unroll
-                            for (int i2 = 0; i2 < KS; ++i2)
-                                lds_read_strip<TN + KS - 1, C::STRIP_ALIGN>(lbase + (cc + 1) * C::PLANE + i2 * C::PITCH,
-                                                                       gr[cur ^ 1][i2]);
+                            for (int u2 = 0; u2 < CU; ++u2)
+                                lds_read_strip<TN, C::STRIP_ALIGN>(lbase + (cc + CU + u2) * C::PLANE, gr[cur ^ 1][u2]);
                         }
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
-            }
-        };
+            };
 #pragma unroll 1
-        for (int cc = 0; cc < ccnt; cc += 2) {
-            one_channel(cc, 0);
-            if (cc + 1 < ccnt) one_channel(cc + 1, 1);
-        }
+            for (int cc = 0; cc < ccnt; cc += 2 * CU) {
+                unit(cc, 0);
+                if (cc + CU < ccnt) unit(cc + CU, 1);
+            }
+        } else {
+            // Software pipeline over the output channels of the chunk, in units of HM input channels
+            // (9*HM contiguous weights): right after the first instruction of a unit, i.e. after the
+            // wait for its operands, the weights of the next unit and (once per output channel) the
+            // gy strips of the next channel are requested.
+            static_assert(CQ == 1, "this pipeline takes one output channel per step");
+            // input channels per unit: keeps ~100 vector instructions per unit and both weight
+            // buffers (2 * 9 * HM SGPRs) well inside the scalar register file
+            constexpr int HM = KS == 1 ? TM : (TN >= 4 ? 1 : 2), NU = TM / HM, HW = HM * KK;
+            static_assert(TM % HM == 0 && (NU % 2 == 0 || NU == 1), "one unit or an even number of units per output channel");
+            float gr[2][KS][TN + KS - 1];
+            float wv[2][HW];
+#pragma unroll
+            for (int i = 0; i < KS; ++i) lds_read_strip<TN + KS - 1, C::STRIP_ALIGN>(lbase + i * C::PITCH, gr[0][i]);
+#pragma unroll
+            for (int e = 0; e < HW; ++e) wv[0][e] = wc[co0 * K + e];
 
+            auto one_channel = [&](const int cc, const int cur) {
+                const int kofs = (co0 + cc) * K;
+                const bool more = cc + 1 < ccnt;
+                const int knext = more ? kofs + K : kofs;
+#pragma unroll
+                for (int h = 0; h < NU; ++h) {
+                    // weight buffer of this unit: the buffers alternate from unit to unit, also across channels
+                    const int wb = (cur * (NU & 1) + h) & 1;
+#pragma unroll
+                    for (int idx = 0; idx < HM * KK * TN; ++idx) {
+                        const int t = idx % TN, j = (idx / TN) % KS, i = (idx / TN / KS) % KS, mm = idx / TN / KK;
+                        const int m = h * HM + mm;
+                        const float wgt = wv[wb][mm * KK + i * KS + j];
+                        const float d = SAT ? sat01(fmaf(wgt, 0.5f, cr[m][t])) : hardtanh(wgt - cr[m][t]);
+                        acc[m][t] = fmaf(d, gr[cur][KS - 1 - i][t + KS - 1 - j], acc[m][t]);
+                        if (idx == 0) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (h + 1 < NU) {
+#pragma unroll
+                                for (int e = 0; e < HW; ++e) wv[wb ^ 1][e] = wc[kofs + (h + 1) * HW + e];
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < HW; ++e) wv[wb ^ 1][e] = wc[knext + e];
+                            }
+                            if (h == 0 && more) {
+#pragma unroll
+                                for (int i2 = 0; i2 < KS; ++i2)
+                                    lds_read_strip<TN + KS - 1, C::STRIP_ALIGN>(lbase + (cc + 1) * C::PLANE + i2 * C::PITCH,
+                                                                           gr[cur ^ 1][i2]);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+            };
+#pragma unroll 1
+            for (int cc = 0; cc < ccnt; cc += 2) {
+                one_channel(cc, 0);
+                if (cc + 1 < ccnt) one_channel(cc + 1, 1);
+            }
+
+        }
 #pragma unroll
         for (int m = 0; m < TM; ++m)
 #pragma unroll
@@ -645,9 +692,9 @@ using GxW32 = Tile3x3Cfg<4, 8, 16, 1, 4, 4, 8, 1>;    // inputs 32 wide: half an
 using GxW16 = Tile3x3Cfg<4, 4, 16, 1, 4, 8, 16, 1>;   // inputs 16 wide: one image x 32 channels
 using GxW8  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 1>;    // inputs 8 wide: two images x 32 channels
 // 1x1, stride 1: (H, W) planes walked as one row; a unit is one output channel x the lane's 8 input channels
-using Gx1x1  = Tile3x3Cfg<2, 64, 1, 1, 8, 8, 16, 1, 1, 1>;    // 128 positions of one image x 64 channels
+using Gx1x1  = Tile3x3Cfg<2, 64, 1, 1, 8, 8, 16, 2, 1, 1>;    // 128 positions of one image x 64 channels
 using Gx1x1s = Tile3x3Cfg<4, 16, 1, 4, 8, 8, 16, 1, 1, 1>;    // planes of <= 64 positions: four images
-using Gx1x1t = Tile3x3Cfg<2, 32, 1, 2, 4, 8, 16, 1, 1, 1>;    // ... two images x 32 channels, where Gx1x1s would leave CUs idle
+using Gx1x1t = Tile3x3Cfg<2, 32, 1, 2, 4, 8, 16, 8, 1, 1>;    // ... two images x 32 channels, where Gx1x1s would leave CUs idle
 static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
               "the launcher checks Ci against one TM per stride");
 
