@@ -278,6 +278,9 @@ using Gm1x1s  = GwMfmaCfg<1, 1, 64, 2, 4, 4, 1, 1, 8, 1>;    // planes of <= 64 
 // waves), 64 positions per staged tile.  The 64 x 64 blocking reads every x tile Co / 64 times and every gy tile
 // Ci / 64 times, which is what bounds it on the wide layers; this one halves that (5-15 % less time).
 using Gm1x1b  = GwMfmaCfg<1, 1, 64, 1, 4, 4, 2, 2, 2, 1>;
+// the same block with 52 positions per tile (2 x 4 waves of 64 x 32, no position split): 14x14 and 7x7 planes
+// (196 = 3 x 52 + 40 and 49 positions) fill tiles of 52 to 94 %, tiles of 64 to 77 %
+using Gm1x1c  = GwMfmaCfg<1, 1, 52, 1, 4, 2, 2, 4, 1, 1>;
 
 template <class G>
 static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
@@ -306,8 +309,10 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.Ci >= 64 && d.Co >= 64) {
         const ConvDims f = mfma_one_row(d);
         if (d.Ci >= 128 && d.Co >= 128) {
-            p.variant = d.stride > 1 ? 11 : 10;                    // 11: x sampled at every stride-th row and column
-            plan_one<Gm1x1b>(f, p);
+            const bool narrow = ceil_div(f.W, Gm1x1c::TW) * Gm1x1c::TW < ceil_div(f.W, Gm1x1b::TW) * Gm1x1b::TW;
+            p.variant = (narrow ? 12 : 10) + (d.stride > 1 ? 1 : 0);   // 11, 13: x sampled at every stride-th row and column
+            if (narrow) plan_one<Gm1x1c>(f, p);
+            else plan_one<Gm1x1b>(f, p);
             return p;
         }
         p.variant = (f.W > 64 ? 6 : 7) + (d.stride > 1 ? 2 : 0);   // 8, 9: x sampled likewise
@@ -369,6 +374,13 @@ int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sg
             const Subsample sub{d.stride, d.Wo, d.W, d.H * d.W};
             return f.Wo % 4 == 0 ? launch_one_v<Gm1x1b, true, true>(gy, x, part, sgpart, f, p, s, sub)
                                  : launch_one_v<Gm1x1b, false, true>(gy, x, part, sgpart, f, p, s, sub);
+        }
+        case 12: return launch_one<Gm1x1c>(gy, x, part, sgpart, mfma_one_row(d), p, s);
+        case 13: {
+            const ConvDims f = mfma_one_row(d);
+            const Subsample sub{d.stride, d.Wo, d.W, d.H * d.W};
+            return f.Wo % 4 == 0 ? launch_one_v<Gm1x1c, true, true>(gy, x, part, sgpart, f, p, s, sub)
+                                 : launch_one_v<Gm1x1c, false, true>(gy, x, part, sgpart, f, p, s, sub);
         }
         case 8:
         case 9: {

@@ -404,18 +404,18 @@ static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w
     return check_launch();
 }
 
-template <class C>
+// picks the element-wise tile loads (rows of the staged tensor that are not whole float4 groups) and the
+// three-instruction form (more terms per output than kSatMaxTerms)
+template <class C, bool SUB = false>
 static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s, const float *gadd = nullptr) {
-    // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
+                               const ConvDims &d, hipStream_t s, const float *gadd = nullptr,
+                               const Subsample sub = Subsample{1, 0, 0, 0}) {
     const bool vec = d.W % 4 == 0;
-    if constexpr (C::KS == 3) {   // (a single tap never has that many terms per output)
-        if (d.Co * C::KK > kSatMaxTerms)
-            return vec ? launch_grad_x_3x3s1_v<C, true, false>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd)
-                       : launch_grad_x_3x3s1_v<C, false, false>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd);
-    }
-    return vec ? launch_grad_x_3x3s1_v<C, true, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd)
-               : launch_grad_x_3x3s1_v<C, false, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd);
+    if (d.Co * C::KK > kSatMaxTerms)
+        return vec ? launch_grad_x_3x3s1_v<C, true, false, SUB>(gy, x, w, gx, d, s, sub, gadd)
+                   : launch_grad_x_3x3s1_v<C, false, false, SUB>(gy, x, w, gx, d, s, sub, gadd);
+    return vec ? launch_grad_x_3x3s1_v<C, true, true, SUB>(gy, x, w, gx, d, s, sub, gadd)
+               : launch_grad_x_3x3s1_v<C, false, true, SUB>(gy, x, w, gx, d, s, sub, gadd);
 }
 
 // ---------------------------------------------------------------------------
@@ -695,6 +695,13 @@ using GxW8  = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 16, 1>;    // inputs 8 wide: two imag
 using Gx1x1  = Tile3x3Cfg<2, 64, 1, 1, 8, 8, 16, 2, 1, 1>;    // 128 positions of one image x 64 channels
 using Gx1x1s = Tile3x3Cfg<4, 16, 1, 4, 8, 8, 16, 1, 1, 1>;    // planes of <= 64 positions: four images
 using Gx1x1t = Tile3x3Cfg<2, 32, 1, 2, 4, 8, 16, 8, 1, 1>;    // ... two images x 32 channels, where Gx1x1s would leave CUs idle
+
+// Planes of <= 64 positions with few images x few channel blocks: the smaller workgroup tile, so that every CU
+// gets work (512 -> 2048 @7x7 at batch 64: 760 us with the larger tile, 305 with this one; from about two
+// workgroups per CU on the larger tile is as fast or faster).
+static bool small_plane_tile(const ConvDims &f) {
+    return (long)ceil_div(f.N, Gx1x1s::NIMG) * ceil_div(f.Ci, Gx1x1s::TM * Gx1x1s::COW) <= 256;
+}
 static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
               "the launcher checks Ci against one TM per stride");
 
@@ -723,11 +730,8 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         f.W = f.Wo = d.H * d.W;
         if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0) {
             if (f.W > 64) return launch_grad_x_3x3s1<Gx1x1>(gy, x, w, gx, f, s);
-            // few images x few channel blocks: smaller workgroup tiles so that every CU gets work (measured on
-            // 512 -> 2048 @7x7, batch 64: 760 -> 550 us; with 256 or more workgroups the larger tile is faster)
-            const long wgs = (long)ceil_div(f.N, Gx1x1s::NIMG) * ceil_div(f.Ci, Gx1x1s::TM * Gx1x1s::COW);
-            return wgs < 256 ? launch_grad_x_3x3s1<Gx1x1t>(gy, x, w, gx, f, s)
-                             : launch_grad_x_3x3s1<Gx1x1s>(gy, x, w, gx, f, s);
+            return small_plane_tile(f) ? launch_grad_x_3x3s1<Gx1x1t>(gy, x, w, gx, f, s)
+                                       : launch_grad_x_3x3s1<Gx1x1s>(gy, x, w, gx, f, s);
         }
     }
     if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride > 1 && d.Ci >= 64 && d.Co >= 64) {
@@ -736,13 +740,10 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         f.W = f.Wo = d.Ho * d.Wo;
         f.stride = 1;
         const Subsample sub{d.stride, d.Wo, d.W, d.H * d.W};
-        const bool vec = f.W % 4 == 0;
-        if (!vec || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) {
-            if (f.W > 64)
-                return vec ? launch_grad_x_3x3s1_v<Gx1x1, true, true, true>(gy, x, w, gx, f, s, sub)
-                           : launch_grad_x_3x3s1_v<Gx1x1, false, true, true>(gy, x, w, gx, f, s, sub);
-            return vec ? launch_grad_x_3x3s1_v<Gx1x1s, true, true, true>(gy, x, w, gx, f, s, sub)
-                       : launch_grad_x_3x3s1_v<Gx1x1s, false, true, true>(gy, x, w, gx, f, s, sub);
+        if (f.W % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) {
+            if (f.W > 64) return launch_grad_x_3x3s1<Gx1x1, true>(gy, x, w, gx, f, s, nullptr, sub);
+            return small_plane_tile(f) ? launch_grad_x_3x3s1<Gx1x1t, true>(gy, x, w, gx, f, s, nullptr, sub)
+                                       : launch_grad_x_3x3s1<Gx1x1s, true>(gy, x, w, gx, f, s, nullptr, sub);
         }
     }
     if (conv1x1_supported(d, gy, gx))

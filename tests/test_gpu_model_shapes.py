@@ -50,7 +50,9 @@ def test_layer_matches_oracle(case, gpu):
 
 @pytest.mark.parametrize("case", [(2, 64, 28, 28, 96, 1, 2, 0), (2, 128, 14, 14, 64, 1, 2, 0), (1, 64, 9, 9, 64, 1, 3, 0),
                                   (3, 64, 7, 7, 128, 1, 2, 0), (2, 72, 10, 6, 64, 1, 2, 0), (5, 64, 8, 8, 64, 1, 4, 0),
-                                  (2, 68, 18, 18, 40, 1, 2, 0), (3, 76, 7, 9, 64, 1, 3, 0)], ids=str)
+                                  (2, 68, 18, 18, 40, 1, 2, 0), (3, 76, 7, 9, 64, 1, 3, 0),
+                                  (2, 256, 28, 28, 128, 1, 2, 0), (3, 128, 14, 14, 256, 1, 2, 0),
+                                  (4, 1024, 14, 14, 2048, 1, 2, 0)], ids=str)
 def test_strided_1x1_with_many_channels_walks_the_sampled_positions(case, gpu):
     """From 64 channels on, the tiled kernels walk the sampled positions x[:, :, ::s, ::s] of a strided 1x1
     layer like a stride-1 plane; results and both gradients (the input gradient stored together with the
