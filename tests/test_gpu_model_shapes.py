@@ -30,6 +30,10 @@ SHAPES = [
     (5, 132, 8, 8, 48, 1, 1, 0),       # ... on 64-position planes
     (6, 372, 4, 4, 48, 1, 1, 0),       # ... the last dense stage: 16-position planes
     (2, 180, 16, 16, 96, 1, 2, 0),     # ... with a stride
+    (2, 64, 12, 12, 65, 1, 1, 0),      # 1x1 grad_X units of two output channels, odd channel count
+    (2, 64, 7, 7, 70, 1, 1, 0),        # ... units of eight output channels, 70 = 8 * 8 + 6
+    (3, 72, 14, 14, 67, 1, 2, 0),      # ... the same on a sampled (strided) layer
+    (2, 128, 5, 5, 130, 1, 1, 0),      # 128 x 128-channel weight-gradient blocks with a 2-channel tail, 25-position planes
 ]
 
 
