@@ -724,7 +724,8 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s, gadd);
     }
     if (gadd) return ADDER_ERR_UNSUPPORTED;
-    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 64) {
+        // (from 48 output channels on the tiled kernel is ahead of the plain one: DenseNet's 48-channel bottlenecks)
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 48) {
         ConvDims f = d;   // every (H, W) plane as one row of H*W positions
         f.H = f.Ho = 1;
         f.W = f.Wo = d.H * d.W;
