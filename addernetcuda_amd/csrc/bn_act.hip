@@ -63,8 +63,14 @@ __global__ __launch_bounds__(kBnThreads) void bn_partial_kernel(const float *__r
             const size_t off = ((size_t)n * C + c) * HW4 + q;
             const Pack<V> xv = ld<V>(x, off);
             if (!BWD) {
+                // squares and sums in fp64: x * x is exact there, so E[x^2] - E[x]^2 keeps its digits when
+                // |mean| >> std (a rounded fp32 square of x = -100 is already off by 5e-4)
 #pragma unroll
-                for (int e = 0; e < V; ++e) { s1 += xv.v[e]; s2 = fmaf(xv.v[e], xv.v[e], s2); }
+                for (int e = 0; e < V; ++e) {
+                    const double xd = (double)xv.v[e];
+                    a += xd;
+                    b = fma(xd, xd, b);
+                }
             } else {
                 Pack<V> g = ld<V>(dy, off);
                 if (relu && mask) {
@@ -80,7 +86,7 @@ __global__ __launch_bounds__(kBnThreads) void bn_partial_kernel(const float *__r
                 for (int e = 0; e < V; ++e) { s1 += g.v[e]; s2 = fmaf(g.v[e], (xv.v[e] - mu) * rs, s2); }
             }
         }
-        a += (double)s1;   // at most four elements per fp32 partial, everything above in fp64
+        a += (double)s1;   // backward: at most four elements per fp32 partial, everything above in fp64
         b += (double)s2;
     }
     __shared__ double ra[kBnThreads / 64], rb[kBnThreads / 64];

@@ -58,6 +58,27 @@ def test_matches_torch_in_float64(shape, relu, with_res, gpu):
     assert int(m.num_batches_tracked) == 1
 
 
+@pytest.mark.parametrize("shape", [(6, 12, 8, 8), (3, 7, 5, 3), (16, 4, 16, 32)], ids=str)
+def test_statistics_survive_a_mean_far_from_zero(shape, gpu):
+    """Inputs with |mean| = 1000 x std (x = -100 + 0.1 z): a sum of fp32 squares has no digit of the variance left;
+    the statistics pass squares and sums in float64.  No ReLU here -- with the mean kept in float32 a gate that
+    sits on a value of 1e-4 may flip, which is not what this test is about."""
+    from addernetcuda_amd.bn_act import BatchNormAct2d
+    g = torch.Generator().manual_seed(sum(shape))
+    x = torch.randn(shape, generator=g) * 0.1 - 100.0
+    dy = torch.randn(shape, generator=g)
+    m = BatchNormAct2d(shape[1], relu=False).to(gpu).train()
+    xg = x.to(gpu).requires_grad_(True)
+    y = m(xg)
+    y.backward(dy.to(gpu))
+    torch.cuda.synchronize()
+    want = _reference(x, None, m.weight.detach().cpu(), m.bias.detach().cpu(), False, dy, m.eps)
+    # x - mean carries the float32 spacing of values around 100 (7.6e-6) over a std of 0.1
+    assert_close(y, want[0], "y", rtol=1e-3, atol=1e-3)
+    assert_close(xg.grad, want[1], "dx", rtol=1e-3, atol=1e-2)
+    assert_close(m.running_var, want[6], "running_var", rtol=1e-4, atol=1e-6)
+
+
 def test_eval_mode_and_state_dict_are_those_of_batchnorm2d(gpu):
     from addernetcuda_amd.bn_act import BatchNormAct2d
     a = BatchNormAct2d(8, relu=True).to(gpu)
