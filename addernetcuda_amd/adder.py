@@ -137,9 +137,13 @@ class _adder_nchw(Function):
             if slots > 0:
                 # partial sums of out and out**2 per channel for the BatchNorm that follows (bn_act.py)
                 stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64)
-                check(lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots, *dims,
-                                                     stream_ptr(dev)), "adder_conv2d_fwd_stats_f32")
-            else:
+                status = lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots, *dims,
+                                                        stream_ptr(dev))
+                if status == -7:   # e.g. tensors that are not 16-byte aligned: the kernel that sums was turned down
+                    stats, slots = None, 0
+                else:
+                    check(status, "adder_conv2d_fwd_stats_f32")
+            if slots <= 0:
                 check(lib.adder_conv2d_fwd_f32(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_f32")
         ctx.save_for_backward(X, W)  # the NCHW input, not the 9x larger X_col the reference keeps
         ctx.dims, ctx.eta = dims, eta

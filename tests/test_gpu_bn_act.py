@@ -134,6 +134,18 @@ def test_layers_without_the_epilogue_report_none(gpu):
         assert stats is None and torch.equal(y, adder.adder2d_function(x, w, s, p))
     layer = adder.adder2d(8, 4, 3, padding=1, bias=True).to(gpu)
     assert layer.forward_with_stats(x)[1] is None          # the bias would not be in the sums
+    # a tensor that is not 16-byte aligned: whichever kernel takes it, the output is the plain call's and the
+    # statistics, if any, are its sums
+    for shape, co, k, p in (((2, 64, 8, 8), 64, 1, 0), ((2, 16, 8, 8), 8, 3, 1)):
+        numel = shape[0] * shape[1] * shape[2] * shape[3]
+        xm = torch.randn(numel + 1, device=gpu)[1:].view(shape)
+        assert xm.data_ptr() % 16 == 4
+        w = torch.randn(co, shape[1], k, k, device=gpu)
+        y, stats = adder.adder2d_function_with_stats(xm, w, 1, p)
+        want = adder.adder2d_function(xm.clone(), w, 1, p)
+        assert torch.allclose(y, want, rtol=1e-6, atol=1e-4)
+        if stats is not None:
+            assert torch.allclose(stats.sum(dim=1)[:, 0], want.double().sum(dim=(0, 2, 3)), rtol=1e-6, atol=1e-3)
 
 
 @pytest.mark.parametrize("with_res", [False, True])
