@@ -39,6 +39,23 @@ __device__ __forceinline__ float hardtanh(float v) {
     return __builtin_amdgcn_fmed3f(v, -1.0f, 1.0f);
 }
 
+// Kernels with more than 48 KB of dynamic LDS need hipFuncAttributeMaxDynamicSharedMemorySize, once per device
+// (the attribute belongs to the device's copy of the function).  One flag word per kernel instantiation.
+int record_hip_error(hipError_t e);
+template <auto Kernel>
+inline int allow_dynamic_lds(int bytes) {
+    static unsigned long long done = 0;   // bit d: set on device d (benign race: setting it twice is harmless)
+    if (bytes <= 48 * 1024) return 0;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return record_hip_error(e);
+    if (dev >= 0 && dev < 64 && ((done >> dev) & 1ull)) return 0;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return record_hip_error(e);
+    if (dev >= 0 && dev < 64) done |= 1ull << dev;
+    return 0;
+}
+
 __host__ __device__ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
 __host__ __device__ constexpr long ceil_div_l(long a, long b) { return (a + b - 1) / b; }
 __host__ __device__ constexpr int round_up(int a, int b) { return ceil_div(a, b) * b; }

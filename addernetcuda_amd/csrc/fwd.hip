@@ -273,13 +273,7 @@ static int launch_fwd_3x3_v(const float *x, const float *w, float *y, double *st
     const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gy = ceil_div(d.Co, C::TM * C::COW);
     if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    static bool attr_set = false;
-    if (!attr_set && C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_3x3_kernel<C, VEC, SUB, MUL>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-        if (e != hipSuccess) return record_hip_error(e);
-        attr_set = true;
-    }
+    if (int rc = allow_dynamic_lds<&fwd_3x3_kernel<C, VEC, SUB, MUL>>(C::LDS_BYTES)) return rc;
     hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC, SUB, MUL>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
                        stats, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, sub);
     return check_launch();

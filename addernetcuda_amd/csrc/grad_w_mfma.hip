@@ -338,13 +338,7 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
 template <class G, bool VEC, bool SUB = false>
 static int launch_one_v(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
                       const GradWMfmaPlan &p, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
-    static bool attr_set = false;
-    if (!attr_set && G::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_w_mfma_kernel<G, VEC, SUB>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
-        if (e != hipSuccess) return record_hip_error(e);
-        attr_set = true;
-    }
+    if (int rc = allow_dynamic_lds<&grad_w_mfma_kernel<G, VEC, SUB>>(G::LDS_BYTES)) return rc;
     hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC, SUB>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
                        part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles, sub);
     return check_launch();

@@ -391,14 +391,8 @@ static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    static bool attr_set = false;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
-    if (!attr_set && LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&grad_x_3x3s1_kernel<C, VEC, SAT, SUB>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-        if (e != hipSuccess) return record_hip_error(e);
-        attr_set = true;
-    }
+    if (int rc = allow_dynamic_lds<&grad_x_3x3s1_kernel<C, VEC, SAT, SUB>>(LDS_BYTES)) return rc;
     hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW, sub, gadd);
     return check_launch();
