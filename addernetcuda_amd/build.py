@@ -11,7 +11,6 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libaddernet_hip.so")
-PROBE = os.path.join(HERE, "valu_issue_probe")   # stand-alone program: the machine's vector issue ceiling
 SOURCES = ["api.hip", "fwd.hip", "grad_x.hip", "grad_w.hip", "grad_w_mfma.hip", "conv1x1.hip", "col.hip", "bn_act.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -43,13 +42,6 @@ def build(verbose=False, jobs=4):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           os.path.join(CSRC, "valu_issue_probe.hip"), "-o", PROBE]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if r.returncode:
-        raise RuntimeError("hipcc failed on valu_issue_probe.hip:\n" + r.stdout)
     return LIB
 
 

@@ -29,7 +29,7 @@ PEAK_FP64_MFMA_TFLOPS = 78.6       # MI355X fp64 matrix peak: the 3x3 weight gra
 PEAK_FP32_TFLOPS = 157.3           # MI355X vendor fp32 vector peak (256 CU x 64 lanes x 2 (packed) x 2 (FMA) x 2.4 GHz)
 # lane-instructions per second: a SIMD starts two vector instructions per 4-cycle slot when two of its
 # waves are ready (one per wave), so 256 CU x 4 SIMD x 2 x 64 lanes / 4 cycles x 2.4 GHz; with an FMA in
-# every slot this is the 157.3 TFLOP/s above.  addernetcuda_amd/valu_issue_probe measures it.
+# every slot this is the 157.3 TFLOP/s above.
 PEAK_VALU_ISSUE = 2 * 256 * 64 * 2.4e9
 BATCH = 256
 ETA = 0.1
@@ -147,31 +147,12 @@ def dominant_kernel(dev, steps):
         "algorithmic_bytes": 4 * (2 * BATCH * Ci * H * W + BATCH * Co * H * W + Co * Ci * k * k),
         "avg_launch_us": round(t * 1e6, 2), "flop_per_launch": flop,
         "valu_issue_util": round(OPS["grad_x"][1] * E / t / PEAK_VALU_ISSUE, 4),
-        "issue_probe_T_lane_instr_per_s": issue_probe(),
         "note": "fp32 VALU-bound (|a-b| accumulation has no FMA/MFMA form). The 157.3 TFLOP/s peak needs an FMA "
                 "in each of the two vector issue slots a SIMD has per 4 cycles; this op spends 2 instructions "
                 "(v_fma with the clamp modifier, v_fmac) on the 4 flop of a term (sub, clamp, mul, add), so the "
                 "peak itself is its ceiling. valu_issue_util is the share of the two-slot issue rate taken by "
-                "those 2 instructions per term; the probe table is that rate measured with a bare instruction stream.",
+                "those 2 instructions per term.",
     }
-
-
-def issue_probe():
-    """Run the stand-alone vector issue-rate probe (a child process) and return its table, or None."""
-    import subprocess
-    exe = os.path.join(ROOT, "addernetcuda_amd", "valu_issue_probe")
-    if not os.path.exists(exe):
-        return None
-    try:
-        out = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60).stdout
-    except (OSError, subprocess.SubprocessError):
-        return None
-    table = {}
-    for line in out.splitlines():
-        f = line.split()
-        if len(f) == 3 and f[0] in ("fwd_pair", "gradx_pair", "sgpr_only", "vgpr_pair"):
-            table.setdefault(f[0], {})[f"{f[1]}_waves_per_simd"] = round(float(f[2]) / 1e12, 2)
-    return table or None
 
 
 def make_step(model, opt, x, y):
