@@ -131,6 +131,42 @@ def bench_layers(dev, warmup=5, iters=20, which="resnet20"):
     return rows
 
 
+# column-matrix shapes (Co, K, NL) for the literal ADDER_* entry points: the default of the reference's
+# comparison script (adder_cuda/test_cuda.py:161-176) and the dominant ResNet-20 layer as adder.py:22-41 unfolds it
+COL_SHAPES = [(32, 288, 1024), (16, 144, 262144)]
+PEAK_HBM_GBS = 8000.0
+
+
+def bench_col(dev, warmup=3, iters=10):
+    """The four entry points of the reference extension on (K, NL) column matrices: time, GB/s against the HBM
+    peak (these kernels stream X_col, which is 9x the activation for a 3x3 layer) and TFLOP/s."""
+    from addernetcuda_amd import adder_cuda
+    rows = []
+    for Co, K, NL in COL_SHAPES:
+        g = torch.Generator(device=dev).manual_seed(1000 + Co + K)
+        X = torch.randn(K, NL, device=dev, generator=g)
+        Wm = torch.randn(Co, K, device=dev, generator=g) * math.sqrt(2.0 / K)
+        gy = torch.randn(Co, NL, device=dev, generator=g)
+        out, gW, gX = torch.empty(Co, NL, device=dev), torch.zeros(Co, K, device=dev), torch.zeros(K, NL, device=dev)
+        E = Co * K * NL
+        # algorithmic HBM bytes; gradients are accumulated into (read + written), as the reference's atomicAdd does
+        b_x, b_w, b_y = 4 * K * NL, 4 * Co * K, 4 * Co * NL
+        ops = {
+            "ADDER_CONV": (lambda: adder_cuda.ADDER_CONV(X, Wm, out), 2, b_x + b_w + b_y),
+            "ADDER_CONV_WEIGHT": (lambda: adder_cuda.ADDER_CONV_WEIGHT(gy, X, Wm, gW), 3, b_x + b_y + 3 * b_w),
+            "ADDER_CONV_INPUT": (lambda: adder_cuda.ADDER_CONV_INPUT(gy, X, Wm, gX), 4, 3 * b_x + b_y + b_w),
+            "ADDER_BACKWARD": (lambda: adder_cuda.ADDER_BACKWARD(gy, X, Wm, gW, gX), 7, 3 * b_x + b_y + 3 * b_w),
+        }
+        for name, (fn, flop, nbytes) in ops.items():
+            t = event_time(fn, warmup, iters)
+            rows.append({"shape": f"Co={Co} K={K} NL={NL}", "op": name, "us": round(t * 1e6, 2),
+                         "algorithmic_bytes": nbytes, "gbs": round(nbytes / t / 1e9, 1),
+                         "frac_hbm_peak": round(nbytes / t / 1e9 / PEAK_HBM_GBS, 4),
+                         "tflops": round(flop * E / t / 1e12, 2),
+                         "frac_fp32_peak": round(flop * E / t / 1e12 / PEAK_FP32_TFLOPS, 4)})
+    return rows
+
+
 def dominant_kernel(dev, steps):
     """grad_x of the 16->16 3x3 @32x32 layer: the kernel with the largest share of a training step."""
     cnt, Ci, H, W, Co, k, s, p = RESNET20_LAYERS[0]
@@ -289,9 +325,10 @@ def main():
     ap.add_argument("--stock-modules", action="store_true",
                     help="with --model vgg_small / resnet50 / densenet_cifar: build the network from stock "
                          "nn.BatchNorm2d / ReLU modules as the reference's model files do (only the adder layers differ)")
-    ap.add_argument("--layer-set", choices=sorted(LAYER_SETS), default="resnet20",
+    ap.add_argument("--layer-set", choices=sorted(LAYER_SETS) + ["col"], default="resnet20",
                     help="with --layers-only: the adder layers of ResNet-20 (batch 256), the VGG-small stack "
-                         "(batch 128) or ResNet-50 at 224x224 (batch 64)")
+                         "(batch 128), ResNet-50 at 224x224 (batch 64), or col: the reference extension's four "
+                         "column-matrix entry points (adder_cuda.ADDER_*) at two shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (every box here has a single MI355X)")
@@ -307,6 +344,10 @@ def main():
             dst.copy_(src)            # 256 MiB read + 256 MiB written per launch
         torch.cuda.synchronize()
         print(json.dumps({"roofline": dominant_kernel(dev, args.steps), "copy_bytes_each_way": src.numel() * 4}))
+        return
+
+    if args.layers_only and args.layer_set == "col":
+        print(json.dumps({"layer_set": "col", "layers": bench_col(dev, iters=max(3, min(args.steps, 20)))}))
         return
 
     if args.layers_only:
