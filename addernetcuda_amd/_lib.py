@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(_HERE, "libaddernet_hip.so")
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
-        f"{LIB_PATH} is missing: build it with `python -m addernetcuda_amd.build` "
+        f"{LIB_PATH} is missing: build it with `python addernetcuda_amd/build.py` "
         "(hipcc, gfx950). There is no fallback implementation.")
 
 lib = ctypes.CDLL(LIB_PATH)
@@ -30,6 +30,7 @@ _SIGNATURES = {
     "adder_conv2d_bwd_workspace_bytes": (_i, [_i] * 9 + [_szp]),
     "adder_conv2d_bwd_f32": (_i, [_p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_add_f32": (_i, [_p, _p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
+    "adder_conv2d_bwd_noalloc_f32": (_i, [_p, _p, _p, _p, _p, _f] + [_i] * 9 + [_p]),
     "adder_col_fwd_f32": (_i, [_p, _p, _p, _i, _l, _i, _p]),
     "adder_col_bwd_workspace_bytes": (_i, [_i, _l, _i, _szp]),
     "adder_col_bwd_f32": (_i, [_p, _p, _p, _p, _p, _i, _l, _i, _p, _sz, _p]),

@@ -3,6 +3,7 @@
 // exercised on a machine without a GPU.
 #include "common.hpp"
 
+#include <atomic>
 #include <cstdlib>
 #include <string>
 
@@ -21,6 +22,30 @@ int check_launch() {
 }
 
 static const long kMaxElems = 0x7fffffffL;
+
+// Scratch of the allocation-free backward (adder_conv2d_bwd_noalloc_f32): part of the device image, one copy per
+// GPU.  In host code `scratch` is only a handle for hipGetSymbolAddress -- never a device address; the address
+// each device gives its copy is looked up once per device and kept in g_scratch.
+static __device__ __align__(256) unsigned char scratch[ADDER_NOALLOC_SCRATCH_BYTES];
+static constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch[kMaxDevices];
+
+// Device address of the current device's copy of `scratch`.
+static int scratch_of_current_device(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return record_hip_error(e);
+    if (dev < 0 || dev >= kMaxDevices) return ADDER_ERR_UNSUPPORTED;
+    void *p = g_scratch[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));   // the address on the device that is current now
+        if (e != hipSuccess) return record_hip_error(e);
+        if (!p) return ADDER_ERR_HIP;
+        g_scratch[dev].store(p, std::memory_order_release);   // two threads racing here store the same address
+    }
+    *out = p;
+    return ADDER_OK;
+}
 
 static int make_dims(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, ConvDims &d) {
     if (N <= 0 || Ci <= 0 || H <= 0 || W <= 0 || Co <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || pad < 0)
@@ -176,6 +201,24 @@ static int conv2d_bwd(const float *gy, const float *x, const float *w, const flo
     if (gw)
         if (int rc = launch_grad_w(gy, x, w, gw, eta, ws, ws_bytes, d, s)) return rc;
     return ADDER_OK;
+}
+
+int adder_conv2d_bwd_noalloc_f32(const float *gy, const float *x, const float *w, float *gx, float *gw, float eta,
+                                 int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad,
+                                 void *stream) {
+    if (!gy || !x || !w) return ADDER_ERR_NULL_POINTER;
+    if (!gx && !gw) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    void *ws = nullptr;
+    size_t need = 0;
+    if (gw) {   // only the weight gradient uses scratch
+        need = grad_w_workspace_bytes(d);
+        if (need > ADDER_NOALLOC_SCRATCH_BYTES) return ADDER_ERR_WORKSPACE;   // before any HIP call
+        if (int rc = scratch_of_current_device(&ws)) return rc;
+    }
+    // every kernel writes the part of the scratch it later reads (slabs, norm partials): nothing to clear
+    return conv2d_bwd(gy, x, w, nullptr, gx, gw, eta, ws, need, N, Ci, H, W, Co, kh, kw, stride, pad, stream);
 }
 
 static int check_col(int K, long NL, int Co) {

@@ -113,6 +113,23 @@ ADDER_API int adder_conv2d_bwd_add_f32(const float *gy, const float *x, const fl
                          int N, int Ci, int H, int W, int Co, int kh, int kw,
                          int stride, int pad, void *stream);
 
+/* adder_conv2d_bwd_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc) and have no workspace to hand over.  It has no counterpart in
+ * the reference, whose backward takes every buffer from torch's allocator (adder.py:66-67).  The partial slabs
+ * and norm partials live in a buffer of ADDER_NOALLOC_SCRATCH_BYTES that is part of the library's device image
+ * (every GPU the library runs on holds one copy until the process ends); the call allocates and frees nothing.
+ * Same arguments and results as adder_conv2d_bwd_f32 without ws / ws_bytes.  Layers whose
+ * adder_conv2d_bwd_workspace_bytes exceeds ADDER_NOALLOC_SCRATCH_BYTES are refused with ADDER_ERR_WORKSPACE
+ * before anything is launched (every ResNet-20 layer at batch 256 fits).  All calls on one GPU share that
+ * GPU's buffer: calls that overlap in time on one GPU (different streams, or threads) race; serialise them.
+ * The first call on a device looks the buffer's address up (hipGetSymbolAddress); make that call outside
+ * stream capture. */
+#define ADDER_NOALLOC_SCRATCH_BYTES (8u << 20)
+ADDER_API int adder_conv2d_bwd_noalloc_f32(const float *gy, const float *x, const float *w,
+                         float *gx, float *gw, float eta,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream);
+
 /* ------------------------------------------------------------------------
  * Column-matrix path: the literal signatures of the reference extension.
  *   Xcol (K, NL)   Wcol (Co, K)   out, gy (Co, NL)   gW (Co, K)   gX (K, NL)
