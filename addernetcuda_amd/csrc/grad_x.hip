@@ -160,16 +160,14 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
             acc[m][t] = tot[m][t] = 0.f;
         }
     }
-    // per tile position, the sum of gy over all output channels (threads own plane elements)
+    // per tile position, the sum of gy over all output channels: every thread owns GITER elements of the
+    // plane and adds them up in double in registers (one conversion and one add per chunk -- the sum is taken
+    // off a sum of the same size at the end, so its rounding counts), the plane itself is written once
     constexpr int GN = C::NIMG * C::PLANE, GITER = ceil_div(GN, C::NTHREADS);
     float *gplane = smem + 2 * C::BUF;
-    if constexpr (SAT) {
+    double gsum[GITER];
 #pragma unroll
-        for (int it = 0; it < GITER; ++it) {
-            const int e = threadIdx.x + it * C::NTHREADS;
-            if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
-        }
-    }
+    for (int it = 0; it < GITER; ++it) gsum[it] = 0.0;
 
     const int lane_off = img * C::CC * C::PLANE + row * C::PITCH + strip * TN;
     const int nchunks = ceil_div(Co, C::CC);
@@ -293,10 +291,15 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
             }
 
         }
+        // a single tap makes a chunk only CC terms long: fold every fourth chunk, so that the two levels of
+        // the sum stay comparable in length (2048 output channels: 64 x 32 instead of 16 x 128)
+        constexpr int FOLD = KS == 1 ? 4 : 1;
+        if (FOLD == 1 || (c & (FOLD - 1)) == FOLD - 1 || c + 1 == nchunks) {
 #pragma unroll
-        for (int m = 0; m < TM; ++m)
+            for (int m = 0; m < TM; ++m)
 #pragma unroll
-            for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+                for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+        }
 
         // channel sum of this chunk (planes past Co were staged as zeros)
         if constexpr (SAT) {
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
                     float sum = 0.f;
 #pragma unroll
                     for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
-                    gplane[e] += sum;   // always the same thread for a given e: no race
+                    gsum[it] += (double)sum;
                 }
             }
         }
@@ -318,8 +321,13 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
     }
 
     // sum over (co, taps) of the gy values a position met = box sum of the channel-sum plane
-    // (the loop's last barrier has made every thread's part of the plane visible)
     if constexpr (SAT) {
+#pragma unroll
+        for (int it = 0; it < GITER; ++it) {
+            const int e = threadIdx.x + it * C::NTHREADS;
+            if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = (float)gsum[it];
+        }
+        __syncthreads();
         float gs[KS][TN + KS - 1];
 #pragma unroll
         for (int i = 0; i < KS; ++i)
@@ -380,8 +388,10 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 // The two-instruction form doubles a sum of products whose factors lie in [0, 1] and takes a second
 // sum off it, which about triples the rounding error of the three-instruction form (measured against
 // fp64: 0.2 of the parity tolerance |err| <= 1e-4 + 1e-5 |gx| at 144 terms per output, 0.4 at 576, 0.9
-// at 4608).  Layers with more terms per output than this keep the three-instruction form.
-static constexpr int kSatMaxTerms = 2304;
+// at 4608).  Layers with more terms per output than this keep the three-instruction form.  Single-tap
+// layers stop at 1024: their chunks are CC terms long, not 9 * CC, so the second level of the sum is long
+// and carries the full magnitude (512 -> 2048 @7x7 at batch 64 had one element in 1e5 at 1.2 of the tolerance).
+static constexpr int kSatMaxTerms = 2304, kSatMaxTerms1x1 = 1024;
 
 template <class C, bool VEC, bool SAT, bool SUB = false>
 static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w, float *gx,
@@ -405,7 +415,7 @@ static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, 
                                const ConvDims &d, hipStream_t s, const float *gadd = nullptr,
                                const Subsample sub = Subsample{1, 0, 0, 0}) {
     const bool vec = d.W % 4 == 0;
-    if (d.Co * C::KK > kSatMaxTerms)
+    if (d.Co * C::KK > (C::KS == 1 ? kSatMaxTerms1x1 : kSatMaxTerms))
         return vec ? launch_grad_x_3x3s1_v<C, true, false, SUB>(gy, x, w, gx, d, s, sub, gadd)
                    : launch_grad_x_3x3s1_v<C, false, false, SUB>(gy, x, w, gx, d, s, sub, gadd);
     return vec ? launch_grad_x_3x3s1_v<C, true, true, SUB>(gy, x, w, gx, d, s, sub, gadd)
@@ -488,13 +498,9 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     }
     constexpr int GN = C::NIMG * C::PLANE, GITER = ceil_div(GN, C::NTHREADS);
     float *gplane = smem + 2 * C::BUF;   // per tile position, the sum of gy over all output channels
-    if constexpr (SAT) {
+    double gsum[GITER];                  // ... collected in double in registers, as in the stride-1 kernel
 #pragma unroll
-        for (int it = 0; it < GITER; ++it) {
-            const int e = threadIdx.x + it * C::NTHREADS;
-            if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = 0.f;
-        }
-    }
+    for (int it = 0; it < GITER; ++it) gsum[it] = 0.0;
 
     const int lane_off = img * C::CC * C::PLANE + brow * C::PITCH + bcol * (TNW / 2);
     const int nchunks = ceil_div(Co, C::CC);
@@ -584,7 +590,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
                     float sum = 0.f;
 #pragma unroll
                     for (int cc = 0; cc < C::CC; ++cc) sum += src[cc * C::PLANE];
-                    gplane[e] += sum;   // always the same thread for a given e: no race
+                    gsum[it] += (double)sum;
                 }
             }
         }
@@ -595,6 +601,12 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 
     // clamp = 2 * sat - 1: take off the sum of the gy values each position met (same taps as above)
     if constexpr (SAT) {
+#pragma unroll
+        for (int it = 0; it < GITER; ++it) {
+            const int e = threadIdx.x + it * C::NTHREADS;
+            if (GN % C::NTHREADS == 0 || e < GN) gplane[e] = (float)gsum[it];
+        }
+        __syncthreads();
         constexpr int RP[3] = {0, 1, 1}, RG[3] = {0, 1, 0};
         float gs[2][GSTRIP], sg[2][TNW];
 #pragma unroll

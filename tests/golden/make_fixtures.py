@@ -22,6 +22,12 @@ CASES = [  # N, Ci, H, W, Co, k, stride, pad
     (2, 3, 5, 5, 4, 3, 1, 0),
     (2, 3, 6, 5, 4, 1, 2, 0),
     (1, 2, 4, 6, 3, 3, 2, 1),
+    # large enough for the tiled GPU kernels (>= 8 channels): stride 1, stride 2, and a layer with more than
+    # 2304 terms per input position (a different arithmetic form of the input gradient on the GPU)
+    (2, 8, 8, 8, 8, 3, 1, 1),
+    (2, 8, 8, 8, 16, 3, 2, 1),
+    (1, 8, 4, 4, 260, 3, 1, 1),
+    (2, 64, 4, 4, 64, 1, 1, 0),
 ]
 
 

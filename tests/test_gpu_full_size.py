@@ -1,6 +1,9 @@
-"""The benchmark's own layer shapes at batch 256: checks that do not need a CPU oracle pass over
-6e8 terms -- a slice of images against the float64 C oracle (forward and grad_X are per-image),
-an independent float64 GEMM on the GPU for grad_W, and size-independent properties."""
+"""The layer shapes of the three model configurations at their full batch sizes (ResNet-20 at 256, the
+VGG-small stack at 128, ResNet-50 at 224x224 at 64): launch grids, partial-slab counts and workspace sizes all
+depend on the batch, so the reduced-batch parity tests do not cover these code paths.  Checks that do not
+need a CPU oracle pass over 1e10 terms: a slice of images against the float64 C oracle (forward and grad_X are
+per-image), an independent float64 GEMM on the GPU for grad_W (raw and eta-scaled, element by element), and
+size-independent properties."""
 import math
 
 import pytest
@@ -11,14 +14,26 @@ from tests.util import assert_close
 
 pytestmark = pytest.mark.gpu
 
-N = 256
-# (Ci, H, W, Co, k, stride, pad): the ResNet-20 adder-layer shapes
-LAYERS = [(16, 32, 32, 16, 3, 1, 1), (32, 16, 16, 32, 3, 1, 1), (64, 8, 8, 64, 3, 1, 1), (16, 32, 32, 32, 3, 2, 1),
-          (32, 16, 16, 64, 3, 2, 1), (16, 32, 32, 32, 1, 2, 0), (32, 16, 16, 64, 1, 2, 0)]
-PICK = [0, 1, 100, 255]
+# (N, Ci, H, W, Co, k, stride, pad)
+RESNET20 = [(256,) + l for l in [                       # resnet20.py:16-20, 52-54, 66-70
+    (16, 32, 32, 16, 3, 1, 1), (32, 16, 16, 32, 3, 1, 1), (64, 8, 8, 64, 3, 1, 1), (16, 32, 32, 32, 3, 2, 1),
+    (32, 16, 16, 64, 3, 2, 1), (16, 32, 32, 32, 1, 2, 0), (32, 16, 16, 64, 1, 2, 0)]]
+VGG_SMALL = [(128,) + l for l in [                      # 3x3 layers at 128 / 256 / 512 channels, K up to 4608
+    (128, 32, 32, 128, 3, 1, 1), (128, 16, 16, 256, 3, 1, 1), (256, 16, 16, 256, 3, 1, 1),
+    (256, 8, 8, 512, 3, 1, 1), (512, 8, 8, 512, 3, 1, 1)]]
+RESNET50 = [(64,) + l for l in [                        # every distinct layer shape of resnet50.py:19-33, 84-98
+    (64, 56, 56, 256, 1, 1, 0), (64, 56, 56, 64, 1, 1, 0), (64, 56, 56, 64, 3, 1, 1),
+    (256, 56, 56, 64, 1, 1, 0), (256, 56, 56, 512, 1, 2, 0), (256, 56, 56, 128, 1, 1, 0),
+    (128, 56, 56, 128, 3, 2, 1), (128, 28, 28, 512, 1, 1, 0), (512, 28, 28, 128, 1, 1, 0),
+    (128, 28, 28, 128, 3, 1, 1), (512, 28, 28, 1024, 1, 2, 0), (512, 28, 28, 256, 1, 1, 0),
+    (256, 28, 28, 256, 3, 2, 1), (256, 14, 14, 1024, 1, 1, 0), (1024, 14, 14, 256, 1, 1, 0),
+    (256, 14, 14, 256, 3, 1, 1), (1024, 14, 14, 2048, 1, 2, 0), (1024, 14, 14, 512, 1, 1, 0),
+    (512, 14, 14, 512, 3, 2, 1), (512, 7, 7, 2048, 1, 1, 0), (2048, 7, 7, 512, 1, 1, 0),
+    (512, 7, 7, 512, 3, 1, 1)]]
+LAYERS = RESNET20 + VGG_SMALL + RESNET50
 
 
-def _data(Ci, H, W, Co, k, s, p, gpu):
+def _data(N, Ci, H, W, Co, k, s, p, gpu):
     g = torch.Generator(device=gpu).manual_seed(1000 + Ci + Co + k + s)
     x = torch.randn(N, Ci, H, W, device=gpu, generator=g)
     w = torch.randn(Co, Ci, k, k, device=gpu, generator=g) * math.sqrt(2.0 / (Ci * k * k))
@@ -30,8 +45,10 @@ def _data(Ci, H, W, Co, k, s, p, gpu):
 @pytest.mark.parametrize("layer", LAYERS, ids=str)
 def test_full_batch_layer(layer, gpu):
     from addernetcuda_amd import adder
-    from oracle import c_oracle
-    Ci, H, W, Co, k, s, p = layer
+    from oracle import c_oracle, adder_oracle
+    N, Ci, H, W, Co, k, s, p = layer
+    PICK = [0, 1, N // 2 - 1, N - 1] if Co * Ci * k * k * H * W <= 2 ** 28 else [0, N - 1]   # oracle time
+    CH = 32 if Ci * k * k * H * W <= 2 ** 21 else 4                                       # images per unfold
     x, w, gy = _data(*layer, gpu)
     xg, wg = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
     y = adder.adder2d_function(xg, wg, s, p, eta=0.0)
@@ -45,18 +62,20 @@ def test_full_batch_layer(layer, gpu):
 
     # grad_W sums over the whole batch: float64 GEMM identity on the GPU, image by image
     acc = torch.zeros(Co, Ci * k * k, dtype=torch.float64, device=gpu)
-    for a in range(0, N, 32):
-        cols = F.unfold(x[a:a + 32].double(), k, padding=p, stride=s)            # (n, K, L)
-        acc += torch.einsum("ncl,nkl->ck", gy[a:a + 32].double().flatten(2), cols)
+    for a in range(0, N, CH):
+        cols = F.unfold(x[a:a + CH].double(), k, padding=p, stride=s)            # (n, K, L)
+        acc += torch.einsum("ncl,nkl->ck", gy[a:a + CH].double().flatten(2), cols)
+        del cols
     want = acc.view_as(w) - w.double() * gy.double().sum(dim=(0, 2, 3)).view(-1, 1, 1, 1)
     assert_close(wg.grad, want, f"grad_W {layer}")
 
-    # properties: y <= 0; backward is linear in gy; eta fixes the norm of grad_W
+    # properties: y <= 0; backward is linear in gy; the scaling of adder.py:78, element by element
     assert (y <= 0).all()
     xg.grad = wg.grad = None
     y2 = adder.adder2d_function(xg, wg, s, p, eta=0.1)
     assert torch.equal(y2, y)                                                      # deterministic
     y2.backward(2.0 * gy)
+    assert_close(wg.grad, adder_oracle.eta_scale(2.0 * want, 0.1), f"eta-scaled grad_W {layer}")
     assert wg.grad.norm().item() == pytest.approx(0.1 * math.sqrt(w.numel()), rel=1e-4)
     xg2 = x.clone().requires_grad_(True)
     adder.adder2d_function(xg2, w, s, p).backward(gy)

@@ -13,7 +13,8 @@ def _pair(gpu, batch, eta=0.1, seed=0):
     from oracle import adder_oracle
     torch.manual_seed(seed)
     hip = resnet20(eta=eta).to(gpu)
-    ref = resnet20(adder2d_cls=adder_oracle.adder2d, eta=eta).to(gpu)   # pure-torch unfold formulas, run on the GPU
+    # pure-torch unfold formulas inside stock torch modules, run on the GPU
+    ref = resnet20(adder2d_cls=adder_oracle.adder2d, eta=eta, fused=False).to(gpu)
     ref.load_state_dict(hip.state_dict())
     g = torch.Generator(device=gpu).manual_seed(seed + 1)
     x = torch.randn(batch, 3, 32, 32, device=gpu, generator=g)
@@ -52,36 +53,154 @@ def test_one_step_matches_the_unfold_reference_path(gpu):
     assert statistics.median(rel.values()) <= 0.02, sorted(rel.items(), key=lambda kv: -kv[1])[:5]
 
 
-def test_loss_curves_track_the_reference_path(gpu):
-    """50 SGD steps (momentum 0.9, lr 0.1, wd 5e-4, eta 0.1) on one synthetic batch of 64.
+BATCH, STEPS = 256, 50     # BASELINE config 3: batch 256, 50 steps, SGD momentum 0.9, eta 0.1
 
-    The first two losses must agree tightly (same weights, one update).  After that fp32 training of this
-    network is chaotic: two runs of the *same* code already differ by up to ~0.2-0.35 in loss at single steps
-    because torch's BatchNorm / reduction kernels are not run-to-run reproducible and the eta-normalised
-    updates amplify a flipped ReLU gate.  So from there on the curves are compared as means over windows of
-    ten steps: within 30 % + 0.05 over the first twenty steps, within a quarter of the initial loss later
-    (both curves are then small and noisy, and a relative bound on their difference is a coin toss), and
-    both must fit the batch (loss down to a quarter of its start)."""
-    hip, ref, x, y = _pair(gpu, 64)
-    curves = []
-    for m in (hip, ref):
-        opt = torch.optim.SGD(m.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4)
-        losses = []
-        for _ in range(50):
-            opt.zero_grad(set_to_none=True)
-            loss = torch.nn.functional.cross_entropy(m(x), y)
-            loss.backward()
-            opt.step()
-            losses.append(loss.item())
-        curves.append(losses)
-    a, b = curves
-    for i in range(2):
-        assert abs(a[i] - b[i]) <= 1e-3 * max(1.0, abs(b[i])), (i, a[i], b[i])
-    for lo in range(0, 50, 10):
-        ma, mb = sum(a[lo:lo + 10]) / 10, sum(b[lo:lo + 10]) / 10
-        bound = 0.3 * max(ma, mb) + 0.05 if lo < 20 else 0.25 * b[0]
-        assert abs(ma - mb) <= bound, (lo, ma, mb)
-    assert min(a[-5:]) < 0.25 * a[0] and min(b[-5:]) < 0.25 * b[0]
+
+def _sgd(model):
+    return torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4)   # main.py:67
+
+
+def _train(model, x, y, steps=STEPS):
+    opt = _sgd(model)
+    losses = []
+    for _ in range(steps):
+        opt.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.cross_entropy(model(x), y)
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    return losses
+
+
+def _reference_net(gpu, state, dtype):
+    """The reference's model file as it stands (stock Conv2d / BatchNorm2d / ReLU modules, resnet20.py:28-39,
+    80-93) around the oracle's unfold-formula adder layer: nothing of the HIP library runs in it."""
+    from addernetcuda_amd.resnet20 import resnet20
+    from oracle import adder_oracle
+    net = resnet20(adder2d_cls=adder_oracle.adder2d, eta=0.1, fused=False).to(gpu)
+    net.load_state_dict(state)
+    return net.to(dtype)
+
+
+def test_training_is_bit_reproducible_at_batch_256(gpu):
+    """Two runs of 50 training steps from the same weights give the same 50 losses, bit for bit, and the same
+    final weights: no kernel of the step adds in an order that changes from run to run (the reference's
+    backward does, adder.cu:266-267).  The classifier runs as a matrix product for this reason (resnet20.py
+    of this package): the vendor convolution's weight gradient was the one kernel that did not reproduce."""
+    hip, _, x, y = _pair(gpu, BATCH)
+    state = copy.deepcopy(hip.state_dict())
+    first = _train(hip, x, y)
+    end = copy.deepcopy(hip.state_dict())
+    hip.load_state_dict(state)
+    second = _train(hip, x, y)
+    assert first == second
+    for k, v in hip.state_dict().items():
+        assert torch.equal(v, end[k]), k
+
+
+def test_every_step_of_a_50_step_run_matches_the_reference_step(gpu):
+    """Config 3 (batch 256, 50 steps), one step at a time along the reference trajectory.
+
+    The trajectory is the reference path's own, computed in float64.  At every step t the HIP network and the
+    reference path in fp32 are both put into the float64 run's state (weights, BatchNorm buffers, momentum),
+    take one training step, and are compared with what the float64 step gives from that state:
+      * the loss at the common state (the forward pass) -- to 1e-5 relative;
+      * the loss after the step, i.e. the float64 network's loss at the weights each fp32 step produced against
+        its loss at its own new weights (the backward pass, the eta scaling and the update in one number) -- to
+        1e-3 * max(1, |loss|) at each of the 50 steps, and
+        to three times the largest deviation the reference path's own fp32 step has shown so far (+ 1e-5).
+    Measured on MI355X: forward <= 9e-7 (fp32 reference path: 7e-6), step <= 5e-5 (fp32 reference path: 1.5e-4).
+    Compared like this, nothing accumulates: see the free-running test below for why that matters."""
+    import torch.nn.functional as F
+    from addernetcuda_amd.resnet20 import resnet20
+    torch.manual_seed(0)
+    hip = resnet20(eta=0.1).to(gpu)
+    ref32 = _reference_net(gpu, hip.state_dict(), torch.float32)
+    ref64 = _reference_net(gpu, hip.state_dict(), torch.float64)
+    probe = copy.deepcopy(ref64)
+    g = torch.Generator(device=gpu).manual_seed(1)
+    x = torch.randn(BATCH, 3, 32, 32, device=gpu, generator=g)
+    y = torch.randint(0, 10, (BATCH,), device=gpu, generator=g)
+    xd = x.double()
+    o_hip, o_32, o_64 = _sgd(hip), _sgd(ref32), _sgd(ref64)
+
+    def put_into_reference_state(model, opt):
+        model.load_state_dict(ref64.state_dict())
+        for p, q in zip(model.parameters(), ref64.parameters()):
+            buf = o_64.state.get(q, {}).get("momentum_buffer")
+            if buf is not None:
+                opt.state[p]["momentum_buffer"] = buf.to(p.dtype).clone()
+
+    def one_step(model, opt, inp):
+        opt.zero_grad(set_to_none=True)
+        loss = F.cross_entropy(model(inp), y)
+        loss.backward()
+        opt.step()
+        return loss.item()
+
+    envelope = 0.0
+    worst = {"fwd_hip": 0.0, "fwd_ref32": 0.0, "step_hip": 0.0, "step_ref32": 0.0}
+    for t in range(STEPS):
+        put_into_reference_state(hip, o_hip)
+        put_into_reference_state(ref32, o_32)
+        l_hip, l_32, l_64 = one_step(hip, o_hip, x), one_step(ref32, o_32, x), one_step(ref64, o_64, xd)
+        assert abs(l_hip - l_64) <= 1e-5 * max(1.0, abs(l_64)), (t, l_hip, l_64)
+        with torch.no_grad():
+            after_64 = F.cross_entropy(ref64(xd), y).item()
+            dev = {}
+            for name, m in (("hip", hip), ("ref32", ref32)):
+                probe.load_state_dict(m.state_dict())
+                dev[name] = abs(F.cross_entropy(probe(xd), y).item() - after_64)
+        envelope = max(envelope, dev["ref32"])
+        assert dev["hip"] <= 1e-3 * max(1.0, abs(after_64)), (t, dev)
+        assert dev["hip"] <= 3.0 * envelope + 1e-5, (t, dev, envelope)
+        for k, v in (("fwd_hip", abs(l_hip - l_64)), ("fwd_ref32", abs(l_32 - l_64)), ("step_hip", dev["hip"]),
+                     ("step_ref32", dev["ref32"])):
+            worst[k] = max(worst[k], v)
+    print("largest deviations from the float64 reference step over 50 steps:", worst)
+    assert l_64 < 0.5 * 2.7276   # the trajectory does fit the batch (loss 2.73 -> 0.83)
+
+
+def test_free_running_loss_curves_track_the_float64_reference(gpu):
+    """Config 3 free-running: 50 steps of the HIP network and of the reference path in fp32, each on its own
+    trajectory, against the reference path in float64, all from the same weights on the same batch.
+
+    fp32 training of this network does not keep two implementations together: the eta-normalised updates at
+    lr 0.1 amplify a last-bit difference by one to two orders of magnitude per step in the first steps
+    (measured, MI355X: the reference path's fp32 run is 1e-6 from its float64 run at step 0, 1.4e-5 at step 1,
+    6e-4 at step 2, 1.3e-3 at step 3, 2e-2 at step 7, 5e-2 at step 10, and two runs of that same fp32 code are
+    5e-3 apart at step 6 because torch's fold / reduction kernels add in varying order).  The per-step gate
+    proposed for this curve -- 1e-3 for ten steps -- is therefore missed by the reference against itself from
+    step 3 on, and which implementation is closer at a given later step is a coin toss.  What is asserted:
+      * steps 0-2 within 1e-3 * max(1, |loss|) of the float64 curve (measured 5e-4 at step 2; a wrong eta, a
+        dropped padding tap or a wrong sign in one layer shows as > 1e-2 there);
+      * over all 50 steps, the HIP curve tracks the float64 curve as closely as the reference's own fp32 run
+        does: mean log10 deviation no more than log10(3) above that of the fp32 reference, over the first ten
+        steps and over all fifty (a mean over steps is what makes this a measurement instead of a coin toss);
+      * all three fit the batch.
+    The per-step comparison that does hold 1e-3 at each of the 50 steps is the test above."""
+    import math
+    from addernetcuda_amd.resnet20 import resnet20
+    torch.manual_seed(0)
+    hip = resnet20(eta=0.1).to(gpu)
+    state = copy.deepcopy(hip.state_dict())
+    g = torch.Generator(device=gpu).manual_seed(1)
+    x = torch.randn(BATCH, 3, 32, 32, device=gpu, generator=g)
+    y = torch.randint(0, 10, (BATCH,), device=gpu, generator=g)
+    c_hip = _train(hip, x, y)
+    c_32 = _train(_reference_net(gpu, state, torch.float32), x, y)
+    c_64 = _train(_reference_net(gpu, state, torch.float64), x.double(), y)
+    d_hip = [abs(a - b) for a, b in zip(c_hip, c_64)]
+    d_32 = [abs(a - b) for a, b in zip(c_32, c_64)]
+    for t in range(3):
+        assert d_hip[t] <= 1e-3 * max(1.0, abs(c_64[t])), (t, c_hip[t], c_64[t])
+    mean_log = lambda d: sum(math.log10(v + 1e-7) for v in d) / len(d)
+    print("mean log10 deviation from the float64 curve: hip %.2f, fp32 reference %.2f; largest: %.3f, %.3f"
+          % (mean_log(d_hip), mean_log(d_32), max(d_hip), max(d_32)))
+    assert mean_log(d_hip[:10]) <= mean_log(d_32[:10]) + math.log10(3.0)
+    assert mean_log(d_hip) <= mean_log(d_32) + math.log10(3.0)
+    for c in (c_hip, c_32, c_64):
+        assert min(c[-5:]) < 0.5 * c[0]
 
 
 def test_captured_graph_replays_match_the_eager_step(gpu):
