@@ -244,6 +244,14 @@ int adder_col_bwd_workspace_bytes(int K, long NL, int Co, size_t *bytes) {
     return ADDER_OK;
 }
 
+// the slab workspace of the column-matrix weight gradient (none for matrices the slab kernel does not serve)
+static int check_col_ws(const void *ws, size_t ws_bytes, int K, long NL, int Co) {
+    const size_t need = col_grad_w_workspace_bytes(K, NL, Co);
+    if (need == 0) return ADDER_OK;
+    if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
+    return ADDER_OK;
+}
+
 static int col_alias(const float *gy, const float *X, const float *Wm, const float *gW, const float *gX, int K,
                      long NL, int Co) {
     const size_t nx = sizeof(float) * (size_t)K * NL, nw = sizeof(float) * (size_t)Co * K,
@@ -260,7 +268,7 @@ int adder_col_gradw_f32(const float *gy, const float *Xcol, const float *Wcol, f
     if (!gy || !Xcol || !Wcol || !gW) return ADDER_ERR_NULL_POINTER;
     if (int rc = check_col(K, NL, Co)) return rc;
     if (int rc = col_alias(gy, Xcol, Wcol, gW, nullptr, K, NL, Co)) return rc;
-    if (ws_bytes < col_grad_w_workspace_bytes(K, NL, Co)) return ADDER_ERR_WORKSPACE;
+    if (int rc = check_col_ws(ws, ws_bytes, K, NL, Co)) return rc;
     return launch_col_grad_w(gy, Xcol, Wcol, gW, K, NL, Co, ws, static_cast<hipStream_t>(stream));
 }
 
@@ -277,7 +285,7 @@ int adder_col_bwd_f32(const float *gy, const float *Xcol, const float *Wcol, flo
     if (!gy || !Xcol || !Wcol || !gW || !gX) return ADDER_ERR_NULL_POINTER;
     if (int rc = check_col(K, NL, Co)) return rc;
     if (int rc = col_alias(gy, Xcol, Wcol, gW, gX, K, NL, Co)) return rc;
-    if (ws_bytes < col_grad_w_workspace_bytes(K, NL, Co)) return ADDER_ERR_WORKSPACE;
+    if (int rc = check_col_ws(ws, ws_bytes, K, NL, Co)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (int rc = launch_col_grad_x(gy, Xcol, Wcol, gX, K, NL, Co, s)) return rc;
     return launch_col_grad_w(gy, Xcol, Wcol, gW, K, NL, Co, ws, s);

@@ -172,6 +172,8 @@ size_t norm_scale_batched_workspace_bytes(int count);
 int launch_norm_scale_batched(int count, float *const *g, const long *n, const float *eta, float eps, void *ws,
                               hipStream_t s);
 
+int launch_grad_w_slab_finalize(const double *part, const double *sgpart, const float *w, float *gw, int slots, int Co,
+                                int K, bool accumulate, hipStream_t s);
 int launch_col_fwd(const float *X, const float *W, float *out, int K, long NL, int Co, hipStream_t s);
 size_t col_grad_w_workspace_bytes(int K, long NL, int Co);
 int launch_col_grad_w(const float *gy, const float *X, const float *W, float *gW, int K, long NL,

@@ -89,7 +89,8 @@ __global__ __launch_bounds__(256) void grad_w_generic_kernel(const float *__rest
 // chain is slots/kFinLanes long.
 // ---------------------------------------------------------------------------
 static constexpr int kFinOut = 16, kFinLanes = 16;   // a wave reads four full 64-byte runs per slot row
-template <typename PT>
+// ACC: the result is added to gw (the column-matrix entry points accumulate, as the reference's atomicAdd does).
+template <typename PT, bool ACC = false>
 __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ part, const PT *__restrict__ sgpart,
                                                       const float *__restrict__ w, float *__restrict__ gw,
                                                       double *__restrict__ ss, int slots, int Co, int K, int block) {
@@ -126,7 +127,8 @@ __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ par
         for (int k = 0; k < kFinLanes; ++k) { ta += ra[k][o]; ts += rs[k][o]; }
         double v = 0.0;
         if (idx < total) {
-            const float r = (float)(w ? ta - (double)w[idx] * ts : ta);   // no weights: the plain sum of x * gy
+            float r = (float)(w ? ta - (double)w[idx] * ts : ta);   // no weights: the plain sum of x * gy
+            if constexpr (ACC) r += gw[idx];
             gw[idx] = r;
             v = (double)r * (double)r;
         }
@@ -136,14 +138,27 @@ __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ par
     }
 }
 
-template <typename PT>
+template <typename PT, bool ACC = false>
 __global__ __launch_bounds__(kFinOut * kFinLanes) void grad_w_finalize_kernel(const PT *__restrict__ part,
                                                                               const PT *__restrict__ sgpart,
                                                                               const float *__restrict__ w,
                                                                               float *__restrict__ gw,
                                                                               double *__restrict__ ss, int slots,
                                                                               int Co, int K) {
-    grad_w_finalize_block<PT>(part, sgpart, w, gw, ss, slots, Co, K, blockIdx.x);
+    grad_w_finalize_block<PT, ACC>(part, sgpart, w, gw, ss, slots, Co, K, blockIdx.x);
+}
+
+// gw (+)= sum of `slots` fp64 slabs - w * sum of the gy partials: the finalize on its own, for the column-matrix path
+int launch_grad_w_slab_finalize(const double *part, const double *sgpart, const float *w, float *gw, int slots, int Co,
+                                int K, bool accumulate, hipStream_t s) {
+    const int nb = (int)ceil_div_l((long)Co * K, kFinOut);
+    if (accumulate)
+        hipLaunchKernelGGL((grad_w_finalize_kernel<double, true>), dim3(nb), dim3(kFinOut * kFinLanes), 0, s, part, sgpart,
+                           w, gw, nullptr, slots, Co, K);
+    else
+        hipLaunchKernelGGL((grad_w_finalize_kernel<double, false>), dim3(nb), dim3(kFinOut * kFinLanes), 0, s, part, sgpart,
+                           w, gw, nullptr, slots, Co, K);
+    return check_launch();
 }
 
 // The finalize of up to kGwFinishMax layers in one launch and their scaling in a second: for callers that

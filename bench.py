@@ -98,6 +98,9 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
     ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=dev)
     st = stream_ptr(dev)
     E = Co * Ci * k * k * N * Ho * Wo
+    nx, ny, nw = 4 * x.numel(), 4 * y.numel(), 4 * w.numel()
+    # algorithmic HBM bytes of each call: every tensor it reads or writes crosses HBM once
+    nbytes = {"fwd": nx + nw + ny, "grad_x": 2 * nx + ny + nw, "grad_w": nx + ny + 2 * nw}
     keep = (x, w, y, gy, gx, gw, ws)
     ops = {
         "fwd": lambda: check(lib.adder_conv2d_fwd_f32(ptr(x), ptr(w), ptr(y), *dims, st), "fwd"),
@@ -106,14 +109,14 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
         "grad_w": lambda: check(lib.adder_conv2d_bwd_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gw), ETA, ptr(ws),
                                                          need.value, *dims, st), "grad_w"),
     }
-    return E, ops, keep
+    return E, ops, keep, nbytes
 
 
 def bench_layers(dev, warmup=5, iters=20, which="resnet20"):
     rows = []
     batch, layers = LAYER_SETS[which]
     for cnt, Ci, H, W, Co, k, s, p in layers:
-        E, ops, keep = layer_ops(batch, Ci, H, W, Co, k, s, p, dev)
+        E, ops, keep, nbytes = layer_ops(batch, Ci, H, W, Co, k, s, p, dev)
         for name, fn in ops.items():
             t = event_time(fn, warmup, iters)
             flop, slots = OPS[name]
@@ -121,6 +124,8 @@ def bench_layers(dev, warmup=5, iters=20, which="resnet20"):
                 "layer": f"{Ci}->{Co} k{k} s{s} p{p} @{H}x{W}", "count": cnt, "op": name, "us": round(t * 1e6, 2),
                 "tflops": round(flop * E / t / 1e12, 2),
                 "frac_fp32_peak": round(flop * E / t / 1e12 / PEAK_FP32_TFLOPS, 4),
+                "hbm_gbs": round(nbytes[name] / t / 1e9, 1),
+                "frac_hbm_peak": round(nbytes[name] / t / 1e9 / PEAK_HBM_GBS, 4),
             }
             if name == "grad_w" and k == 3:   # fp64 matrix-core kernel (+ finalize and scaling launches)
                 row["frac_fp64_mfma_peak"] = round(2 * E / t / 1e12 / PEAK_FP64_MFMA_TFLOPS, 4)
@@ -170,7 +175,7 @@ def bench_col(dev, warmup=3, iters=10):
 def dominant_kernel(dev, steps):
     """grad_x of the 16->16 3x3 @32x32 layer: the kernel with the largest share of a training step."""
     cnt, Ci, H, W, Co, k, s, p = RESNET20_LAYERS[0]
-    E, ops, keep = layer_ops(BATCH, Ci, H, W, Co, k, s, p, dev)
+    E, ops, keep, _ = layer_ops(BATCH, Ci, H, W, Co, k, s, p, dev)
     t = event_time(ops["grad_x"], 5, max(20, steps))
     flop = OPS["grad_x"][0] * E
     achieved = flop / t / 1e12
@@ -214,7 +219,7 @@ def build_training(dev, seed=0, which="resnet20", fused=True):
     batch, size, classes = MODELS[which]
     if which == "resnet20":
         from addernetcuda_amd.resnet20 import resnet20
-        model = resnet20(eta=ETA)
+        model = resnet20(eta=ETA, fused=fused)
     else:
         from addernetcuda_amd import models
         model = getattr(models, which)(num_classes=classes, eta=ETA, fused=fused)
@@ -277,6 +282,62 @@ def graph_matches_eager(dev, replays=4, which="resnet20", fused=True):
     return ok, worst, losses
 
 
+def layer_set_summary(rows):
+    """Adder-kernel time per training step of a layer set and the flop-weighted fraction of the fp32 vector peak
+    over all of its adder kernels (forward 2, grad_X 4, grad_W 3 flop per term)."""
+    t = sum(r["us"] * r["count"] for r in rows) * 1e-6
+    flop = sum(r["tflops"] * 1e12 * r["us"] * 1e-6 * r["count"] for r in rows)
+    return {"adder_kernel_ms_per_step": round(t * 1e3, 3), "adder_kernels_tflops": round(flop / t / 1e12, 2),
+            "adder_kernels_frac_fp32_peak": round(flop / t / 1e12 / PEAK_FP32_TFLOPS, 4)}
+
+
+def time_training(dev, which, fused, steps, warmup, use_graph=True, replays=2):
+    """ms per training step of one model configuration: captured as one HIP graph when its replays reproduce
+    the eager step from the same state, eagerly otherwise."""
+    mode, graph_check = "eager", None
+    if use_graph:
+        ok, worst, losses = graph_matches_eager(dev, replays=replays, which=which, fused=fused)
+        graph_check = {"ok": ok, "max_param_diff_vs_eager_step": worst,
+                       "loss_graph_vs_eager": [[round(a, 6), round(b, 6)] for a, b in losses]}
+        if ok:
+            mode = "hipgraph"
+    model, opt, x, y = build_training(dev, which=which, fused=fused)
+    if mode == "hipgraph":
+        graph, loss = capture_step(model, opt, x, y)
+        run = graph.replay
+    else:
+        run = make_step(model, opt, x, y)
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    del run, model, opt
+    if mode == "hipgraph":
+        del graph, loss
+    torch.cuda.empty_cache()
+    return ms, mode, graph_check
+
+
+def other_configs(dev):
+    """The two other model configurations and the stock-module ResNet-20, one compact record each."""
+    out = []
+    for which, fused, label in (("resnet20", False, "ResNet-20 bs256, the reference's model file with stock nn.Conv2d / "
+                                                    "BatchNorm2d / ReLU modules (only the adder layers differ)"),
+                                ("vgg_small", True, "VGG-small AdderNet bs128, 3x32x32 (K up to 4608)"),
+                                ("resnet50", True, "ResNet-50 AdderNet bs64, 3x224x224, 1000 classes")):
+        ms, mode, check = time_training(dev, which, fused, steps=10, warmup=3)
+        rec = {"config": label, "ms_per_step": round(ms, 3), "images_per_s": round(MODELS[which][0] / ms * 1e3, 1),
+               "step_mode": mode, "graph_check_ok": None if check is None else check["ok"]}
+        if which in LAYER_SETS and fused:
+            rec.update(layer_set_summary(bench_layers(dev, warmup=2, iters=5, which=which)))
+        out.append(rec)
+    return out
+
+
 def cpu_baseline(repeats=15):   # ~10 s of host work
     """The CPU oracle's ResNet-20 training step at batch 8 (seeded), median of `repeats`, scaled to batch 256."""
     from addernetcuda_amd.resnet20 import resnet20
@@ -312,6 +373,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time the eager step instead of the captured HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
+    ap.add_argument("--no-other", action="store_true",
+                    help="skip the other model configurations (VGG-small bs128, ResNet-50 bs64, stock-module ResNet-20)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="launch only the dominant kernel (and one 256 MiB device copy as a counter yardstick); "
                          "meant to run under rocprofv3 --pmc / --kernel-trace")
@@ -353,36 +416,14 @@ def main():
     if args.layers_only:
         rows = bench_layers(dev, warmup=2, iters=max(3, min(args.steps, 20)), which=args.layer_set)
         print(json.dumps({"layer_set": args.layer_set, "batch": LAYER_SETS[args.layer_set][0], "layers": rows,
-                          "adder_kernel_ms_per_step": round(sum(r["us"] * r["count"] for r in rows) / 1e3, 3)}))
+                          **layer_set_summary(rows)}))
         return
 
-    mode = "eager"
-    graph_check = None
     fused = not args.stock_modules
-    model, opt, x, y = build_training(dev, which=args.model, fused=fused)
-    if not args.no_graph:
-        ok, worst, losses = graph_matches_eager(dev, replays=4 if args.model == "resnet20" else 2, which=args.model,
-                                                fused=fused)
-        graph_check = {"ok": ok, "max_param_diff_vs_eager_step": worst,
-                       "loss_graph_vs_eager": [[round(a, 6), round(b, 6)] for a, b in losses]}
-        if ok:
-            mode = "hipgraph"
-    if mode == "hipgraph":
-        graph, loss = capture_step(model, opt, x, y)
-        run = graph.replay
-    else:
-        run = make_step(model, opt, x, y)
+    ms, mode, graph_check = time_training(dev, args.model, fused, args.steps, args.warmup, use_graph=not args.no_graph,
+                                          replays=4 if args.model == "resnet20" else 2)
 
-    for _ in range(args.warmup):
-        run()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    if args.model != "resnet20":
+    if args.model != "resnet20" or not fused:
         batch, size, classes = MODELS[args.model]
         print(json.dumps({
             "metric": f"{args.model} AdderNet train ms/batch (bs{batch})", "value": round(ms, 3), "unit": "ms/batch",
@@ -400,7 +441,11 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ResNet-20 AdderNet, batch 256, 3x32x32, 10 classes, SGD momentum 0.9 lr 0.1 wd 5e-4, "
-                               "adaptive eta 0.1, fwd+bwd+optimizer", "step_mode": mode},
+                               "adaptive eta 0.1, fwd+bwd+optimizer; BatchNorm / ReLU / residual add run as this "
+                               "library's fused kernels (BatchNormAct2d) and the regular 3->16 stem convolution "
+                               "through the tiled forward / slab weight-gradient kernels (StemConv2d); the same step "
+                               "with stock torch modules is other_configs[0]",
+                   "step_mode": mode},
         "images_per_s": round(BATCH / ms * 1e3, 1),
         "roofline": dominant_kernel(dev, args.steps),
     }
@@ -409,7 +454,10 @@ def main():
     if not args.no_layers:
         rows = bench_layers(dev)
         out["layers"] = rows
-        out["adder_kernel_ms_per_step"] = round(sum(r["us"] * r["count"] for r in rows) / 1e3, 3)
+        out.update(layer_set_summary(rows))
+        out["col_path"] = bench_col(dev)
+    if not args.no_other:
+        out["other_configs"] = other_configs(dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

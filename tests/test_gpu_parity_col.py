@@ -8,7 +8,11 @@ pytestmark = pytest.mark.gpu
 
 # (Co, K, NL): test_cuda.py:165-171 default (N=16, Co=32, Ci=32, k=3, HWo=8), then ragged sizes the
 # reference aborts on (adder.cu:286-297: Co and NL must both be multiples of 16 or of 12)
-CASES = [(32, 288, 1024), (16, 144, 512), (12, 36, 240), (7, 27, 101), (1, 1, 1), (33, 5, 300), (5, 130, 64)]
+CASES = [(32, 288, 1024), (16, 144, 512), (12, 36, 240), (7, 27, 101), (1, 1, 1), (33, 5, 300), (5, 130, 64),
+         # many columns (two columns per lane, slabs from every workgroup) with a ragged last group; 17..32 and more
+         # than 32 output channels (other kernels); tile tails on both sides of the weight-gradient product
+         (16, 144, 65544), (9, 20, 70004), (24, 50, 66000), (48, 40, 2052), (64, 576, 1000), (20, 200, 4100),
+         (40, 150, 66562)]
 
 
 def _data(Co, K, NL, seed=0, scale=1.0):
