@@ -6,7 +6,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libaddernet_hip.so")
+# ADDERNET_HIP_LIB: another build of the same library (a debug build, a tuning variant) instead of the in-tree one
+LIB_PATH = os.environ.get("ADDERNET_HIP_LIB") or os.path.join(_HERE, "libaddernet_hip.so")
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(

@@ -65,7 +65,8 @@ class batched_eta_scaling:
 
     It only takes over layers whose weight is a leaf with ``grad is None`` when their backward runs (the usual
     ``zero_grad(set_to_none=True)`` loop); all others are finished on the spot as always.  One backward pass
-    per block.  Not for code that looks at weight gradients from hooks during the backward pass, nor for
+    per block.  If the block is left by an exception, the gradients of the layers it had taken over are set to
+    None (they were never finished).  Not for code that looks at weight gradients from hooks during the backward pass, nor for
     ``torch.autograd.grad``."""
 
     def __enter__(self):
@@ -78,12 +79,22 @@ class batched_eta_scaling:
     def __exit__(self, exc_type, exc, tb):
         global _eta_batch
         pending, _eta_batch = _eta_batch, None
+
+        def drop_pending_gradients():
+            # a staged weight's .grad is allocated memory whose slabs were never summed (or a raw, unscaled
+            # gradient): it must not survive an exceptional exit, or a caller that catches the error and steps the
+            # optimizer anyway would apply it
+            for W, _, _, _ in pending:
+                W.grad = None
+
         if exc_type is not None:
+            drop_pending_gradients()
             return False
         by_device, staged = {}, {}
         for W, eta, stage, ws in pending:
             g = W.grad
             if g is None or g.dtype != torch.float32 or not g.is_contiguous():
+                drop_pending_gradients()
                 raise RuntimeError("batched_eta_scaling: a weight's .grad is missing or not a contiguous float32 "
                                    "tensor at the end of the block")
             if stage is None:

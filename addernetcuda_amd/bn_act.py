@@ -101,4 +101,12 @@ class BatchNormAct2d(nn.BatchNorm2d):
         rm = self.running_mean if self.track_running_stats else None
         rv = self.running_var if self.track_running_stats else None
         nb = self.num_batches_tracked if self.track_running_stats else None   # advanced inside the kernel
-        return _bn_act.apply(x, self.weight, self.bias, residual, rm, rv, nb, self.momentum, self.eps, self.relu, stats)
+        weight, bias = self.weight.contiguous(), self.bias.contiguous()
+        if residual is not None and (residual.shape != x.shape or residual.dtype != torch.float32
+                                     or residual.device != x.device):
+            # the kernels read the residual as a dense fp32 tensor shaped like x; anything else (a broadcast
+            # shape, another dtype) is added the way the reference adds it (resnet20.py:37): BatchNorm alone
+            # from the kernels, then torch's add and ReLU
+            out = _bn_act.apply(x, weight, bias, None, rm, rv, nb, self.momentum, self.eps, False, stats) + residual
+            return F.relu(out) if self.relu else out
+        return _bn_act.apply(x, weight, bias, residual, rm, rv, nb, self.momentum, self.eps, self.relu, stats)

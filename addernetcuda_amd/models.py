@@ -6,6 +6,10 @@ of [3, 4, 6, 3] bottleneck blocks whose 1x1 / 3x3 / 1x1 convolutions are adder2d
 adder2d 1x1 + BatchNorm downsample on the first block of every stage (resnet50.py:84-90), global average
 pooling, a regular 1x1 convolution classifier followed by BatchNorm (resnet50.py:72-74, 110-114).
 
+``vgg11`` ... ``vgg19_bn`` (and the ``_nd`` / ``_nd_s`` / ``_nd_ss`` / ``vgg19_small_add`` variants) are the VGG family
+of vgg.py:21-170 with its state_dict keys: all-adder features including the 3-channel first layer, five poolings,
+the Linear(512) classifier stacks.  ``DenseNet121`` / ``169`` / ``201`` / ``161`` are densenet.py:93-106.
+
 ``vgg_small`` is the CIFAR VGG-small stack, 128-128-M-256-256-M-512-512-M on 32x32 inputs (4x4 maps at the end)
 with conv - BatchNorm - ReLU units as built by vgg.py:66-80; the layers are adder2d 3x3 pad 1 (vgg.py:16-18)
 except, by default, the first one on the 3-channel image (``first_adder=True`` makes that one an adder layer
@@ -173,7 +177,99 @@ class VGGSmall(nn.Module):
 
 
 def vgg_small(**kwargs):
+    """The BASELINE configuration "VGG-small-style AdderNet" (128-128-M-256-256-M-512-512-M, batch 128).  It is a
+    harness for those layer shapes, not one of vgg.py's networks: its keys and its 8192-wide classifier match no
+    reference VGG checkpoint -- for those use the ``vgg11`` ... ``vgg19_bn`` factories below."""
     return VGGSmall(**kwargs)
+
+
+# ---- the VGG family of vgg.py ---------------------------------------------------------------------------
+VGG_CFG = {   # vgg.py:75-81: channels per adder layer, "M" = 2x2 max pooling
+    "A": (64, "M", 128, "M", 256, 256, "M", 512, 512, "M", 512, 512, "M"),
+    "B": (64, 64, "M", 128, 128, "M", 256, 256, "M", 512, 512, "M", 512, 512, "M"),
+    "D": (64, 64, "M", 128, 128, "M", 256, 256, 256, "M", 512, 512, 512, "M", 512, 512, 512, "M"),
+    "E": (64, 64, "M", 128, 128, "M", 256, 256, 256, 256, "M", 512, 512, 512, 512, "M", 512, 512, 512, 512, "M"),
+}
+
+
+class VGG(nn.Module):
+    """vgg.py:21-57 with the same module indices, hence the same state_dict keys (``features.<i>.adder``,
+    ``features.<i+1>.weight`` ..., ``classifier.<j>.weight``): every convolution is an adder layer, the one on the
+    3-channel image included (vgg.py:60-66); five poolings take a 32x32 input to 1x1 x 512; the classifier is
+    [Dropout] - [Linear 512 - ReLU - [Dropout]] - [Linear 512 - ReLU] - Linear(512, classes) depending on
+    ``dropout`` / ``small`` / ``supersmall`` (vgg.py:28-39).  ``fused``: the BatchNorm modules are
+    ``BatchNormAct2d`` and run the ReLU that follows them (which stays in ``features`` as a placeholder)."""
+
+    def __init__(self, cfg, num_classes=10, dropout=True, small=False, supersmall=False, batch_norm=True,
+                 adder2d_cls=None, fused=True, **adder_kw):
+        super().__init__()
+        make = adder2d_cls or _adder.adder2d
+        self.fused = fused and batch_norm
+        layers, channels = [], 3
+        for v in VGG_CFG[cfg] if isinstance(cfg, str) else cfg:
+            if v == "M":
+                layers.append(nn.MaxPool2d(kernel_size=2, stride=2))
+                continue
+            layers.append(make(channels, v, kernel_size=3, stride=1, padding=1, bias=False, **adder_kw))
+            if batch_norm:
+                layers.append(_bn(v, True, self.fused))
+            layers.append(nn.ReLU(inplace=False))
+            channels = v
+        self.features = nn.Sequential(*layers)
+        head = []
+        if dropout or supersmall:
+            head.append(nn.Dropout())
+        if not (small or supersmall):
+            head += [nn.Linear(512, 512), nn.ReLU()]
+            if dropout:
+                head.append(nn.Dropout())
+        if not supersmall:
+            head += [nn.Linear(512, 512), nn.ReLU()]
+        head.append(nn.Linear(512, num_classes))
+        self.classifier = nn.Sequential(*head)
+
+    def forward(self, x):
+        if not self.fused:
+            x = self.features(x)
+        else:
+            mods = list(self.features)
+            i = 0
+            while i < len(mods):
+                if isinstance(mods[i], nn.MaxPool2d):
+                    x, i = mods[i](x), i + 1
+                else:
+                    x, i = _conv_bn(mods[i], mods[i + 1], x), i + 3   # adder layer, BatchNorm + ReLU, (ReLU placeholder)
+        return self.classifier(x.view(x.size(0), -1))
+
+
+def _vgg_factory(cfg, doc, **fixed):
+    def build(**kwargs):
+        return VGG(cfg, **{**fixed, **kwargs})
+    build.__doc__ = doc
+    return build
+
+
+# vgg.py:84-170 (every variant there builds its features with batch normalisation: make_layers' default)
+vgg11 = _vgg_factory("A", "vgg.py:84-86")
+vgg11_nd = _vgg_factory("A", "vgg.py:88-90", dropout=False)
+vgg11_nd_s = _vgg_factory("A", "vgg.py:92-94", dropout=False, small=True)
+vgg11_nd_ss = _vgg_factory("A", "vgg.py:96-98", dropout=False, small=True, supersmall=True)
+vgg11_bn = _vgg_factory("A", "vgg.py:100-102")
+vgg13 = _vgg_factory("B", "vgg.py:105-107")
+vgg13_nd = _vgg_factory("B", "vgg.py:109-111", dropout=False)
+vgg13_nd_s = _vgg_factory("B", "vgg.py:113-115", dropout=False, small=True)
+vgg13_nd_ss = _vgg_factory("B", "vgg.py:117-119", dropout=False, small=True, supersmall=True)
+vgg13_bn = _vgg_factory("B", "vgg.py:122-124")
+vgg16 = _vgg_factory("D", "vgg.py:127-129")
+vgg16_nd = _vgg_factory("D", "vgg.py:131-133", dropout=False)
+vgg16_nd_s = _vgg_factory("D", "vgg.py:135-137", dropout=False, small=True)
+vgg16_nd_ss = _vgg_factory("D", "vgg.py:139-141", dropout=False, small=True, supersmall=True)
+vgg16_bn = _vgg_factory("D", "vgg.py:144-146")
+vgg19 = _vgg_factory("E", "vgg.py:149-151")
+vgg19_nd = _vgg_factory("E", "vgg.py:153-155", dropout=False)
+vgg19_small_add = _vgg_factory("E", "vgg.py:157-159", dropout=False, small=True)
+vgg19_nd_ss = _vgg_factory("E", "vgg.py:161-163", dropout=False, small=True, supersmall=True)
+vgg19_bn = _vgg_factory("E", "vgg.py:168-170")
 
 
 class _PreAct:
@@ -249,3 +345,23 @@ class DenseNet(nn.Module):
 def densenet_cifar(**kwargs):
     """densenet.py:108-109."""
     return DenseNet((6, 12, 24, 16), growth_rate=12, **kwargs)
+
+
+def DenseNet121(**kwargs):
+    """densenet.py:93-94."""
+    return DenseNet((6, 12, 24, 16), growth_rate=32, **kwargs)
+
+
+def DenseNet169(**kwargs):
+    """densenet.py:97-98."""
+    return DenseNet((6, 12, 32, 32), growth_rate=32, **kwargs)
+
+
+def DenseNet201(**kwargs):
+    """densenet.py:101-102."""
+    return DenseNet((6, 12, 48, 32), growth_rate=32, **kwargs)
+
+
+def DenseNet161(**kwargs):
+    """densenet.py:105-106."""
+    return DenseNet((6, 12, 36, 24), growth_rate=48, **kwargs)

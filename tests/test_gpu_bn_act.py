@@ -178,3 +178,20 @@ def test_batchnorm_from_precomputed_statistics_equals_its_own_pass(with_res, gpu
         # back-propagated through them to ~1e-5 of the largest entry
         assert torch.allclose(got, want, rtol=1e-4, atol=1e-4 * max(1.0, want.abs().max().item())), name
     assert int(a.num_batches_tracked) == 1
+
+
+def test_a_residual_that_is_not_shaped_like_x_is_added_the_way_torch_adds_it(gpu):
+    """The kernels read the residual as a dense fp32 tensor shaped like x; a broadcast shape or another dtype
+    goes through torch's add instead of being misread."""
+    from addernetcuda_amd.bn_act import BatchNormAct2d
+    torch.manual_seed(5)
+    x = torch.randn(4, 6, 8, 8, device=gpu)
+    for res in (torch.randn(1, 6, 1, 1, device=gpu), torch.randn(4, 6, 8, 8, device=gpu).double()):
+        for relu in (True, False):
+            bn = BatchNormAct2d(6, relu=relu).to(gpu)
+            ref = torch.nn.BatchNorm2d(6).to(gpu).double()
+            want = ref(x.double()) + res.double()
+            want = torch.relu(want) if relu else want
+            got = bn(x, residual=res)
+            assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-5)
+            assert torch.allclose(bn.running_var.double(), ref.running_var, rtol=1e-5, atol=1e-6)

@@ -134,3 +134,24 @@ def test_npz_loader_accepts_both_image_layouts(tmp_path):
     d = load_arrays(str(p), torch.device("cpu"))
     assert d["train"][0].shape == (6, 3, 32, 32) and torch.equal(d["train"][0], d["test"][0])
     assert d["train"][1].dtype == torch.int64
+
+
+def test_batched_eta_scaling_drops_unfinished_gradients_on_an_exceptional_exit():
+    """A weight the block had taken over holds an allocated but unfinished .grad; leaving the block through an
+    exception (or failing in its exit) must not leave that memory where an optimizer could apply it."""
+    import pytest
+    from addernetcuda_amd import adder
+    w1 = torch.nn.Parameter(torch.zeros(4, 3, 3, 3))
+    w2 = torch.nn.Parameter(torch.zeros(2, 2))
+    with pytest.raises(KeyboardInterrupt):
+        with adder.batched_eta_scaling():
+            w1.grad = torch.full_like(w1, 123.0)              # stands for the unsummed slabs' target
+            adder._eta_batch.append((w1, 0.2, None, None))
+            raise KeyboardInterrupt
+    assert w1.grad is None and adder._eta_batch is None
+    with pytest.raises(RuntimeError, match="missing"):
+        with adder.batched_eta_scaling():
+            w1.grad = torch.full_like(w1, 123.0)
+            adder._eta_batch.append((w1, 0.2, None, None))
+            adder._eta_batch.append((w2, 0.2, None, None))    # its .grad never arrived
+    assert w1.grad is None and w2.grad is None and adder._eta_batch is None

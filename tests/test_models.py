@@ -45,6 +45,51 @@ def test_vgg_small_layout_and_cpu_forward():
     assert net(x).shape == (2, 10) and plain(x).shape == (2, 10)
 
 
+def test_vgg_family_has_the_reference_module_indices_and_classifiers():
+    """vgg.py:21-170: all-adder features (the 3-channel first layer included), conv / BatchNorm / ReLU triples with
+    a pooling after each stage, and the three classifier stacks; keys written out by hand from the source."""
+    from addernetcuda_amd import models
+    torch.manual_seed(0)
+    net = models.vgg11(adder2d_cls=_oracle_layer())
+    keys = list(net.state_dict())
+    conv_at = [0, 4, 8, 11, 15, 18, 22, 25]                      # cfg A: 64 M 128 M 256 256 M 512 512 M 512 512 M
+    assert [k for k in keys if k.endswith(".adder")] == [f"features.{i}.adder" for i in conv_at]
+    assert tuple(net.features[0].adder.shape) == (64, 3, 3, 3)   # the first layer is an adder layer too
+    for i in conv_at:
+        assert f"features.{i + 1}.running_mean" in keys and f"features.{i + 1}.weight" in keys
+    # dropout=True, small=False: Dropout, Linear, ReLU, Dropout, Linear, ReLU, Linear
+    assert [k for k in keys if k.startswith("classifier")] == [
+        "classifier.1.weight", "classifier.1.bias", "classifier.4.weight", "classifier.4.bias",
+        "classifier.6.weight", "classifier.6.bias"]
+    assert [k for k in models.vgg19_small_add(adder2d_cls=_oracle_layer()).state_dict() if k.startswith("classifier")] == [
+        "classifier.0.weight", "classifier.0.bias", "classifier.2.weight", "classifier.2.bias"]
+    assert [k for k in models.vgg16_nd_ss(adder2d_cls=_oracle_layer()).state_dict() if k.startswith("classifier")] == [
+        "classifier.1.weight", "classifier.1.bias"]
+    counts = {"vgg11": 8, "vgg13_bn": 10, "vgg16_nd": 13, "vgg19": 16}
+    for name, n in counts.items():
+        m = getattr(models, name)(adder2d_cls=_oracle_layer())
+        assert sum(k.endswith(".adder") for k in m.state_dict()) == n, name
+    # the fused and the stock-module builds have the same keys and the same function
+    plain = models.vgg11_nd_s(adder2d_cls=_oracle_layer(), fused=False)
+    fused = models.vgg11_nd_s(adder2d_cls=_oracle_layer())
+    assert list(plain.state_dict()) == list(fused.state_dict())
+    plain.load_state_dict(fused.state_dict())
+    x = torch.randn(2, 3, 32, 32)
+    a, b = fused(x), plain(x)
+    assert a.shape == (2, 10) and torch.allclose(a, b, rtol=1e-4, atol=1e-4)
+
+
+def test_densenet_variants_have_the_reference_depths():
+    """densenet.py:93-106: block counts and growth rates; one adder 1x1 + one adder 3x3 per bottleneck, one adder
+    1x1 per transition."""
+    from addernetcuda_amd import models
+    for name, blocks, growth in (("DenseNet121", (6, 12, 24, 16), 32), ("DenseNet169", (6, 12, 32, 32), 32),
+                                 ("DenseNet201", (6, 12, 48, 32), 32), ("DenseNet161", (6, 12, 36, 24), 48)):
+        net = getattr(models, name)(adder2d_cls=_oracle_layer())
+        assert sum(k.endswith(".adder") for k in net.state_dict()) == 2 * sum(blocks) + 3, name
+        assert net.conv1.out_channels == 2 * growth and net.dense1[0].conv2.adder.shape[0] == growth
+
+
 def test_densenet_keys_and_cpu_forward():
     from addernetcuda_amd.models import densenet_cifar
     torch.manual_seed(0)
