@@ -31,6 +31,8 @@ _SIGNATURES = {
     "adder_conv2d_bwd_workspace_bytes": (_i, [_i] * 9 + [_szp]),
     "adder_conv2d_bwd_f32": (_i, [_p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_add_f32": (_i, [_p, _p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
+    "adder_conv2d_fwd_bf16": (_i, [_p, _p, _p] + [_i] * 9 + [_p]),
+    "adder_conv2d_bwd_bf16": (_i, [_p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_noalloc_f32": (_i, [_p, _p, _p, _p, _p, _f] + [_i] * 9 + [_p]),
     "adder_col_fwd_f32": (_i, [_p, _p, _p, _i, _l, _i, _p]),
     "adder_col_bwd_workspace_bytes": (_i, [_i, _l, _i, _szp]),
@@ -71,6 +73,18 @@ def check(status, what):
         if status == -5:
             msg += ": " + lib.adder_last_hip_error().decode()
         raise RuntimeError(f"{what}: {msg}")
+
+
+def require_gpu_bf16(t, name):
+    """The same checks for an activation tensor of the optional bfloat16 storage mode."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype != torch.bfloat16:
+        raise RuntimeError(f"{name} must be bfloat16, got {t.dtype}")
 
 
 def require_gpu_f32(t, name):

@@ -5,6 +5,10 @@
 and the adaptive grad_W scaling of adder.py:78 happens inside the backward
 launch.  ``adder.apply(W_col, X_col)`` keeps the column-matrix contract of
 adder.py:43-80 for callers that build X_col themselves.
+
+Everything is float32, like the reference.  One optional mode deviates, and only when asked for by passing a
+bfloat16 input: activations and their gradients stored as bfloat16, weights and all accumulation unchanged
+(``_adder_nchw_bf16``).
 """
 import ctypes
 import math
@@ -14,8 +18,8 @@ import torch.nn as nn
 from torch.autograd import Function
 
 from . import adder_cuda
-from ._lib import (lib, check, ptr, require_gpu_f32, same_device, stream_ptr, conv_dims, conv2d_bwd_workspace,
-                   fwd_stats_slots, on_device, GradWStage)
+from ._lib import (lib, check, ptr, require_gpu_f32, require_gpu_bf16, same_device, stream_ptr, conv_dims,
+                   conv2d_bwd_workspace, fwd_stats_slots, on_device, GradWStage)
 
 DEFAULT_ETA = 0.2  # adder.py:78 divides by 5
 
@@ -226,6 +230,44 @@ class _adder_nchw(Function):
         return gx, gw_out, None, None, None, None, None
 
 
+class _adder_nchw_bf16(Function):
+    """The optional reduced-storage mode: X, the output and their gradients are bfloat16 tensors (half the HBM
+    traffic and activation memory), W and its gradient stay float32, and every sum is accumulated exactly as in the
+    float32 path (fp32 for the output and grad_X, fp64 for grad_W); results are rounded to bfloat16 once, on the
+    way out.  The reference has no such mode (adder.cu:310-318 is float only); it is chosen by passing a bfloat16
+    input and is never a default."""
+
+    @staticmethod
+    def forward(ctx, X, W, stride, padding, eta):
+        X, W = X.contiguous(), W.contiguous()
+        require_gpu_bf16(X, "X")
+        require_gpu_f32(W, "W")
+        dev = same_device(X, W)
+        dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
+        out = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.bfloat16)
+        with on_device(dev):
+            check(lib.adder_conv2d_fwd_bf16(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_bf16")
+        ctx.save_for_backward(X, W)
+        ctx.dims, ctx.eta = dims, eta
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        X, W = ctx.saved_tensors
+        grad_out = grad_out.to(torch.bfloat16).contiguous()
+        require_gpu_bf16(grad_out, "grad_output")
+        dev = X.device
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        gx = torch.empty_like(X) if need_x else None
+        gw = torch.empty_like(W) if need_w else None
+        if need_x or need_w:
+            with on_device(dev):
+                ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev) if need_w else (None, 0)
+                check(lib.adder_conv2d_bwd_bf16(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw), float(ctx.eta or 0.0),
+                                                ptr(ws), nbytes, *ctx.dims, stream_ptr(dev)), "adder_conv2d_bwd_bf16")
+        return gx, gw, None, None, None
+
+
 def plain_conv2d_forward(X, W, stride, padding):
     """An *ordinary* convolution ``F.conv2d(X, W, None, stride, padding)`` through the adder forward's tiled
     kernel (3x3 / stride 1 / pad 1), with the BatchNorm partial sums of its output: (y, stats), or (None, None)
@@ -281,6 +323,8 @@ def adder2d_function(X, W, stride=1, padding=0, eta=DEFAULT_ETA):
     if W.size(2) != W.size(3):
         # the reference passes only h_filter to unfold (adder.py:32): kernels are square
         raise RuntimeError("adder2d_function expects a square kernel")
+    if X.dtype == torch.bfloat16:   # opt-in: bfloat16 activations, float32 weights and accumulation
+        return _adder_nchw_bf16.apply(X, W if W.dtype == torch.float32 else W.float(), int(stride), int(padding), eta)
     return _adder_nchw.apply(X, W, int(stride), int(padding), eta)
 
 
@@ -323,7 +367,7 @@ class adder2d(nn.Module):
     def forward(self, x):
         output = adder2d_function(x, self.adder, self.stride, self.padding, self.eta)
         if self.bias:
-            output = output + self.b.unsqueeze(0).unsqueeze(2).unsqueeze(3)
+            output = output + self.b.to(output.dtype).unsqueeze(0).unsqueeze(2).unsqueeze(3)
         return output
 
     def forward_with_stats(self, x, with_shortcut=False):
@@ -331,7 +375,7 @@ class adder2d(nn.Module):
         ``BatchNormAct2d.forward(..., stats=stats)``, or None (bias layers, shapes without the epilogue).
         ``with_shortcut``: (output, stats, shortcut) with ``shortcut`` = x routed through this layer's
         autograd node (see ``adder2d_function_with_stats``)."""
-        if self.bias:
+        if self.bias or x.dtype != torch.float32:   # (the statistics epilogue belongs to the float32 kernels)
             return (self.forward(x), None, x) if with_shortcut else (self.forward(x), None)
         return adder2d_function_with_stats(x, self.adder, self.stride, self.padding, self.eta, with_shortcut)
 

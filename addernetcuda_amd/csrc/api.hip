@@ -86,7 +86,7 @@ const char *adder_strerror(int status) {
 
 const char *adder_last_hip_error(void) { return g_last_hip_error.c_str(); }
 
-int adder_abi_version(void) { return 2; }
+int adder_abi_version(void) { return 3; }
 
 int adder_out_dim(int h, int k, int pad, int stride) {
     if (h <= 0 || k <= 0 || pad < 0 || stride <= 0 || h + 2 * pad < k) return 0;
@@ -200,6 +200,45 @@ static int conv2d_bwd(const float *gy, const float *x, const float *w, const flo
         if (int rc = launch_grad_x(gy, x, w, gx, d, s, gx_add)) return rc;
     if (gw)
         if (int rc = launch_grad_w(gy, x, w, gw, eta, ws, ws_bytes, d, s)) return rc;
+    return ADDER_OK;
+}
+
+int adder_conv2d_fwd_bf16(const adder_bf16 *x, const float *w, adder_bf16 *y, int N, int Ci, int H, int W, int Co,
+                          int kh, int kw, int stride, int pad, void *stream) {
+    if (!x || !w || !y) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const size_t nx = sizeof(adder_bf16) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(adder_bf16) * (size_t)N * Co * d.Ho * d.Wo;
+    if (overlaps(y, ny, x, nx) || overlaps(y, ny, w, nw)) return ADDER_ERR_ALIAS;
+    return launch_fwd_bf16(x, w, y, d, static_cast<hipStream_t>(stream));
+}
+
+int adder_conv2d_bwd_bf16(const adder_bf16 *gy, const adder_bf16 *x, const float *w, adder_bf16 *gx, float *gw,
+                          float eta, void *ws, size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw,
+                          int stride, int pad, void *stream) {
+    if (!gy || !x || !w) return ADDER_ERR_NULL_POINTER;
+    if (!gx && !gw) return ADDER_ERR_NULL_POINTER;
+    if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const size_t nx = sizeof(adder_bf16) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(adder_bf16) * (size_t)N * Co * d.Ho * d.Wo;
+    if (overlaps(gx, nx, x, nx) || overlaps(gx, nx, w, nw) || overlaps(gx, nx, gy, ny) || overlaps(gw, nw, x, nx) ||
+        overlaps(gw, nw, w, nw) || overlaps(gw, nw, gy, ny) || overlaps(gw, nw, gx, nx))
+        return ADDER_ERR_ALIAS;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (gw) {
+        const size_t need = grad_w_workspace_bytes(d);
+        if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
+        if (overlaps(ws, need, x, nx) || overlaps(ws, need, w, nw) || overlaps(ws, need, gy, ny) ||
+            overlaps(ws, need, gx, nx) || overlaps(ws, need, gw, nw))
+            return ADDER_ERR_ALIAS;
+    }
+    if (gx)
+        if (int rc = launch_grad_x_bf16(gy, x, w, gx, d, s)) return rc;
+    if (gw)
+        if (int rc = launch_grad_w_bf16(gy, x, w, gw, eta, ws, ws_bytes, d, s)) return rc;
     return ADDER_OK;
 }
 

@@ -30,6 +30,43 @@ __device__ __forceinline__ void l2_warm(const float *p, int rows, int pitch, int
     }
 }
 
+// Storage types of activations: float, or bfloat16 (the upper half of a float, round to nearest even on the way
+// out) for the optional reduced-storage mode; arithmetic is fp32 (fp64 for the weight gradient) either way.
+typedef uint16_t bf16_t;
+__device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    u += 0x7fffu + ((u >> 16) & 1u);   // round to nearest, ties to even (NaN payloads are not preserved)
+    return (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ float ldf(const float *p) { return *p; }
+__device__ __forceinline__ float ldf(const bf16_t *p) { return bf16_to_f32(*p); }
+__device__ __forceinline__ void stf(float *p, float v) { *p = v; }
+__device__ __forceinline__ void stf(bf16_t *p, float v) { *p = f32_to_bf16(v); }
+// four / two consecutive elements at an address aligned to their total size
+__device__ __forceinline__ float4 ldf4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 ldf4(const bf16_t *p) {
+    const uint2 u = *reinterpret_cast<const uint2 *>(p);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                       __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void stf4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ void stf4(bf16_t *p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+    u.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+    *reinterpret_cast<uint2 *>(p) = u;
+}
+__device__ __forceinline__ float2 ldf2(const float *p) { return *reinterpret_cast<const float2 *>(p); }
+__device__ __forceinline__ float2 ldf2(const bf16_t *p) {
+    const uint32_t u = *reinterpret_cast<const uint32_t *>(p);
+    return make_float2(__uint_as_float(u << 16), __uint_as_float(u & 0xffff0000u));
+}
+__device__ __forceinline__ void stf2(float *p, float2 v) { *reinterpret_cast<float2 *>(p) = v; }
+__device__ __forceinline__ void stf2(bf16_t *p, float2 v) {
+    *reinterpret_cast<uint32_t *>(p) = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+}
+
 // Clamp to [0, 1]: the compiler folds it into the clamp output modifier of the instruction that
 // produces v, so it costs no instruction of its own.
 __device__ __forceinline__ float sat01(float v) { return __builtin_amdgcn_fmed3f(v, 0.f, 1.f); }
@@ -174,6 +211,14 @@ int launch_norm_scale_batched(int count, float *const *g, const long *n, const f
 
 int launch_grad_w_slab_finalize(const double *part, const double *sgpart, const float *w, float *gw, int slots, int Co,
                                 int K, bool accumulate, hipStream_t s);
+// bfloat16 storage of x / y / gy / gx (weights and weight gradients stay fp32): the tiled 3x3 / pad-1 kernels and
+// the generic ones
+int launch_fwd_bf16(const bf16_t *x, const float *w, bf16_t *y, const ConvDims &d, hipStream_t s);
+int launch_grad_x_bf16(const bf16_t *gy, const bf16_t *x, const float *w, bf16_t *gx, const ConvDims &d, hipStream_t s);
+int launch_grad_w_bf16(const bf16_t *gy, const bf16_t *x, const float *w, float *gw, float eta, void *ws, size_t ws_bytes,
+                       const ConvDims &d, hipStream_t s);
+int launch_grad_w_mfma_bf16(const bf16_t *gy, const bf16_t *x, double *part, double *sgpart, const ConvDims &d,
+                            const GradWMfmaPlan &p, hipStream_t s);
 int launch_col_fwd(const float *X, const float *W, float *out, int K, long NL, int Co, hipStream_t s);
 size_t col_grad_w_workspace_bytes(int K, long NL, int Co);
 int launch_col_grad_w(const float *gy, const float *X, const float *W, float *gW, int K, long NL,

@@ -22,10 +22,10 @@ namespace adder {
 // One output position per lane, TM output channels per lane, input read
 // straight from global memory with bounds checks.
 // ---------------------------------------------------------------------------
-template <int TM>
-__global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restrict__ x,
+template <int TM, class T = float>
+__global__ __launch_bounds__(256) void fwd_generic_kernel(const T *__restrict__ x,
                                                           const float *__restrict__ w,
-                                                          float *__restrict__ y, ConvDims d) {
+                                                          T *__restrict__ y, ConvDims d) {
     const int total = d.N * d.Ho * d.Wo;
     int pos = blockIdx.x * 256 + threadIdx.x;
     const bool active = pos < total;
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 #pragma unroll
     for (int m = 0; m < TM; ++m) wrow[m] = min(co0 + m, d.Co - 1) * K;
 
-    const float *xn = x + (size_t)n * d.Ci * d.H * d.W;
+    const T *xn = x + (size_t)n * d.Ci * d.H * d.W;
     for (int ci = 0; ci < d.Ci; ++ci) {
         for (int i = 0; i < d.kh; ++i) {
             const int hi = ho * d.stride + i - d.pad;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
             for (int j = 0; j < d.kw; ++j) {
                 const int wi = wo * d.stride + j - d.pad;
                 const bool v = hv && wi >= 0 && wi < d.W;
-                const float xv = v ? xn[((size_t)ci * d.H + hi) * d.W + wi] : 0.f;
+                const float xv = v ? ldf(xn + ((size_t)ci * d.H + hi) * d.W + wi) : 0.f;
                 const int k = (ci * d.kh + i) * d.kw + j;
 #pragma unroll
                 for (int m = 0; m < TM; ++m) acc[m] -= fabsf(wc[wrow[m] + k] - xv);
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
     if (active) {
 #pragma unroll
         for (int m = 0; m < TM; ++m)
-            if (co0 + m < d.Co) y[(((size_t)n * d.Co + co0 + m) * d.Ho + ho) * d.Wo + wo] = tot[m];
+            if (co0 + m < d.Co) stf(y + (((size_t)n * d.Co + co0 + m) * d.Ho + ho) * d.Wo + wo, tot[m]);
     }
 }
 
@@ -86,10 +86,11 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const float *__restric
 // ---------------------------------------------------------------------------
 // MUL: the same kernel as an ordinary convolution, y = sum w * x (one v_fmac per term), for the regular
 // stem layer that precedes the adder layers of a network.
-template <class C, bool VEC = true, bool SUB = false, bool MUL = false>
-__global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__restrict__ x,
+// T: storage type of x and y (float, or bf16_t for the reduced-storage mode); the arithmetic is fp32 either way.
+template <class C, bool VEC = true, bool SUB = false, bool MUL = false, class T = float>
+__global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restrict__ x,
                                                                 const float *__restrict__ w,
-                                                                float *__restrict__ y,
+                                                                T *__restrict__ y,
                                                                 double *__restrict__ stats, int N, int Ci,
                                                                 int H, int W, int Co, int Ho, int Wo,
                                                                 int tilesH, int tilesW, const Subsample sub) {
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
     const int nchunks = ceil_div(Ci, C::CC);
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch, VEC, SUB>(st, x, 0, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W, sub);
+    tile_fetch<typename C::Patch, VEC, SUB, T>(st, x, 0, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W, sub);
     {   // this workgroup's output channels: one contiguous run of weights
         const int co_blk = blockIdx.y * C::COW * TM;
         l2_warm(w + (size_t)co_blk * K, 1, 0, min(C::COW * TM, Co - co_blk) * K);
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
 
     for (int c = 0; c < nchunks; ++c) {
         const int ci0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC, SUB>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W, sub);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC, SUB, T>(st, x, ci0 + C::CC, Ci, n0, N, h0 * S - C::PAD, w0 * S, H, W, sub);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Ci - ci0);
@@ -250,41 +251,40 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const float *__res
         for (int m = 0; m < TM; ++m) {
             const int co = co_base + m;
             if (co < Co) {
-                float *dst = y + (((size_t)n * Co + co) * Ho + ho) * Wo + wo;
+                T *dst = y + (((size_t)n * Co + co) * Ho + ho) * Wo + wo;
                 if (vec) {
 #pragma unroll
                     for (int t = 0; t + 3 < TN; t += 4)
-                        *reinterpret_cast<float4 *>(dst + t) =
-                            make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]);
+                        stf4(dst + t, make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]));
                 } else {
 #pragma unroll
                     for (int t = 0; t < TN; ++t)
-                        if (wo + t < Wo) dst[t] = tot[m][t];
+                        if (wo + t < Wo) stf(dst + t, tot[m][t]);
                 }
             }
         }
     }
 }
 
-template <class C, bool VEC, bool SUB = false, bool MUL = false>
-static int launch_fwd_3x3_v(const float *x, const float *w, float *y, double *stats, const ConvDims &d,
+template <class C, bool VEC, bool SUB = false, bool MUL = false, class T = float>
+static int launch_fwd_3x3_v(const T *x, const float *w, T *y, double *stats, const ConvDims &d,
                             hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
     const int tilesH = ceil_div(d.Ho, C::TH), tilesW = ceil_div(d.Wo, C::TW);
     const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gy = ceil_div(d.Co, C::TM * C::COW);
     if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    if (int rc = allow_dynamic_lds<&fwd_3x3_kernel<C, VEC, SUB, MUL>>(C::LDS_BYTES)) return rc;
-    hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC, SUB, MUL>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
+    if (int rc = allow_dynamic_lds<&fwd_3x3_kernel<C, VEC, SUB, MUL, T>>(C::LDS_BYTES)) return rc;
+    hipLaunchKernelGGL((fwd_3x3_kernel<C, VEC, SUB, MUL, T>), dim3((unsigned)gx, gy), dim3(C::NTHREADS), C::LDS_BYTES, s, x, w, y,
                        stats, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, sub);
     return check_launch();
 }
 
-template <class C>
-static int launch_fwd_3x3(const float *x, const float *w, float *y, double *stats, const ConvDims &d,
+template <class C, class T = float>
+static int launch_fwd_3x3(const T *x, const float *w, T *y, double *stats, const ConvDims &d,
                           hipStream_t s) {
-    // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
-    if (d.W % 4 == 0) return launch_fwd_3x3_v<C, true>(x, w, y, stats, d, s);
-    return launch_fwd_3x3_v<C, false>(x, w, y, stats, d, s);
+    // element-wise tile loads when the rows of the staged tensor are not whole groups of four
+    if (d.W % 4 == 0) return launch_fwd_3x3_v<C, true, false, false, T>(x, w, y, stats, d, s);
+    return launch_fwd_3x3_v<C, false, false, false, T>(x, w, y, stats, d, s);
 }
 
 // the same tile shapes as an ordinary convolution (3x3 / stride 1 / pad 1 only)
@@ -420,6 +420,30 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
     constexpr int TM = 8;
     const long total = (long)d.N * d.Ho * d.Wo;
     hipLaunchKernelGGL(fwd_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Co, TM)),
+                       dim3(256), 0, s, x, w, y, d);
+    return check_launch();
+}
+
+// bfloat16 storage: the tiled 3x3 / pad-1 kernels (stride 1 or 2), the generic kernel for everything else
+int launch_fwd_bf16(const bf16_t *x, const float *w, bf16_t *y, const ConvDims &d, hipStream_t s) {
+    const bool k3p1 = d.kh == 3 && d.kw == 3 && d.pad == 1 &&
+                      (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 7) == 0) &&
+                      (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 7) == 0);
+    if (k3p1) {
+        const int variant = d.stride == 1 ? (d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3)) : (d.stride == 2 ? (d.Wo > 8 ? 4 : 5) : 0);
+        switch (variant) {
+            case 1: return launch_fwd_3x3<FwdW32, bf16_t>(x, w, y, nullptr, d, s);
+            case 2: return launch_fwd_3x3<FwdW16, bf16_t>(x, w, y, nullptr, d, s);
+            case 3: return launch_fwd_3x3<FwdW8, bf16_t>(x, w, y, nullptr, d, s);
+            case 4: return launch_fwd_3x3<FwdW16S2, bf16_t>(x, w, y, nullptr, d, s);
+            case 5: return d.Ci >= 128 ? launch_fwd_3x3<FwdW8S2L, bf16_t>(x, w, y, nullptr, d, s)
+                                       : launch_fwd_3x3<FwdW8S2, bf16_t>(x, w, y, nullptr, d, s);
+            default: break;
+        }
+    }
+    constexpr int TM = 8;
+    const long total = (long)d.N * d.Ho * d.Wo;
+    hipLaunchKernelGGL((fwd_generic_kernel<TM, bf16_t>), dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Co, TM)),
                        dim3(256), 0, s, x, w, y, d);
     return check_launch();
 }

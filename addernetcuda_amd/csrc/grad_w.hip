@@ -20,9 +20,9 @@ static constexpr int kNormBlocksMax = 16384;  // sum-of-squares partials kept at
 // Generic kernel: one workgroup per (co, ci) [KH x KW taps in registers] or,
 // for KH = 0, one workgroup per (co, ci, i, j).  Direct (x - w) * g form.
 // ---------------------------------------------------------------------------
-template <int KH, int KW>
-__global__ __launch_bounds__(256) void grad_w_generic_kernel(const float *__restrict__ gy,
-                                                             const float *__restrict__ x,
+template <int KH, int KW, class ST = float>
+__global__ __launch_bounds__(256) void grad_w_generic_kernel(const ST *__restrict__ gy,
+                                                             const ST *__restrict__ x,
                                                              const float *__restrict__ w,
                                                              float *__restrict__ gw, ConvDims d) {
     constexpr int T = KH > 0 ? KH * KW : 1;
@@ -53,13 +53,13 @@ __global__ __launch_bounds__(256) void grad_w_generic_kernel(const float *__rest
     for (int pos = threadIdx.x; pos < total; pos += 256) {
         const int l = pos % L, n = pos / L;
         const int ho = l / d.Wo, wo = l % d.Wo;
-        const float g = gy[((size_t)n * d.Co + co) * L + l];
-        const float *xp = x + ((size_t)n * d.Ci + ci) * d.H * d.W;
+        const float g = ldf(gy + ((size_t)n * d.Co + co) * L + l);
+        const ST *xp = x + ((size_t)n * d.Ci + ci) * d.H * d.W;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const int hi = ho * d.stride + ti[t] - d.pad, wi = wo * d.stride + tj[t] - d.pad;
             const bool v = hi >= 0 && hi < d.H && wi >= 0 && wi < d.W;
-            const float xv = v ? xp[(size_t)hi * d.W + wi] : 0.f;
+            const float xv = v ? ldf(xp + (size_t)hi * d.W + wi) : 0.f;
             acc[t] = fmaf(xv - wv[t], g, acc[t]);
         }
         if (++it == 64) {  // keep fp32 runs short; carry the rest in fp64
@@ -409,6 +409,40 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
                            gw, d);
     int rc = check_launch();
     if (rc) return rc;
+    if (eta > 0.f) return launch_norm_scale(gw, n, eta, 1e-12f, ws, s);
+    return ADDER_OK;
+}
+
+// bfloat16 storage of gy and x (gw and w stay fp32): the matrix-core kernel for 3x3 / pad-1 layers, the generic
+// kernel for everything else; the same finalize and scaling as the fp32 path
+int launch_grad_w_bf16(const bf16_t *gy, const bf16_t *x, const float *w, float *gw, float eta, void *ws,
+                       size_t ws_bytes, const ConvDims &d, hipStream_t s) {
+    if (ws_bytes < grad_w_workspace_bytes(d)) return ADDER_ERR_WORKSPACE;
+    GradWPlan p = plan_grad_w(d);
+    const bool tiled = p.variant == 2 && d.kh == 3 && (d.W % 4 != 0 || (reinterpret_cast<uintptr_t>(x) & 7) == 0) &&
+                       (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 7) == 0);
+    double *ss = reinterpret_cast<double *>(ws);
+    const int K = d.K();
+    const long n = (long)d.Co * K;
+    if (tiled) {
+        double *part = reinterpret_cast<double *>(ss + kNormBlocksMax);
+        double *sgpart = part + (size_t)p.slots * d.Co * K;
+        if (int rc = launch_grad_w_mfma_bf16(gy, x, part, sgpart, d, p.mfma, s)) return rc;
+        const int nb = (int)ceil_div_l(n, kFinOut);
+        hipLaunchKernelGGL(grad_w_finalize_kernel<double>, dim3(nb), dim3(kFinOut * kFinLanes), 0, s, part, sgpart, w, gw,
+                           nullptr, p.slots, d.Co, K);
+    } else {
+        const int KK = d.kh * d.kw;
+        const long wgs = (long)d.Co * d.Ci;
+        if (d.kh == 3 && d.kw == 3)
+            hipLaunchKernelGGL((grad_w_generic_kernel<3, 3, bf16_t>), dim3((unsigned)wgs), dim3(256), 0, s, gy, x, w, gw, d);
+        else if (d.kh == 1 && d.kw == 1)
+            hipLaunchKernelGGL((grad_w_generic_kernel<1, 1, bf16_t>), dim3((unsigned)wgs), dim3(256), 0, s, gy, x, w, gw, d);
+        else
+            hipLaunchKernelGGL((grad_w_generic_kernel<0, 0, bf16_t>), dim3((unsigned)(wgs * KK)), dim3(256), 0, s, gy, x, w,
+                               gw, d);
+    }
+    if (int rc = check_launch()) return rc;
     if (eta > 0.f) return launch_norm_scale(gw, n, eta, 1e-12f, ws, s);
     return ADDER_OK;
 }

@@ -59,8 +59,8 @@ struct GwMfmaCfg {
 template <class G>
 struct GyStageM { float4 v[G::GITER]; };
 
-template <class G, bool VEC>
-__device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const float *__restrict__ gy, int co0, int Co, int n0,
+template <class G, bool VEC, class T = float>
+__device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const T *__restrict__ gy, int co0, int Co, int n0,
                                            int N, int h0, int w0, int Ho, int Wo) {
 #pragma unroll
     for (int it = 0; it < G::GITER; ++it) {
@@ -73,14 +73,14 @@ __device__ __forceinline__ void gy_fetch_m(GyStageM<G> &st, const float *__restr
         const bool ok = (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) && n < N && co < Co && ho < Ho && wo < Wo;
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok) {
-            const float *row = gy + (((n * Co + co) * Ho + ho) * Wo + wo);
+            const T *row = gy + (((n * Co + co) * Ho + ho) * Wo + wo);
             if constexpr (VEC) {
-                val = *reinterpret_cast<const float4 *>(row);
-            } else {   // rows are not 16-byte aligned (Wo % 4 != 0)
-                val.x = row[0];
-                if (wo + 1 < Wo) val.y = row[1];
-                if (wo + 2 < Wo) val.z = row[2];
-                if (wo + 3 < Wo) val.w = row[3];
+                val = ldf4(row);
+            } else {   // rows are not whole aligned groups of four (Wo % 4 != 0)
+                val.x = ldf(row);
+                if (wo + 1 < Wo) val.y = ldf(row + 1);
+                if (wo + 2 < Wo) val.z = ldf(row + 2);
+                if (wo + 3 < Wo) val.w = ldf(row + 3);
             }
         }
         st.v[it] = val;
@@ -103,9 +103,10 @@ __device__ __forceinline__ void gy_commit_m(const GyStageM<G> &st, float *buf) {
 
 // SUB (single tap only): x is a sampled tensor (see Subsample), read element by element at the sampled
 // positions; gy is dense.  VEC then only says how gy is read.
-template <class G, bool VEC = true, bool SUB = false>
-__global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *__restrict__ gy,
-                                                                  const float *__restrict__ x,
+// T: storage type of gy and x (float, or bf16_t for the reduced-storage mode); staged as fp32, multiplied in fp64.
+template <class G, bool VEC = true, bool SUB = false, class T = float>
+__global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__restrict__ gy,
+                                                                  const T *__restrict__ x,
                                                                   double *__restrict__ part,
                                                                   double *__restrict__ sgpart, int N, int Ci, int H,
                                                                   int W, int Co, int Ho, int Wo, int tilesH,
@@ -150,8 +151,8 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
     };
     if (tile < ntiles) {
         decode(tile);
-        tile_fetch<XP, VEC && !SUB, SUB>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
-        gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+        tile_fetch<XP, VEC && !SUB, SUB, T>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
+        gy_fetch_m<G, VEC, T>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         tile_commit<XP>(xs, smem);
         gy_commit_m<G>(gs, smem + XP::BUF);
     }
@@ -162,8 +163,8 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const float *_
         const int next = tile + gridDim.x;
         if (next < ntiles) {   // next tile's global loads fly during this tile's arithmetic
             decode(next);
-            tile_fetch<XP, VEC && !SUB, SUB>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
-            gy_fetch_m<G, VEC>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+            tile_fetch<XP, VEC && !SUB, SUB, T>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
+            gy_fetch_m<G, VEC, T>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         }
         const float *base = smem + cur * G::BUF;
         auto steps = [&](const int first, const int last) {
@@ -335,21 +336,34 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     return p;
 }
 
-template <class G, bool VEC, bool SUB = false>
-static int launch_one_v(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+template <class G, bool VEC, bool SUB = false, class T = float>
+static int launch_one_v(const T *gy, const T *x, double *part, double *sgpart, const ConvDims &d,
                       const GradWMfmaPlan &p, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
-    if (int rc = allow_dynamic_lds<&grad_w_mfma_kernel<G, VEC, SUB>>(G::LDS_BYTES)) return rc;
-    hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC, SUB>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
+    if (int rc = allow_dynamic_lds<&grad_w_mfma_kernel<G, VEC, SUB, T>>(G::LDS_BYTES)) return rc;
+    hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC, SUB, T>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
                        part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles, sub);
     return check_launch();
 }
 
-template <class G>
-static int launch_one(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+template <class G, class T = float>
+static int launch_one(const T *gy, const T *x, double *part, double *sgpart, const ConvDims &d,
                       const GradWMfmaPlan &p, hipStream_t s) {
-    // element-wise tile loads unless the rows of both x and gy are whole float4 groups
-    if (d.W % 4 == 0 && d.Wo % 4 == 0) return launch_one_v<G, true>(gy, x, part, sgpart, d, p, s);
-    return launch_one_v<G, false>(gy, x, part, sgpart, d, p, s);
+    // element-wise tile loads unless the rows of both x and gy are whole groups of four
+    if (d.W % 4 == 0 && d.Wo % 4 == 0) return launch_one_v<G, true, false, T>(gy, x, part, sgpart, d, p, s);
+    return launch_one_v<G, false, false, T>(gy, x, part, sgpart, d, p, s);
+}
+
+// bfloat16 storage of gy and x: the 3x3 / pad-1 variants (1..5 of the plan)
+int launch_grad_w_mfma_bf16(const bf16_t *gy, const bf16_t *x, double *part, double *sgpart, const ConvDims &d,
+                            const GradWMfmaPlan &p, hipStream_t s) {
+    switch (p.variant) {
+        case 1: return launch_one<GmW32, bf16_t>(gy, x, part, sgpart, d, p, s);
+        case 2: return launch_one<GmW16, bf16_t>(gy, x, part, sgpart, d, p, s);
+        case 3: return launch_one<GmW8, bf16_t>(gy, x, part, sgpart, d, p, s);
+        case 4: return launch_one<GmW16S2, bf16_t>(gy, x, part, sgpart, d, p, s);
+        case 5: return launch_one<GmW8S2, bf16_t>(gy, x, part, sgpart, d, p, s);
+        default: return ADDER_ERR_UNSUPPORTED;
+    }
 }
 
 int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,

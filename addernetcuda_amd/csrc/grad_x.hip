@@ -29,11 +29,11 @@ namespace adder {
 // ---------------------------------------------------------------------------
 // Generic kernel: any kernel size / stride / padding.
 // ---------------------------------------------------------------------------
-template <int TM>
-__global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__restrict__ gy,
-                                                             const float *__restrict__ x,
+template <int TM, class T = float>
+__global__ __launch_bounds__(256) void grad_x_generic_kernel(const T *__restrict__ gy,
+                                                             const T *__restrict__ x,
                                                              const float *__restrict__ w,
-                                                             float *__restrict__ gx, ConvDims d) {
+                                                             T *__restrict__ gx, ConvDims d) {
     const int total = d.N * d.H * d.W;
     int pos = blockIdx.x * 256 + threadIdx.x;
     const bool active = pos < total;
@@ -51,11 +51,11 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = min(ci0 + m, d.Ci - 1);
-        xr[m] = x[(((size_t)n * d.Ci + ci) * d.H + hi) * d.W + wi];
+        xr[m] = ldf(x + (((size_t)n * d.Ci + ci) * d.H + hi) * d.W + wi);
         acc[m] = tot[m] = 0.f;
         wofs[m] = ci * KK;
     }
-    const float *gn = gy + (size_t)n * d.Co * d.Ho * d.Wo;
+    const T *gn = gy + (size_t)n * d.Co * d.Ho * d.Wo;
     for (int co = 0; co < d.Co; ++co) {
         for (int i = 0; i < d.kh; ++i) {
             const int th = hi + d.pad - i;
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
                 const int tw = wi + d.pad - j;
                 const int wo = tw / d.stride;
                 const bool v = hv && tw >= 0 && wo * d.stride == tw && wo < d.Wo;
-                const float g = v ? gn[((size_t)co * d.Ho + ho) * d.Wo + wo] : 0.f;
+                const float g = v ? ldf(gn + ((size_t)co * d.Ho + ho) * d.Wo + wo) : 0.f;
                 const int kofs = co * K + i * d.kw + j;
 #pragma unroll
                 for (int m = 0; m < TM; ++m)
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
     if (active) {
 #pragma unroll
         for (int m = 0; m < TM; ++m)
-            if (ci0 + m < d.Ci) gx[(((size_t)n * d.Ci + ci0 + m) * d.H + hi) * d.W + wi] = tot[m];
+            if (ci0 + m < d.Ci) stf(gx + (((size_t)n * d.Ci + ci0 + m) * d.H + hi) * d.W + wi, tot[m]);
     }
 }
 
@@ -95,14 +95,15 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const float *__rest
 // SUB (single tap only): x and gx are sampled tensors (see Subsample); the kernel walks the sampled
 // positions as one row per plane, reads x there, and stores each result together with the zeros of the
 // s x s block of input positions around it that the layer never read.
-template <class C, bool VEC = true, bool SAT = true, bool SUB = false>
-__global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const float *__restrict__ gy,
-                                                                   const float *__restrict__ x,
+// T: storage type of gy, x, gx and gadd (float, or bf16_t for the reduced-storage mode).
+template <class C, bool VEC = true, bool SAT = true, bool SUB = false, class T = float>
+__global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *__restrict__ gy,
+                                                                   const T *__restrict__ x,
                                                                    const float *__restrict__ w,
-                                                                   float *__restrict__ gx, int N, int Ci,
+                                                                   T *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int tilesH,
                                                                    int tilesW, const Subsample sub,
-                                                                   const float *__restrict__ gadd) {
+                                                                   const T *__restrict__ gadd) {
     static_assert(!SUB || C::KS == 1, "sampling is for single-tap layers");
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
@@ -152,10 +153,10 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
-        const float *src = x + ((size_t)nc * Ci + ci) * xplane;
+        const T *src = x + ((size_t)nc * Ci + ci) * xplane;
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
-            const float xv = src[xoff[t]];
+            const float xv = ldf(src + xoff[t]);
             cr[m][t] = SAT ? fmaf(-0.5f, xv, 0.5f) : xv;
             acc[m][t] = tot[m][t] = 0.f;
         }
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
     const int nchunks = ceil_div(Co, C::CC);
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, h0 - C::PAD, w0, H, W);
+    tile_fetch<typename C::Patch, VEC, false, T>(st, gy, 0, Co, n0, N, h0 - C::PAD, w0, H, W);
     {   // this workgroup's input channels: one run of weights per output channel
         const int ci_blk = min((int)blockIdx.y * C::COW * TM, Ci - TM);
         l2_warm(w + ci_blk * KK, Co, K, min(C::COW * TM, Ci - ci_blk) * KK);
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 
     for (int c = 0; c < nchunks; ++c) {
         const int co0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, gy, co0 + C::CC, Co, n0, N, h0 - C::PAD, w0, H, W);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC, false, T>(st, gy, co0 + C::CC, Co, n0, N, h0 - C::PAD, w0, H, W);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
@@ -351,7 +352,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
             const int ci = ci_base + m;
             if (ci >= ci_first) {
                 if constexpr (SUB) {
-                    float *plane = gx + ((size_t)n * Ci + ci) * sub.plane;
+                    T *plane = gx + ((size_t)n * Ci + ci) * sub.plane;
                     const int rows = sub.plane / sub.pitch;
 #pragma unroll
                     for (int t = 0; t < TN; ++t) {
@@ -359,26 +360,26 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
                         const int r0 = xoff[t] / sub.pitch, c0 = xoff[t] - r0 * sub.pitch;
                         for (int a = 0; a < sub.s && r0 + a < rows; ++a)
                             for (int b = 0; b < sub.s && c0 + b < sub.pitch; ++b)
-                                plane[xoff[t] + a * sub.pitch + b] = (a | b) ? 0.f : tot[m][t];
+                                stf(plane + xoff[t] + a * sub.pitch + b, (a | b) ? 0.f : tot[m][t]);
                     }
                     continue;
                 }
                 const size_t o = (((size_t)n * Ci + ci) * H + hi) * W + wi0;
-                float *dst = gx + o;
+                T *dst = gx + o;
                 if (TN % 4 == 0 && (W & 3) == 0 && wi0 + TN <= W) {
 #pragma unroll
                     for (int t = 0; t < TN; t += 4) {
                         float4 v = make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]);
                         if (gadd) {   // a second gradient of the same tensor (a residual shortcut), added on the way out
-                            const float4 a = *reinterpret_cast<const float4 *>(gadd + o + t);
+                            const float4 a = ldf4(gadd + o + t);
                             v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
                         }
-                        *reinterpret_cast<float4 *>(dst + t) = v;
+                        stf4(dst + t, v);
                     }
                 } else {
 #pragma unroll
                     for (int t = 0; t < TN; ++t)
-                        if (wi0 + t < W) dst[t] = gadd ? tot[m][t] + gadd[o + t] : tot[m][t];
+                        if (wi0 + t < W) stf(dst + t, gadd ? tot[m][t] + ldf(gadd + o + t) : tot[m][t]);
                 }
             }
         }
@@ -393,33 +394,33 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const floa
 // and carries the full magnitude (512 -> 2048 @7x7 at batch 64 had one element in 1e5 at 1.2 of the tolerance).
 static constexpr int kSatMaxTerms = 2304, kSatMaxTerms1x1 = 1024;
 
-template <class C, bool VEC, bool SAT, bool SUB = false>
-static int launch_grad_x_3x3s1_v(const float *gy, const float *x, const float *w, float *gx,
+template <class C, bool VEC, bool SAT, bool SUB = false, class T = float>
+static int launch_grad_x_3x3s1_v(const T *gy, const T *x, const float *w, T *gx,
                                const ConvDims &d, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0},
-                               const float *gadd = nullptr) {
+                               const T *gadd = nullptr) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
-    if (int rc = allow_dynamic_lds<&grad_x_3x3s1_kernel<C, VEC, SAT, SUB>>(LDS_BYTES)) return rc;
-    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
+    if (int rc = allow_dynamic_lds<&grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T>>(LDS_BYTES)) return rc;
+    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW, sub, gadd);
     return check_launch();
 }
 
 // picks the element-wise tile loads (rows of the staged tensor that are not whole float4 groups) and the
 // three-instruction form (more terms per output than kSatMaxTerms)
-template <class C, bool SUB = false>
-static int launch_grad_x_3x3s1(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s, const float *gadd = nullptr,
+template <class C, bool SUB = false, class T = float>
+static int launch_grad_x_3x3s1(const T *gy, const T *x, const float *w, T *gx,
+                               const ConvDims &d, hipStream_t s, const T *gadd = nullptr,
                                const Subsample sub = Subsample{1, 0, 0, 0}) {
     const bool vec = d.W % 4 == 0;
     if (d.Co * C::KK > (C::KS == 1 ? kSatMaxTerms1x1 : kSatMaxTerms))
-        return vec ? launch_grad_x_3x3s1_v<C, true, false, SUB>(gy, x, w, gx, d, s, sub, gadd)
-                   : launch_grad_x_3x3s1_v<C, false, false, SUB>(gy, x, w, gx, d, s, sub, gadd);
-    return vec ? launch_grad_x_3x3s1_v<C, true, true, SUB>(gy, x, w, gx, d, s, sub, gadd)
-               : launch_grad_x_3x3s1_v<C, false, true, SUB>(gy, x, w, gx, d, s, sub, gadd);
+        return vec ? launch_grad_x_3x3s1_v<C, true, false, SUB, T>(gy, x, w, gx, d, s, sub, gadd)
+                   : launch_grad_x_3x3s1_v<C, false, false, SUB, T>(gy, x, w, gx, d, s, sub, gadd);
+    return vec ? launch_grad_x_3x3s1_v<C, true, true, SUB, T>(gy, x, w, gx, d, s, sub, gadd)
+               : launch_grad_x_3x3s1_v<C, false, true, SUB, T>(gy, x, w, gx, d, s, sub, gadd);
 }
 
 // ---------------------------------------------------------------------------
@@ -447,14 +448,14 @@ struct GradX3x3S2Cfg {
     static_assert(TNW % 2 == 0 && TH % 2 == 0, "lanes own 2 x 2 parity blocks");
 };
 
-template <class C, bool VEC = true, bool SAT = true>
-__global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *__restrict__ gy,
-                                                                   const float *__restrict__ x,
+template <class C, bool VEC = true, bool SAT = true, class T = float>
+__global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__restrict__ gy,
+                                                                   const T *__restrict__ x,
                                                                    const float *__restrict__ w,
-                                                                   float *__restrict__ gx, int N, int Ci,
+                                                                   T *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int Ho, int Wo,
                                                                    int tilesH, int tilesW,
-                                                                   const float *__restrict__ gadd) {
+                                                                   const T *__restrict__ gadd) {
     constexpr int TNW = C::TNW, TM = C::TM, GSTRIP = C::GSTRIP;
     extern __shared__ __align__(16) float smem[];
 
@@ -487,10 +488,10 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
         const int ci = ci_base + m;
 #pragma unroll
         for (int rp = 0; rp < 2; ++rp) {
-            const float *src = x + (((size_t)nc * Ci + ci) * H + min(hi0 + rp, H - 1)) * W;
+            const T *src = x + (((size_t)nc * Ci + ci) * H + min(hi0 + rp, H - 1)) * W;
 #pragma unroll
             for (int t = 0; t < TNW; ++t) {
-                const float xv = src[min(wi0 + t, W - 1)];
+                const float xv = ldf(src + min(wi0 + t, W - 1));
                 cr[m][rp][t] = SAT ? fmaf(-0.5f, xv, 0.5f) : xv;
                 acc[m][rp][t] = tot[m][rp][t] = 0.f;
             }
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
     const int hb = h0 / 2, wb = w0 / 2;
 
     TileStage<typename C::Patch> st;
-    tile_fetch<typename C::Patch, VEC>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
+    tile_fetch<typename C::Patch, VEC, false, T>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
     {   // this workgroup's input channels: one run of weights per output channel
         const int ci_blk = min((int)blockIdx.y * C::CIW * TM, Ci - TM);
         l2_warm(w + ci_blk * 9, Co, K, min(C::CIW * TM, Ci - ci_blk) * 9);
@@ -517,7 +518,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
 
     for (int c = 0; c < nchunks; ++c) {
         const int co0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC>(st, gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
+        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC, false, T>(st, gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
         const int ccnt = min(C::CC, Co - co0);
@@ -640,51 +641,51 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const float *
                 const int hi = hi0 + rp;
                 if (hi >= H) continue;
                 const size_t o = (((size_t)n * Ci + ci) * H + hi) * W + wi0;
-                float *dst = gx + o;
+                T *dst = gx + o;
                 if ((W & 1) == 0 && wi0 + TNW <= W) {
 #pragma unroll
                     for (int t = 0; t < TNW; t += 2) {
                         float2 v = make_float2(tot[m][rp][t], tot[m][rp][t + 1]);
                         if (gadd) {   // a second gradient of the same tensor, added on the way out
-                            const float2 a = *reinterpret_cast<const float2 *>(gadd + o + t);
+                            const float2 a = ldf2(gadd + o + t);
                             v.x += a.x; v.y += a.y;
                         }
-                        *reinterpret_cast<float2 *>(dst + t) = v;
+                        stf2(dst + t, v);
                     }
                 } else {
 #pragma unroll
                     for (int t = 0; t < TNW; ++t)
-                        if (wi0 + t < W) dst[t] = gadd ? tot[m][rp][t] + gadd[o + t] : tot[m][rp][t];
+                        if (wi0 + t < W) stf(dst + t, gadd ? tot[m][rp][t] + ldf(gadd + o + t) : tot[m][rp][t]);
                 }
             }
         }
     }
 }
 
-template <class C, bool VEC, bool SAT>
-static int launch_grad_x_3x3s2_v(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s, const float *gadd) {
+template <class C, bool VEC, bool SAT, class T = float>
+static int launch_grad_x_3x3s2_v(const T *gy, const T *x, const float *w, T *gx,
+                               const ConvDims &d, hipStream_t s, const T *gadd) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
-    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
+    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
                        gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, gadd);
     return check_launch();
 }
 
-template <class C>
-static int launch_grad_x_3x3s2(const float *gy, const float *x, const float *w, float *gx,
-                               const ConvDims &d, hipStream_t s, const float *gadd) {
-    // element-wise tile loads when the rows of the staged tensor are not whole float4 groups
+template <class C, class T = float>
+static int launch_grad_x_3x3s2(const T *gy, const T *x, const float *w, T *gx,
+                               const ConvDims &d, hipStream_t s, const T *gadd) {
+    // element-wise tile loads when the rows of the staged tensor are not whole groups of four
     const bool vec = d.Wo % 4 == 0;
     if (d.Co * 4 > kSatMaxTerms)   // an input position meets at most four of the nine taps per output channel
-        return vec ? launch_grad_x_3x3s2_v<C, true, false>(gy, x, w, gx, d, s, gadd)
-                   : launch_grad_x_3x3s2_v<C, false, false>(gy, x, w, gx, d, s, gadd);
-    return vec ? launch_grad_x_3x3s2_v<C, true, true>(gy, x, w, gx, d, s, gadd)
-               : launch_grad_x_3x3s2_v<C, false, true>(gy, x, w, gx, d, s, gadd);
+        return vec ? launch_grad_x_3x3s2_v<C, true, false, T>(gy, x, w, gx, d, s, gadd)
+                   : launch_grad_x_3x3s2_v<C, false, false, T>(gy, x, w, gx, d, s, gadd);
+    return vec ? launch_grad_x_3x3s2_v<C, true, true, T>(gy, x, w, gx, d, s, gadd)
+               : launch_grad_x_3x3s2_v<C, false, true, T>(gy, x, w, gx, d, s, gadd);
 }
 
 //                              TNW BPR TH NIMG TM CIW CC
@@ -748,9 +749,9 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         f.stride = 1;
         const Subsample sub{d.stride, d.Wo, d.W, d.H * d.W};
         if (f.W % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 15) == 0) {
-            if (f.W > 64) return launch_grad_x_3x3s1<Gx1x1, true>(gy, x, w, gx, f, s, nullptr, sub);
-            return small_plane_tile(f) ? launch_grad_x_3x3s1<Gx1x1t, true>(gy, x, w, gx, f, s, nullptr, sub)
-                                       : launch_grad_x_3x3s1<Gx1x1s, true>(gy, x, w, gx, f, s, nullptr, sub);
+            if (f.W > 64) return launch_grad_x_3x3s1<Gx1x1, true>(gy, x, w, gx, f, s, (const float *)nullptr, sub);
+            return small_plane_tile(f) ? launch_grad_x_3x3s1<Gx1x1t, true>(gy, x, w, gx, f, s, (const float *)nullptr, sub)
+                                       : launch_grad_x_3x3s1<Gx1x1s, true>(gy, x, w, gx, f, s, (const float *)nullptr, sub);
         }
     }
     if (conv1x1_supported(d, gy, gx))
@@ -758,6 +759,28 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
     constexpr int TM = 8;
     const long total = (long)d.N * d.H * d.W;
     hipLaunchKernelGGL(grad_x_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Ci, TM)),
+                       dim3(256), 0, s, gy, x, w, gx, d);
+    return check_launch();
+}
+
+// bfloat16 storage: the tiled 3x3 / pad-1 kernels (stride 1 or 2), the generic kernel for everything else
+int launch_grad_x_bf16(const bf16_t *gy, const bf16_t *x, const float *w, bf16_t *gx, const ConvDims &d,
+                       hipStream_t s) {
+    const bf16_t *none = nullptr;
+    if (d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1 && d.Ci >= GxW32::TM &&
+        (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 7) == 0)) {
+        if (d.W > 16) return launch_grad_x_3x3s1<GxW32, false, bf16_t>(gy, x, w, gx, d, s, none);
+        if (d.W > 8) return launch_grad_x_3x3s1<GxW16, false, bf16_t>(gy, x, w, gx, d, s, none);
+        return launch_grad_x_3x3s1<GxW8, false, bf16_t>(gy, x, w, gx, d, s, none);
+    }
+    if (d.kh == 3 && d.kw == 3 && d.stride == 2 && d.pad == 1 && d.W % 2 == 0 && d.Ci >= GxS2W32::TM &&
+        (d.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(gy) & 7) == 0) && (reinterpret_cast<uintptr_t>(gx) & 3) == 0) {
+        if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32, bf16_t>(gy, x, w, gx, d, s, none);
+        return launch_grad_x_3x3s2<GxS2W16, bf16_t>(gy, x, w, gx, d, s, none);
+    }
+    constexpr int TM = 8;
+    const long total = (long)d.N * d.H * d.W;
+    hipLaunchKernelGGL((grad_x_generic_kernel<TM, bf16_t>), dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Ci, TM)),
                        dim3(256), 0, s, gy, x, w, gx, d);
     return check_launch();
 }

@@ -55,8 +55,9 @@ struct TileStage {
 // tensors whose rows are not float4-aligned (W % 4 != 0): element-wise loads.  Index arithmetic is
 // 32-bit: the C ABI refuses tensors of 2^31 elements or more.
 // SUB: src is sampled as described by `sub`; (H, W) = (1, sampled positions per plane).
-template <class P, bool VEC = true, bool SUB = false>
-__device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__restrict__ src,
+// T: the storage type of src (float or bf16_t); the staged values are floats either way.
+template <class P, bool VEC = true, bool SUB = false, class T = float>
+__device__ __forceinline__ void tile_fetch(TileStage<P> &st, const T *__restrict__ src,
                                            int chan0, int nchan, int n0, int nimg_total, int hb,
                                            int wb, int H, int W, const Subsample sub = Subsample{1, 0, 0, 0}) {
     static_assert(!(SUB && VEC), "sampled tensors are read element by element");
@@ -75,25 +76,25 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
         float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok) {
             if constexpr (SUB) {
-                const float *base = src + (size_t)(n * nchan + ch) * sub.plane;
+                const T *base = src + (size_t)(n * nchan + ch) * sub.plane;
                 int ho = wi / sub.wv, wo = wi - ho * sub.wv;
                 float e[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    e[k] = wi + k < W ? base[ho * sub.s * sub.pitch + wo * sub.s] : 0.f;
+                    e[k] = wi + k < W ? ldf(base + ho * sub.s * sub.pitch + wo * sub.s) : 0.f;
                     if (++wo == sub.wv) { wo = 0; ++ho; }
                 }
                 st.v[it] = make_float4(e[0], e[1], e[2], e[3]);
                 continue;
             }
-            const float *row = src + (((n * nchan + ch) * H + hi) * W + wi);
+            const T *row = src + (((n * nchan + ch) * H + hi) * W + wi);
             if constexpr (VEC) {
-                val = *reinterpret_cast<const float4 *>(row);
-            } else {   // rows are not 16-byte aligned (W % 4 != 0): four guarded dword loads
-                val.x = row[0];
-                if (wi + 1 < W) val.y = row[1];
-                if (wi + 2 < W) val.z = row[2];
-                if (wi + 3 < W) val.w = row[3];
+                val = ldf4(row);
+            } else {   // rows are not whole aligned groups of four (W % 4 != 0): four guarded element loads
+                val.x = ldf(row);
+                if (wi + 1 < W) val.y = ldf(row + 1);
+                if (wi + 2 < W) val.z = ldf(row + 2);
+                if (wi + 3 < W) val.w = ldf(row + 3);
             }
         }
         st.v[it] = val;
@@ -109,7 +110,7 @@ __device__ __forceinline__ void tile_fetch(TileStage<P> &st, const float *__rest
         const int n = n0 + img, ch = chan0 + cc, hi = hb + r, wi = side ? wb + P::ICOLS : wb - 1;
         const bool ok = (P::NUH % P::NTHREADS == 0 || u < P::NUH) && n < nimg_total && ch < nchan &&
                         hi >= 0 && hi < H && wi >= 0 && wi < W;
-        st.h[it] = ok ? src[((n * nchan + ch) * H + hi) * W + wi] : 0.f;
+        st.h[it] = ok ? ldf(src + (((n * nchan + ch) * H + hi) * W + wi)) : 0.f;
     }
 }
 

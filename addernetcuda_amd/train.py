@@ -85,22 +85,33 @@ def synthetic_arrays(n, device, classes=10, seed=0):
     return out
 
 
-def evaluate(net, x_u8, y, batch):
+def forward_pass(net, images, bf16=False):
+    """Logits of a batch.  ``bf16``: the optional reduced-storage mode -- the images enter as bfloat16 under
+    torch.autocast, so every activation between the layers is stored as bfloat16 and the adder layers take their
+    bfloat16-storage kernels (float32 weights, float32 / float64 accumulation); the fused BatchNorm kernels are
+    float32 only, so BatchNorm / ReLU then run as torch's own ops."""
+    if not bf16:
+        return net(images)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        return net(images.bfloat16()).float()
+
+
+def evaluate(net, x_u8, y, batch, bf16=False):
     net.eval()
     correct, loss_sum = 0, 0.0
     with torch.no_grad():
         for i in range(0, x_u8.shape[0], batch):
-            logits = net(normalise(x_u8[i:i + batch]))
+            logits = forward_pass(net, normalise(x_u8[i:i + batch]), bf16)
             loss_sum += F.cross_entropy(logits, y[i:i + batch], reduction="sum").item()
             correct += (logits.argmax(1) == y[i:i + batch]).sum().item()
     n = x_u8.shape[0]
     return loss_sum / n, correct / n
 
 
-def train_step(net, opt, images, labels):
+def train_step(net, opt, images, labels, bf16=False):
     from addernetcuda_amd.adder import batched_eta_scaling
     opt.zero_grad(set_to_none=True)
-    loss = F.cross_entropy(net(images), labels)
+    loss = F.cross_entropy(forward_pass(net, images, bf16), labels)
     with batched_eta_scaling():   # the adaptive scaling of all adder layers in two launches
         loss.backward()
     opt.step()
@@ -115,21 +126,21 @@ class GraphedStep:
     frozen into the graph); BatchNorm's running statistics and the optimizer state are updated by the graph's
     own kernels.  All calls must come from the same (non-default) stream."""
 
-    def __init__(self, net, opt, warmup=3):
-        self.net, self.opt, self.warmup = net, opt, warmup
+    def __init__(self, net, opt, warmup=3, bf16=False):
+        self.net, self.opt, self.warmup, self.bf16 = net, opt, warmup, bf16
         self.graph = self.images = self.labels = self.loss = None
         self.calls = 0
 
     def __call__(self, images, labels):
         self.calls += 1
         if self.graph is None and self.calls <= self.warmup:
-            return train_step(self.net, self.opt, images, labels)
+            return train_step(self.net, self.opt, images, labels, self.bf16)
         if self.graph is None:
             self.images, self.labels = images.clone(), labels.clone()
             self.opt.zero_grad(set_to_none=True)
             self.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(self.graph, stream=torch.cuda.current_stream()):
-                self.loss = train_step(self.net, self.opt, self.images, self.labels)
+                self.loss = train_step(self.net, self.opt, self.images, self.labels, self.bf16)
         else:
             self.images.copy_(images)
             self.labels.copy_(labels)
@@ -137,7 +148,7 @@ class GraphedStep:
         return self.loss.clone()
 
 
-def train_one_epoch(net, opt, x_u8, y, batch, generator=None, graphed=None):
+def train_one_epoch(net, opt, x_u8, y, batch, generator=None, graphed=None, bf16=False):
     """``graphed``: a GraphedStep for batches of exactly ``batch`` images (the tail batch runs eagerly)."""
     net.train()
     n = x_u8.shape[0]
@@ -149,7 +160,7 @@ def train_one_epoch(net, opt, x_u8, y, batch, generator=None, graphed=None):
             break
         images = augment(normalise(x_u8[idx]), generator)
         step = graphed if graphed is not None and idx.numel() == batch else None
-        losses.append(step(images, y[idx]) if step else train_step(net, opt, images, y[idx]))
+        losses.append(step(images, y[idx]) if step else train_step(net, opt, images, y[idx], bf16))
     return torch.stack(losses).mean().item()
 
 
@@ -181,12 +192,12 @@ def run(args):
     lr_now = torch.tensor(float(args.lr), device=dev)
     opt = torch.optim.SGD(net.parameters(), lr=lr_now, momentum=0.9, weight_decay=5e-4, fused=True)
     if args.eval_only:   # the reference's test.py: load a checkpoint, one pass over the test split
-        test_loss, acc = evaluate(net, *data["test"], args.test_batch_size)
+        test_loss, acc = evaluate(net, *data["test"], args.test_batch_size, args.bf16_activations)
         print(f"test loss {test_loss:.4f}  accuracy {acc:.4f}", flush=True)
         return [{"epoch": 0, "test_loss": test_loss, "accuracy": acc}]
     os.makedirs(args.output_dir, exist_ok=True)
     gen = torch.Generator(device=dev).manual_seed(args.seed)
-    graphed = None if args.no_graph else GraphedStep(net, opt)
+    graphed = None if args.no_graph else GraphedStep(net, opt, bf16=args.bf16_activations)
     stream = torch.cuda.Stream()   # graph capture needs a stream of its own; the eager steps share it
     best, history = 0.0, []
     for epoch in range(1, args.epochs + 1):
@@ -196,10 +207,10 @@ def run(args):
         t0 = time.time()
         stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(stream):
-            train_loss = train_one_epoch(net, opt, *data["train"], args.batch_size, gen, graphed)
+            train_loss = train_one_epoch(net, opt, *data["train"], args.batch_size, gen, graphed, args.bf16_activations)
         torch.cuda.synchronize()
         dt = time.time() - t0
-        test_loss, acc = evaluate(net, *data["test"], args.test_batch_size)
+        test_loss, acc = evaluate(net, *data["test"], args.test_batch_size, args.bf16_activations)
         history.append({"epoch": epoch, "lr": lr, "train_loss": train_loss, "test_loss": test_loss, "accuracy": acc,
                         "seconds": dt})
         print(f"epoch {epoch}: lr {lr:.5f}  train loss {train_loss:.4f}  test loss {test_loss:.4f}  "
@@ -223,6 +234,9 @@ def parse_args(argv=None):
     p.add_argument("--lr", type=float, default=0.05, help="peak of the cosine schedule (main.py:71: 2 x 0.025)")
     p.add_argument("--eta", type=float, default=0.2, help="adaptive grad_W scale, adder.py:78 uses 1/5")
     p.add_argument("--no-graph", action="store_true", help="run every training step eagerly instead of as a HIP graph")
+    p.add_argument("--bf16-activations", action="store_true",
+                   help="optional mode: activations stored as bfloat16 between the layers (float32 weights, float32 / "
+                        "float64 accumulation in the adder kernels); the default, like the reference, is float32 throughout")
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--arch", choices=ARCHS, default="resnet20", help="network (main.py:66 trains resnet20)")
     return p.parse_args(argv)

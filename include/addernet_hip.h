@@ -113,6 +113,23 @@ ADDER_API int adder_conv2d_bwd_add_f32(const float *gy, const float *x, const fl
                          int N, int Ci, int H, int W, int Co, int kh, int kw,
                          int stride, int pad, void *stream);
 
+/* Optional reduced-storage mode: the activations and their gradients (x, y, gy, gx) are stored as bfloat16 (the
+ * upper half of an fp32, rounded to nearest even on the way out) and take half the HBM traffic and half the
+ * activation memory; weights and weight gradients stay fp32, every sum is accumulated as in the fp32 entry points
+ * (fp32 for y and gx, fp64 for gw).  The reference computes in fp32 only (adder.cu:310-318 hard-codes
+ * data<float>()), so these have no counterpart there and are never the default.  Same dimensions, semantics, eta
+ * and workspace (adder_conv2d_bwd_workspace_bytes) as adder_conv2d_fwd_f32 / adder_conv2d_bwd_f32.  3x3 / pad 1
+ * layers (stride 1 or 2) run on the tiled kernels, everything else on the generic ones. */
+typedef unsigned short adder_bf16;
+ADDER_API int adder_conv2d_fwd_bf16(const adder_bf16 *x, const float *w, adder_bf16 *y,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream);
+ADDER_API int adder_conv2d_bwd_bf16(const adder_bf16 *gy, const adder_bf16 *x, const float *w,
+                         adder_bf16 *gx, float *gw, float eta,
+                         void *ws, size_t ws_bytes,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream);
+
 /* adder_conv2d_bwd_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc) and have no workspace to hand over.  It has no counterpart in
  * the reference, whose backward takes every buffer from torch's allocator (adder.py:66-67).  The partial slabs

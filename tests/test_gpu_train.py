@@ -42,3 +42,14 @@ def test_other_architectures_train(gpu, tmp_path):
     assert max(h["accuracy"] for h in hist) > 0.4          # 0.72 when written
     state = torch.load(os.path.join(str(tmp_path), "addernet.pt"), map_location="cpu", weights_only=True)
     assert "features.2.adder" in state and "classifier.weight" in state
+
+
+def test_bfloat16_activation_mode_trains(gpu, tmp_path):
+    """--bf16-activations: the optional reduced-storage mode through the same loop, eager and captured."""
+    from addernetcuda_amd import train
+    for extra in (["--no-graph"], []):
+        hist = train.run(train.parse_args(["--synthetic", "2000", "--epochs", "5", "--batch-size", "100", "--test-batch-size",
+                                           "50", "--output-dir", str(tmp_path), "--seed", "3", "--bf16-activations"] + extra))
+        assert all(h["train_loss"] == h["train_loss"] for h in hist)
+        assert hist[-1]["train_loss"] < hist[0]["train_loss"]
+        assert max(h["accuracy"] for h in hist) > 0.4
