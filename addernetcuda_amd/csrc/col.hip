@@ -245,6 +245,130 @@ __global__ __launch_bounds__(256) void col_grad_x_reg_kernel(const float *__rest
                 col_load<COLS, VEC>(gX + (size_t)(k0 + kk) * NL, c0, NL));
 }
 
+// ---------------------------------------------------------------------------
+// ADDER_BACKWARD in one pass over X for layers with at most 16 output channels: the kernel above with the
+// weight gradient folded in, so that X (the largest tensor by far: K rows against the Co rows of gy) crosses
+// HBM once for both gradients.
+//   gX: as above, lane = 2 adjacent columns, gy of those columns in registers, two instructions per term.
+//   gW: per wave and batch of 16 rows of X, the 16 x 16 block  sum_cols gy[co, col] * X[k, col]  over the wave's
+//       128 columns on v_mfma_f64_16x16x4_f64 (32 steps of 4 columns).  The MFMA wants lane l to hold row l % 16
+//       at column 4 * step + l / 16, the streaming layout has lane l hold all rows at columns 2l, 2l + 1: gy is
+//       transposed through LDS once per kernel (its fragments then stay in registers as doubles), every batch of
+//       X once per batch.  The four waves' blocks are added through LDS and go to this workgroup's fp64 slab
+//       (one slab per 512 columns); grad_w.hip's slab finalize adds the slabs and applies - W * sum gy.
+// blockIdx.y selects a block of KB rows (KB a multiple of 16).
+// ---------------------------------------------------------------------------
+static constexpr int kFusedPitch = 132;   // floats per staged row of 128 columns (+4: the 16 rows land in different banks)
+
+__global__ __launch_bounds__(256) void col_bwd_fused_kernel(const float *__restrict__ gy, const float *__restrict__ X,
+                                                            const float *__restrict__ Wm, float *__restrict__ gX,
+                                                            double *__restrict__ part, double *__restrict__ sgpart,
+                                                            int K, long NL, int Co, int KB) {
+    constexpr int COB = 16, PF = 8;
+    extern __shared__ __align__(16) float smem[];
+    float *wt = smem;                                          // [KB][16] transposed weights of this row block
+    float *stage = smem + KB * COB;                            // [4 waves][16][kFusedPitch]: gy once, then batches of X
+    double *cred = reinterpret_cast<double *>(stage + 4 * 16 * kFusedPitch);   // [4 waves][256] blocks to fold
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l16 = lane & 15, lk = lane >> 4;
+    const int k0 = blockIdx.y * KB, kcnt = min(KB, K - k0);
+    for (int i = threadIdx.x; i < kcnt * COB; i += 256) {
+        const int co = i / kcnt, kk = i - co * kcnt;
+        wt[kk * COB + co] = co < Co ? Wm[(size_t)co * K + k0 + kk] : 0.f;
+    }
+    long c0 = ((long)blockIdx.x * 256 + threadIdx.x) * 2;
+    const bool active = c0 < NL;
+    if (!active) c0 = NL - 2;
+    float g[COB][2], s2[2] = {0.f, 0.f};
+    float *mine = stage + wave * 16 * kFusedPitch;
+#pragma unroll
+    for (int co = 0; co < COB; ++co) {
+        float2 t = make_float2(0.f, 0.f);
+        if (co < Co && active) t = *reinterpret_cast<const float2 *>(gy + (size_t)co * NL + c0);   // idle lanes: gy = 0
+        g[co][0] = t.x; g[co][1] = t.y;
+        s2[0] += t.x; s2[1] += t.y;
+        *reinterpret_cast<float2 *>(mine + co * kFusedPitch + 2 * lane) = t;
+    }
+    __syncthreads();
+    double ga[32], sgt = 0.0;   // the wave's gy as MFMA A fragments: row l16, column 4 * step + lk
+#pragma unroll
+    for (int st = 0; st < 32; ++st) {
+        ga[st] = (double)mine[l16 * kFusedPitch + 4 * st + lk];
+        sgt += ga[st];
+    }
+    sgt += __shfl_xor(sgt, 16, 64);
+    sgt += __shfl_xor(sgt, 32, 64);
+    __syncthreads();   // the staging area now takes batches of X
+
+    auto one_row = [&](const int kk, const float2 xv, const float2 old) {
+        const float c0v = fmaf(-0.5f, xv.x, 0.5f), c1v = fmaf(-0.5f, xv.y, 0.5f);
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int q = 0; q < COB / 4; ++q) {
+            const float4 w4 = *reinterpret_cast<const float4 *>(wt + kk * COB + 4 * q);
+            const float wv[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                a0 = fmaf(sat01(fmaf(wv[j], 0.5f, c0v)), g[4 * q + j][0], a0);
+                a1 = fmaf(sat01(fmaf(wv[j], 0.5f, c1v)), g[4 * q + j][1], a1);
+            }
+        }
+        if (active)
+            *reinterpret_cast<float2 *>(gX + (size_t)(k0 + kk) * NL + c0) =
+                make_float2(old.x + fmaf(2.f, a0, -s2[0]), old.y + fmaf(2.f, a1, -s2[1]));
+        *reinterpret_cast<float2 *>(mine + (kk & 15) * kFusedPitch + 2 * lane) = xv;   // for the weight gradient
+    };
+    auto ld2 = [&](const float *base, int kk) {
+        return *reinterpret_cast<const float2 *>(base + (size_t)(k0 + min(kk, kcnt - 1)) * NL + c0);
+    };
+
+    float2 nx[PF], no[PF];
+#pragma unroll
+    for (int r = 0; r < PF; ++r) { nx[r] = ld2(X, r); no[r] = ld2(gX, r); }
+    const int nbatches = ceil_div(kcnt, 16);
+    for (int b = 0; b < nbatches; ++b) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float2 cx[PF], co_[PF];
+#pragma unroll
+            for (int r = 0; r < PF; ++r) { cx[r] = nx[r]; co_[r] = no[r]; }
+            const int kb = b * 16 + h * PF;
+#pragma unroll
+            for (int r = 0; r < PF; ++r) { nx[r] = ld2(X, kb + PF + r); no[r] = ld2(gX, kb + PF + r); }
+#pragma unroll
+            for (int r = 0; r < PF; ++r) {
+                if (kb + r < kcnt) one_row(kb + r, cx[r], co_[r]);
+                else *reinterpret_cast<float2 *>(mine + ((kb + r) & 15) * kFusedPitch + 2 * lane) = make_float2(0.f, 0.f);
+            }
+        }
+        __syncthreads();
+        double4v acc = double4v{0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int st = 0; st < 32; ++st) {
+            const double xb = (double)mine[l16 * kFusedPitch + 4 * st + lk];
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64(ga[st], xb, acc, 0, 0, 0);
+        }
+        // C layout: lane l, register e -> gy row 4 e + l / 16, X row l % 16
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cred[wave * 256 + (4 * e + lk) * 16 + l16] = acc[e];
+        __syncthreads();
+        {
+            const int co = threadIdx.x >> 4, kk = b * 16 + (threadIdx.x & 15);
+            const double v = (cred[threadIdx.x] + cred[256 + threadIdx.x]) + (cred[512 + threadIdx.x] + cred[768 + threadIdx.x]);
+            if (co < Co && kk < kcnt) part[(size_t)blockIdx.x * Co * K + (size_t)co * K + k0 + kk] = v;
+        }
+        // (the next batch's writes to the staging area and to cred come after the next barrier pair's first half:
+        // every wave passes the barrier above only after all reads of this batch's staging data)
+    }
+    if (blockIdx.y == 0) {
+        __syncthreads();
+        if (lane < 16) cred[wave * 16 + lane] = sgt;
+        __syncthreads();
+        if (threadIdx.x < 16 && threadIdx.x < Co)
+            sgpart[(size_t)blockIdx.x * Co + threadIdx.x] =
+                (cred[threadIdx.x] + cred[16 + threadIdx.x]) + (cred[32 + threadIdx.x] + cred[48 + threadIdx.x]);
+    }
+}
+
 // gX[k, nl] += sum_co hardtanh(W[co,k] - X[k,nl]) * gy[co,nl], any number of output channels: lane = column,
 // TK rows of X per lane in registers, gy streamed per output channel.
 template <int TK>
@@ -524,10 +648,36 @@ static ColGwPlan plan_col_grad_w(int K, long NL, int Co) {
     return p;
 }
 
+// the fused backward serves layers with up to 16 output channels on matrices with many columns (one slab per 512)
+static bool col_bwd_fused_applies(int K, long NL, int Co) { return Co <= 16 && NL % 2 == 0 && NL >= 65536 && K >= 16; }
+static int col_bwd_fused_slots(long NL) { return (int)ceil_div_l(NL, 512); }
+
 size_t col_grad_w_workspace_bytes(int K, long NL, int Co) {
     const ColGwPlan p = plan_col_grad_w(K, NL, Co);
-    if (!p.mfma) return 0;
-    return (sizeof(double) * (size_t)p.slots * ((size_t)Co * K + Co) + 255) & ~(size_t)255;
+    int slots = p.mfma ? p.slots : 0;
+    if (col_bwd_fused_applies(K, NL, Co) && col_bwd_fused_slots(NL) > slots) slots = col_bwd_fused_slots(NL);
+    if (!slots) return 0;
+    return (sizeof(double) * (size_t)slots * ((size_t)Co * K + Co) + 255) & ~(size_t)255;
+}
+
+// Both gradients in one pass over X (col_bwd_fused_kernel); ADDER_ERR_UNSUPPORTED (nothing launched) where it does
+// not apply, and the caller runs the two separate kernels.
+int launch_col_bwd_fused(const float *gy, const float *X, const float *Wm, float *gW, float *gX, int K, long NL, int Co,
+                         void *ws, hipStream_t s) {
+    if (!col_bwd_fused_applies(K, NL, Co) || !ws || !aligned8(X) || !aligned8(gy) || !aligned8(gX) ||
+        (reinterpret_cast<uintptr_t>(ws) & 255))
+        return ADDER_ERR_UNSUPPORTED;
+    const int slots = col_bwd_fused_slots(NL);
+    int KB = round_up(K, 16);
+    if (KB > 256) KB = 256;
+    const int lds = KB * 16 * 4 + 4 * 16 * kFusedPitch * 4 + 4 * 256 * 8;
+    if (int rc = allow_dynamic_lds<&col_bwd_fused_kernel>(lds)) return rc;
+    double *part = reinterpret_cast<double *>(ws);
+    double *sgpart = part + (size_t)slots * Co * K;
+    hipLaunchKernelGGL(col_bwd_fused_kernel, dim3(slots, ceil_div(K, KB)), dim3(256), lds, s, gy, X, Wm, gX, part, sgpart,
+                       K, NL, Co, KB);
+    if (int rc = check_launch()) return rc;
+    return launch_grad_w_slab_finalize(part, sgpart, Wm, gW, slots, Co, K, /*accumulate=*/true, s);
 }
 
 template <int CT, int KT>

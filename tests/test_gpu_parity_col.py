@@ -45,7 +45,8 @@ def test_adder_backward_and_its_two_halves(case, gpu):
     gw2, gx2 = torch.zeros_like(Wg), torch.zeros_like(Xg)
     adder_cuda.ADDER_CONV_WEIGHT(Gg, Xg, Wg, gw2)
     adder_cuda.ADDER_CONV_INPUT(Gg, Xg, Wg, gx2)
-    assert torch.equal(gw2, gw) and torch.equal(gx2, gx)
+    # (ADDER_BACKWARD may take both gradients in one pass over X: the same sums in another order for grad_w)
+    assert torch.equal(gx2, gx) and torch.allclose(gw2, gw, rtol=1e-6, atol=1e-6)
 
 
 def test_gradients_accumulate_into_their_outputs(gpu):
