@@ -51,6 +51,10 @@ _SIGNATURES = {
     "adder_bn_act_fwd_f32": (_i, [_p] * 11 + [_f, _f, _i, _i, _i, _i, _p, _sz, _p]),
     "adder_bn_act_fwd_stats_f32": (_i, [_p] * 11 + [_f, _f, _i, _i, _i, _i, _p, _i, _p]),
     "adder_bn_act_bwd_f32": (_i, [_p] * 11 + [_i, _i, _i, _i, _p, _sz, _p]),
+    "adder_conv2d_bwd_bn_slots": (_i, [_i] * 9 + [ctypes.POINTER(ctypes.c_int)]),
+    "adder_conv2d_bwd_bn_f32": (_i, [_p, _p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p, _p]),
+    "adder_conv2d_grad_w_staged_bn_f32": (_i, [_p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p, _p, _p]),
+    "adder_bn_bwd_coef_f32": (_i, [_p, _i, _p, _p, _p, ctypes.c_double, _p, _p, _p, _i, _p]),
 }
 for _name, (_res, _args) in _SIGNATURES.items():
     _fn = getattr(lib, _name)
@@ -64,6 +68,14 @@ class GradWStage(ctypes.Structure):
     _fields_ = [("part", ctypes.c_void_p), ("sgpart", ctypes.c_void_p), ("w", ctypes.c_void_p),
                 ("gw", ctypes.c_void_p), ("slots", ctypes.c_int), ("Co", ctypes.c_int), ("K", ctypes.c_int),
                 ("fp64", ctypes.c_int), ("eta", ctypes.c_float)]
+
+
+class BnLinks(ctypes.Structure):
+    """adder_bn_links of include/addernet_hip.h."""
+    _fields_ = [("out_x", ctypes.c_void_p), ("out_coef", ctypes.c_void_p), ("out_gy", ctypes.c_void_p),
+                ("in_x", ctypes.c_void_p),
+                ("in_mean", ctypes.c_void_p), ("in_rstd", ctypes.c_void_p), ("in_part", ctypes.c_void_p),
+                ("in_slots", ctypes.c_int), ("in_relu", ctypes.c_int)]
 
 
 def check(status, what):
@@ -191,3 +203,11 @@ def bn_act_sizes(N, C, HW):
     check(lib.adder_bn_act_workspace_bytes(N, C, HW, ctypes.byref(need)), "adder_bn_act_workspace_bytes")
     check(lib.adder_bn_act_mask_words(N, C, HW, ctypes.byref(words)), "adder_bn_act_mask_words")
     return need.value, words.value
+
+
+@functools.lru_cache(maxsize=4096)
+def bwd_bn_slots(dims):
+    """Partial-sum slots of the backward kernels that take BatchNorm links for this geometry (0: none do)."""
+    slots = ctypes.c_int(0)
+    check(lib.adder_conv2d_bwd_bn_slots(*dims, ctypes.byref(slots)), "adder_conv2d_bwd_bn_slots")
+    return slots.value

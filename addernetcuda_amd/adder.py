@@ -19,7 +19,7 @@ from torch.autograd import Function
 
 from . import adder_cuda
 from ._lib import (lib, check, ptr, require_gpu_f32, require_gpu_bf16, same_device, stream_ptr, conv_dims,
-                   conv2d_bwd_workspace, fwd_stats_slots, on_device, GradWStage)
+                   conv2d_bwd_workspace, fwd_stats_slots, on_device, GradWStage, BnLinks, bwd_bn_slots)
 
 DEFAULT_ETA = 0.2  # adder.py:78 divides by 5
 
@@ -134,6 +134,164 @@ class batched_eta_scaling:
         return False
 
 
+def conv_forward(X, W, stride, padding, with_stats):
+    """The forward launch shared by the autograd nodes: (out, stats or None, dims) for contiguous float32 GPU
+    tensors.  ``stats`` are the per-channel partial sums of out and out**2 for the BatchNorm that follows
+    (bn_act.py), where ``with_stats`` is set and the layer's kernel has that epilogue."""
+    require_gpu_f32(X, "X")
+    require_gpu_f32(W, "W")
+    dev = same_device(X, W)
+    dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
+    out = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
+    stats = None
+    with on_device(dev):
+        slots = fwd_stats_slots(dims) if with_stats else 0
+        if slots > 0:
+            stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64)
+            status = lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots, *dims, stream_ptr(dev))
+            if status == -7:   # e.g. tensors that are not 16-byte aligned: the kernel that sums was turned down
+                stats, slots = None, 0
+            else:
+                check(status, "adder_conv2d_fwd_stats_f32")
+        if slots <= 0:
+            check(lib.adder_conv2d_fwd_f32(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_f32")
+    return out, stats, dims
+
+
+class BnLink:
+    """What passes between the backward of a layer and the BatchNorm on either side of it when the BatchNorm's
+    backward is folded into the layer's kernels (``adder_bn_links`` of the C ABI; unit.py drives it).
+
+    Made in the forward of the BatchNorm's node, which records the BatchNorm's input, statistics and weight; the
+    layer that consumes the BatchNorm's output keeps a reference.  In the backward pass the consumer runs first:
+    its input-gradient kernel leaves ``dz`` (the gradient of the BatchNorm's output before the ReLU) as its result
+    and the partial sums of the BatchNorm's backward, a small kernel turns those into ``coef`` / ``dgamma`` /
+    ``dbeta``, and the node of the BatchNorm, when it is handed exactly that ``dz`` tensor, skips its own two
+    passes."""
+    __slots__ = ("bn_x", "mean", "rstd", "gamma", "relu", "out_ptr", "out_shape", "out_version", "dz", "dz_version",
+                 "coef", "dgamma", "dbeta")
+
+    def __init__(self, bn_x, mean, rstd, gamma, relu):
+        self.bn_x, self.mean, self.rstd, self.gamma, self.relu = bn_x, mean, rstd, gamma, relu
+        self.out_ptr = self.out_shape = self.out_version = None
+        self.dz = self.dz_version = self.coef = self.dgamma = self.dbeta = None
+
+    def attach(self, out):
+        """Tie the link to the tensor that left the BatchNorm's node; consumers find it as ``out._adder_bn_link``."""
+        self.out_ptr, self.out_shape, self.out_version = out.data_ptr(), tuple(out.shape), out._version
+        out._adder_bn_link = self
+
+    @staticmethod
+    def of(x):
+        """The link of the node that produced ``x``, if ``x`` still is what that node returned."""
+        link = getattr(x, "_adder_bn_link", None)
+        if (link is None or link.out_ptr != x.data_ptr() or link.out_shape != tuple(x.shape)
+                or link.out_version != x._version or not x.is_contiguous()):
+            return None
+        return link
+
+    def claims(self, dy):
+        """Whether ``dy`` is the very tensor the consumer's kernel wrote (not a sum autograd formed from it)."""
+        dz = self.dz
+        return (dz is not None and dy.data_ptr() == dz.data_ptr() and dy.shape == dz.shape
+                and dy._version == self.dz_version and dy.is_contiguous())
+
+
+def _aligned16(*tensors):
+    return all(t is None or t.data_ptr() % 16 == 0 for t in tensors)
+
+
+def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_given, out_link=None, in_link=None):
+    """The backward launches shared by the autograd nodes: (grad_X, grad_W), either None where not needed.
+
+    ``grad_short``: a second gradient of X (a residual shortcut), added to grad_X by the kernel where it can.
+    ``out_link``: a BnLink whose ``coef`` is ready -- ``grad_out`` is then dz of the BatchNorm behind the layer
+    (the caller has checked ``bwd_bn_slots(dims)``, the alignment of the tensors and ``need_w``).
+    ``in_link``: the BnLink of the BatchNorm whose output X is -- grad_X leaves as dz, and the link receives dz,
+    coef, dgamma and dbeta (same checks by the caller, and ``need_x``)."""
+    dev = X.device
+    gx = torch.empty_like(X) if need_x else None
+    gw = torch.empty_like(W) if need_w else None
+    eta = float(eta or 0.0)
+    links = None
+    part = slots = None
+    if out_link is not None or in_link is not None:
+        links = BnLinks()
+        if out_link is not None:
+            gy_formed = torch.empty_like(grad_out)
+            links.out_x, links.out_coef, links.out_gy = ptr(out_link.bn_x), ptr(out_link.coef), ptr(gy_formed)
+        if in_link is not None:
+            slots = bwd_bn_slots(dims)
+            part = torch.empty((X.size(1), slots, 2), device=dev, dtype=torch.float64)
+            links.in_x, links.in_mean, links.in_rstd = ptr(in_link.bn_x), ptr(in_link.mean), ptr(in_link.rstd)
+            links.in_part, links.in_slots, links.in_relu = ptr(part), slots, int(in_link.relu)
+    if _eta_batch is not None and need_w and any(W is entry[0] for entry in _eta_batch):
+        raise RuntimeError("batched_eta_scaling: this weight already has a pending gradient in the block "
+                           "(one backward pass per block, no weight shared between layers)")
+    staged = False
+    if (_eta_batch is not None and need_w and w_is_given and W.is_leaf and W.grad is None):
+        with on_device(dev):
+            ws, nbytes = conv2d_bwd_workspace(dims, dev)
+            stage = GradWStage()
+            if out_link is not None:
+                status = lib.adder_conv2d_grad_w_staged_bn_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gw), eta, ptr(ws), nbytes,
+                                                               *dims, ctypes.byref(links), ctypes.byref(stage),
+                                                               stream_ptr(dev))
+            else:
+                status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gw), eta, ptr(ws), nbytes,
+                                                            *dims, ctypes.byref(stage), stream_ptr(dev))
+        if status == 0:      # slabs only; finished with all the others when the block ends
+            _eta_batch.append((W, eta, stage, ws))
+            staged = True
+        elif status != -7 or out_link is not None:
+            check(status, "adder_conv2d_grad_w_staged_f32")
+        elif eta > 0.0:      # no slab kernel for this layer: raw gradient now, scaled when the block ends
+            _eta_batch.append((W, eta, None, None))
+            eta = 0.0
+    gw_out = gw
+    if staged:
+        gw = None
+        if out_link is not None:   # the staged kernel has formed the gradient of the layer's output
+            grad_out = gy_formed
+            links.out_x = links.out_coef = links.out_gy = None
+    if need_x or gw is not None:
+        with on_device(dev):
+            ws, nbytes = conv2d_bwd_workspace(dims, dev) if gw is not None else (None, 0)
+            if links is not None and (in_link is not None or links.out_x):
+                check(lib.adder_conv2d_bwd_bn_f32(ptr(grad_out), ptr(X), ptr(W), ptr(grad_short), ptr(gx), ptr(gw), eta,
+                                                  ptr(ws), nbytes, *dims, ctypes.byref(links), stream_ptr(dev)),
+                      "adder_conv2d_bwd_bn_f32")
+            else:
+                fused = False
+                if need_x and grad_short is not None:
+                    status = lib.adder_conv2d_bwd_add_f32(ptr(grad_out), ptr(X), ptr(W), ptr(grad_short), ptr(gx),
+                                                          ptr(gw), eta, ptr(ws), nbytes, *dims, stream_ptr(dev))
+                    fused = status == 0
+                    if status not in (0, -7):   # -7: this layer's grad_X kernel has no fused add
+                        check(status, "adder_conv2d_bwd_add_f32")
+                if not fused:
+                    check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw), eta, ptr(ws), nbytes,
+                                                   *dims, stream_ptr(dev)), "adder_conv2d_bwd_f32")
+                    if need_x and grad_short is not None:
+                        gx += grad_short
+            if in_link is not None:
+                C = X.size(1)
+                in_link.coef = torch.empty((C, 4), device=dev, dtype=torch.float32)
+                in_link.dgamma = torch.empty(C, device=dev, dtype=torch.float32)
+                in_link.dbeta = torch.empty(C, device=dev, dtype=torch.float32)
+                count = float(X.numel() // C)
+                check(lib.adder_bn_bwd_coef_f32(ptr(part), slots, ptr(in_link.gamma), ptr(in_link.mean), ptr(in_link.rstd),
+                                                count, ptr(in_link.coef), ptr(in_link.dgamma), ptr(in_link.dbeta), C,
+                                                stream_ptr(dev)), "adder_bn_bwd_coef_f32")
+                in_link.dz, in_link.dz_version = gx, gx._version
+    return gx, gw_out
+
+
+def bn_links_usable(dims, *tensors):
+    """Whether the layer has the backward kernels that take BatchNorm links and the tensors suit them."""
+    return bwd_bn_slots(dims) > 0 and _aligned16(*tensors)
+
+
 class _adder_nchw(Function):
     """Fused NCHW forward / backward (replaces adder.py:22-41 + 43-80 in one step each)."""
 
@@ -141,25 +299,8 @@ class _adder_nchw(Function):
     def forward(ctx, X, W, stride, padding, eta, with_stats=False, with_shortcut=False):
         ctx.w_is_given = W.is_contiguous()   # then the saved W is the caller's own tensor (its .grad is visible)
         X, W = X.contiguous(), W.contiguous()
-        require_gpu_f32(X, "X")
-        require_gpu_f32(W, "W")
-        dev = same_device(X, W)
-        dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
-        out = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
-        stats = None
-        with on_device(dev):
-            slots = fwd_stats_slots(dims) if with_stats else 0
-            if slots > 0:
-                # partial sums of out and out**2 per channel for the BatchNorm that follows (bn_act.py)
-                stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64)
-                status = lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots, *dims,
-                                                        stream_ptr(dev))
-                if status == -7:   # e.g. tensors that are not 16-byte aligned: the kernel that sums was turned down
-                    stats, slots = None, 0
-                else:
-                    check(status, "adder_conv2d_fwd_stats_f32")
-            if slots <= 0:
-                check(lib.adder_conv2d_fwd_f32(ptr(X), ptr(W), ptr(out), *dims, stream_ptr(dev)), "adder_conv2d_fwd_f32")
+        out, stats, dims = conv_forward(X, W, stride, padding, with_stats)
+        dev = X.device
         ctx.save_for_backward(X, W)  # the NCHW input, not the 9x larger X_col the reference keeps
         ctx.dims, ctx.eta = dims, eta
         if not with_stats and not with_shortcut:
@@ -186,48 +327,11 @@ class _adder_nchw(Function):
         X, W = ctx.saved_tensors
         grad_out = grad_out.contiguous()
         require_gpu_f32(grad_out, "grad_output")
-        dev = X.device
-        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        gx = torch.empty_like(X) if need_x else None
-        gw = torch.empty_like(W) if need_w else None
-        eta = float(ctx.eta or 0.0)
-        if _eta_batch is not None and need_w and any(W is entry[0] for entry in _eta_batch):
-            raise RuntimeError("batched_eta_scaling: this weight already has a pending gradient in the block "
-                               "(one backward pass per block, no weight shared between layers)")
-        if (_eta_batch is not None and need_w and ctx.w_is_given and W.is_leaf and W.grad is None):
-            with on_device(dev):
-                ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev)
-                stage = GradWStage()
-                status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gw), eta, ptr(ws), nbytes,
-                                                            *ctx.dims, ctypes.byref(stage), stream_ptr(dev))
-            if status == 0:      # slabs only; finished with all the others when the block ends
-                _eta_batch.append((W, eta, stage, ws))
-                need_w = False
-            elif status != -7:
-                check(status, "adder_conv2d_grad_w_staged_f32")
-            elif eta > 0.0:      # no slab kernel for this layer: raw gradient now, scaled when the block ends
-                _eta_batch.append((W, eta, None, None))
-                eta = 0.0
-        gw_out = gw
-        if not need_w:
-            gw = None
-        if need_x or need_w:
-            with on_device(dev):
-                ws, nbytes = conv2d_bwd_workspace(ctx.dims, dev) if need_w else (None, 0)
-                fused = False
-                if need_x and grad_short is not None:
-                    grad_short = grad_short.contiguous()
-                    status = lib.adder_conv2d_bwd_add_f32(ptr(grad_out), ptr(X), ptr(W), ptr(grad_short), ptr(gx),
-                                                          ptr(gw), eta, ptr(ws), nbytes, *ctx.dims, stream_ptr(dev))
-                    fused = status == 0
-                    if status not in (0, -7):   # -7: this layer's grad_X kernel has no fused add
-                        check(status, "adder_conv2d_bwd_add_f32")
-                if not fused:
-                    check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw), eta, ptr(ws), nbytes,
-                                                   *ctx.dims, stream_ptr(dev)), "adder_conv2d_bwd_f32")
-                    if need_x and grad_short is not None:
-                        gx += grad_short
-        return gx, gw_out, None, None, None, None, None
+        if grad_short is not None:
+            grad_short = grad_short.contiguous()
+        gx, gw = conv_backward(X, W, grad_out, grad_short, ctx.dims, ctx.eta, ctx.needs_input_grad[0],
+                               ctx.needs_input_grad[1], ctx.w_is_given)
+        return gx, gw, None, None, None, None, None
 
 
 class _adder_nchw_bf16(Function):

@@ -20,6 +20,58 @@ def _workspace(N, C, HW, device):
     return torch.empty(max(need, 256), dtype=torch.uint8, device=device), need
 
 
+def bn_forward(x, weight, bias, residual, running_mean, running_var, num_batches, momentum, eps, relu, stats=None):
+    """The forward launches shared by the autograd nodes: (y, mean, rstd, mask) for contiguous float32 GPU
+    tensors; ``mask`` is the ReLU sign mask (None where the kernels have none for this shape)."""
+    N, C = x.shape[0], x.shape[1]
+    HW = x.numel() // (N * C)
+    dev = x.device
+    y = torch.empty_like(x)
+    mean = torch.empty(C, dtype=torch.float32, device=dev)
+    rstd = torch.empty(C, dtype=torch.float32, device=dev)
+    # the backward needs y only for its sign: one bit per element where the kernels offer it
+    mask = None
+    if relu and all(t is None or t.data_ptr() % 16 == 0 for t in (x, y, residual)):
+        words = bn_act_sizes(N, C, HW)[1]
+        if words:
+            mask = torch.empty(words, dtype=torch.int32, device=dev)
+    with on_device(dev):
+        if stats is not None:
+            # the layer that produced x already summed x and x*x per channel (adder.forward_with_stats)
+            if stats.dtype != torch.float64 or stats.dim() != 3 or stats.shape[0] != C or stats.shape[2] != 2 \
+                    or not stats.is_contiguous() or stats.device != dev:
+                raise RuntimeError("stats must be a contiguous float64 tensor (C, slots, 2) on the device of x")
+            check(lib.adder_bn_act_fwd_stats_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mask),
+                                                 ptr(mean), ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
+                                                 float(momentum), float(eps), int(relu), N, C, HW, ptr(stats),
+                                                 int(stats.shape[1]), stream_ptr(dev)), "adder_bn_act_fwd_stats_f32")
+        else:
+            ws, nbytes = _workspace(N, C, HW, dev)
+            check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mask),
+                                           ptr(mean), ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
+                                           float(momentum), float(eps), int(relu), N, C, HW, ptr(ws), nbytes,
+                                           stream_ptr(dev)), "adder_bn_act_fwd_f32")
+    return y, mean, rstd, mask
+
+
+def bn_backward(dy, y, mask, x, weight, mean, rstd, relu, has_res):
+    """The two backward passes: (dx, dres or None, dgamma, dbeta); ``y`` is only read where there is no ``mask``."""
+    N, C = x.shape[0], x.shape[1]
+    HW = x.numel() // (N * C)
+    dev = x.device
+    dx = torch.empty_like(x)
+    dres = torch.empty_like(x) if has_res else None
+    dgamma, dbeta = torch.empty_like(weight), torch.empty_like(weight)
+    if mask is not None and dy.data_ptr() % 16:
+        dy = dy.clone()   # the masked kernels move float4 groups
+    with on_device(dev):
+        ws, nbytes = _workspace(N, C, HW, dev)
+        check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(mask), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
+                                       ptr(dres), ptr(dgamma), ptr(dbeta), int(relu), N, C, HW, ptr(ws), nbytes,
+                                       stream_ptr(dev)), "adder_bn_act_bwd_f32")
+    return dx, dres, dgamma, dbeta
+
+
 class _bn_act(Function):
     @staticmethod
     def forward(ctx, x, weight, bias, residual, running_mean, running_var, num_batches, momentum, eps, relu,
@@ -27,54 +79,16 @@ class _bn_act(Function):
         x = x.contiguous()
         if residual is not None:
             residual = residual.contiguous()
-        N, C = x.shape[0], x.shape[1]
-        HW = x.numel() // (N * C)
-        dev = x.device
-        y = torch.empty_like(x)
-        mean = torch.empty(C, dtype=torch.float32, device=dev)
-        rstd = torch.empty(C, dtype=torch.float32, device=dev)
-        # the backward needs y only for its sign: one bit per element where the kernels offer it
-        mask = None
-        if relu and all(t is None or t.data_ptr() % 16 == 0 for t in (x, y, residual)):
-            words = bn_act_sizes(N, C, HW)[1]
-            if words:
-                mask = torch.empty(words, dtype=torch.int32, device=dev)
-        with on_device(dev):
-            if stats is not None:
-                # the layer that produced x already summed x and x*x per channel (adder.forward_with_stats)
-                if stats.dtype != torch.float64 or stats.dim() != 3 or stats.shape[0] != C or stats.shape[2] != 2 \
-                        or not stats.is_contiguous() or stats.device != dev:
-                    raise RuntimeError("stats must be a contiguous float64 tensor (C, slots, 2) on the device of x")
-                check(lib.adder_bn_act_fwd_stats_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mask),
-                                                     ptr(mean), ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
-                                                     float(momentum), float(eps), int(relu), N, C, HW, ptr(stats),
-                                                     int(stats.shape[1]), stream_ptr(dev)), "adder_bn_act_fwd_stats_f32")
-            else:
-                ws, nbytes = _workspace(N, C, HW, dev)
-                check(lib.adder_bn_act_fwd_f32(ptr(x), ptr(residual), ptr(weight), ptr(bias), ptr(y), ptr(mask),
-                                               ptr(mean), ptr(rstd), ptr(running_mean), ptr(running_var), ptr(num_batches),
-                                               float(momentum), float(eps), int(relu), N, C, HW, ptr(ws), nbytes,
-                                               stream_ptr(dev)), "adder_bn_act_fwd_f32")
+        y, mean, rstd, mask = bn_forward(x, weight, bias, residual, running_mean, running_var, num_batches, momentum,
+                                         eps, relu, stats)
         ctx.save_for_backward(x, y if relu and mask is None else None, weight, mean, rstd, mask)
-        ctx.relu, ctx.has_res, ctx.dims = relu, residual is not None, (N, C, HW)
+        ctx.relu, ctx.has_res = relu, residual is not None
         return y
 
     @staticmethod
     def backward(ctx, dy):
         x, y, weight, mean, rstd, mask = ctx.saved_tensors
-        dy = dy.contiguous()
-        N, C, HW = ctx.dims
-        dev = x.device
-        dx = torch.empty_like(x)
-        dres = torch.empty_like(x) if ctx.has_res else None
-        dgamma, dbeta = torch.empty_like(weight), torch.empty_like(weight)
-        if mask is not None and dy.data_ptr() % 16:
-            dy = dy.clone()   # the masked kernels move float4 groups
-        with on_device(dev):
-            ws, nbytes = _workspace(N, C, HW, dev)
-            check(lib.adder_bn_act_bwd_f32(ptr(dy), ptr(y), ptr(mask), ptr(x), ptr(weight), ptr(mean), ptr(rstd), ptr(dx),
-                                           ptr(dres), ptr(dgamma), ptr(dbeta), int(ctx.relu), N, C, HW, ptr(ws), nbytes,
-                                           stream_ptr(dev)), "adder_bn_act_bwd_f32")
+        dx, dres, dgamma, dbeta = bn_backward(dy.contiguous(), y, mask, x, weight, mean, rstd, ctx.relu, ctx.has_res)
         return dx, dgamma, dbeta, dres, None, None, None, None, None, None, None
 
 

@@ -86,7 +86,7 @@ const char *adder_strerror(int status) {
 
 const char *adder_last_hip_error(void) { return g_last_hip_error.c_str(); }
 
-int adder_abi_version(void) { return 3; }
+int adder_abi_version(void) { return 4; }
 
 int adder_out_dim(int h, int k, int pad, int stride) {
     if (h <= 0 || k <= 0 || pad < 0 || stride <= 0 || h + 2 * pad < k) return 0;
@@ -350,7 +350,17 @@ int adder_grad_norm_scale_f32(float *g, long n, float eta, float eps, void *ws, 
 int adder_conv2d_grad_w_staged_f32(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
                                    size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
                                    int pad, adder_grad_w_stage *stage, void *stream) {
+    return adder_conv2d_grad_w_staged_bn_f32(gy, x, w, gw, eta, ws, ws_bytes, N, Ci, H, W, Co, kh, kw, stride, pad,
+                                             nullptr, stage, stream);
+}
+
+int adder_conv2d_grad_w_staged_bn_f32(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
+                                      size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
+                                      int pad, const adder_bn_links *links, adder_grad_w_stage *stage, void *stream) {
     if (!gy || !x || !gw || !stage) return ADDER_ERR_NULL_POINTER;
+    const float *bn_y = links ? links->out_x : nullptr, *bn_coef = links ? links->out_coef : nullptr;
+    float *gy_out = links ? links->out_gy : nullptr;
+    if ((bn_y == nullptr) != (bn_coef == nullptr) || (gy_out && !bn_y)) return ADDER_ERR_NULL_POINTER;
     if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
     ConvDims d;
     if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
@@ -359,9 +369,78 @@ int adder_conv2d_grad_w_staged_f32(const float *gy, const float *x, const float 
     const size_t need = grad_w_workspace_bytes(d);
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
     if (overlaps(ws, need, x, nx) || overlaps(ws, need, w, nw) || overlaps(ws, need, gy, ny) ||
-        overlaps(ws, need, gw, nw) || overlaps(gw, nw, x, nx) || overlaps(gw, nw, w, nw) || overlaps(gw, nw, gy, ny))
+        overlaps(ws, need, gw, nw) || overlaps(gw, nw, x, nx) || overlaps(gw, nw, w, nw) || overlaps(gw, nw, gy, ny) ||
+        overlaps(ws, need, bn_y, ny) || overlaps(gw, nw, bn_y, ny) || overlaps(ws, need, bn_coef, 16 * (size_t)Co) ||
+        overlaps(gw, nw, bn_coef, 16 * (size_t)Co) || overlaps(gy_out, ny, gy, ny) || overlaps(gy_out, ny, x, nx) ||
+        overlaps(gy_out, ny, w, nw) || overlaps(gy_out, ny, bn_y, ny) || overlaps(gy_out, ny, bn_coef, 16 * (size_t)Co) ||
+        overlaps(gy_out, ny, gw, nw) || overlaps(gy_out, ny, ws, need))
         return ADDER_ERR_ALIAS;
-    return launch_grad_w_staged(gy, x, w, gw, eta, ws, ws_bytes, d, stage, static_cast<hipStream_t>(stream));
+    return launch_grad_w_staged(gy, x, w, gw, eta, ws, ws_bytes, d, stage, static_cast<hipStream_t>(stream), bn_y,
+                                bn_coef, gy_out);
+}
+
+int adder_conv2d_bwd_bn_slots(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, int *slots) {
+    if (!slots) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    // both halves of the links or neither: the layer needs the fused input-gradient and weight-gradient kernels
+    *slots = grad_w_bn_supported(d, nullptr, nullptr, nullptr, nullptr) ? grad_x_bn_slots(d) : 0;
+    return ADDER_OK;
+}
+
+int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, const float *gx_add, float *gx, float *gw,
+                            float eta, void *ws, size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw,
+                            int stride, int pad, const adder_bn_links *links, void *stream) {
+    if (!gy || !x || !w || !links) return ADDER_ERR_NULL_POINTER;
+    if (!gx && !gw) return ADDER_ERR_NULL_POINTER;
+    if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
+    const adder_bn_links bn = *links;
+    if ((bn.out_x == nullptr) != (bn.out_coef == nullptr) || (bn.out_gy && !bn.out_x)) return ADDER_ERR_NULL_POINTER;
+    if (bn.out_x && gx && !bn.out_gy) return ADDER_ERR_NULL_POINTER;   // grad_X reads the gradient grad_W leaves there
+    if (bn.in_part && (!bn.in_x || !bn.in_mean || !bn.in_rstd || !gx)) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const int slots = grad_w_bn_supported(d, nullptr, nullptr, nullptr, nullptr) ? grad_x_bn_slots(d) : 0;
+    if (slots == 0 || (bn.out_x && !gw)) return ADDER_ERR_UNSUPPORTED;   // (the grad_W kernel is the one that forms gy)
+    if (bn.in_part && bn.in_slots != slots) return ADDER_ERR_BAD_SHAPE;
+    const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo, np = sizeof(double) * 2 * (size_t)Ci * slots,
+                 nc = 16 * (size_t)Co;
+    const void *ins[] = {gy, x, w, gx_add, bn.out_x, bn.out_coef, bn.in_x, bn.in_mean, bn.in_rstd};
+    const size_t in_bytes[] = {ny, nx, nw, nx, ny, nc, nx, 4 * (size_t)Ci, 4 * (size_t)Ci};
+    const size_t need = gw ? grad_w_workspace_bytes(d) : 0;
+    if (gw && (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255))) return ADDER_ERR_WORKSPACE;
+    for (int i = 0; i < 9; ++i)
+        if (overlaps(gx, nx, ins[i], in_bytes[i]) || overlaps(gw, nw, ins[i], in_bytes[i]) ||
+            overlaps(bn.in_part, np, ins[i], in_bytes[i]) || overlaps(bn.out_gy, ny, ins[i], in_bytes[i]) ||
+            (gw && overlaps(ws, need, ins[i], in_bytes[i])))
+            return ADDER_ERR_ALIAS;
+    if (overlaps(gx, nx, gw, nw) || overlaps(gx, nx, bn.in_part, np) || overlaps(gw, nw, bn.in_part, np) ||
+        overlaps(bn.out_gy, ny, gx, nx) || overlaps(bn.out_gy, ny, gw, nw) || overlaps(bn.out_gy, ny, bn.in_part, np) ||
+        (gw && (overlaps(ws, need, gx, nx) || overlaps(ws, need, gw, nw) || overlaps(ws, need, bn.in_part, np) ||
+                overlaps(ws, need, bn.out_gy, ny))))
+        return ADDER_ERR_ALIAS;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (bn.out_x && !grad_w_bn_supported(d, gy, x, bn.out_x, bn.out_coef)) return ADDER_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(bn.out_gy) | reinterpret_cast<uintptr_t>(gx) | reinterpret_cast<uintptr_t>(gx_add) |
+         reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(bn.in_x)) & 15)
+        return ADDER_ERR_UNSUPPORTED;   // before the first launch: the grad_X kernel would refuse these
+    // grad_W first: with the out_* half it is the kernel that turns dz into the gradient of y, which grad_X reads
+    if (gw)
+        if (int rc = launch_grad_w(gy, x, w, gw, eta, ws, ws_bytes, d, s, bn.out_x, bn.out_coef, bn.out_gy)) return rc;
+    if (gx)
+        if (int rc = launch_grad_x_bn(bn.out_x ? bn.out_gy : gy, x, w, gx, d, s, gx_add, bn)) return rc;
+    return ADDER_OK;
+}
+
+int adder_bn_bwd_coef_f32(const double *part, int slots, const float *gamma, const float *save_mean,
+                          const float *save_rstd, double count, float *coef, float *dgamma, float *dbeta, int C,
+                          void *stream) {
+    if (!part || !gamma || !save_mean || !save_rstd || !coef || !dgamma || !dbeta) return ADDER_ERR_NULL_POINTER;
+    if (slots <= 0 || C <= 0 || !(count >= 1.0)) return ADDER_ERR_BAD_SHAPE;
+    if (reinterpret_cast<uintptr_t>(coef) & 15) return ADDER_ERR_UNSUPPORTED;
+    return launch_bn_bwd_coef(part, slots, gamma, save_mean, save_rstd, count, coef, dgamma, dbeta, C,
+                              static_cast<hipStream_t>(stream));
 }
 
 static int check_stages(int count, const adder_grad_w_stage *st) {

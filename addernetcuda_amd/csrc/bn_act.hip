@@ -232,6 +232,36 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_apply_kernel(const float *_
     }
 }
 
+// The whole BatchNorm backward that is left when the neighbouring adder layers do the two passes inside their own
+// kernels: one workgroup per channel adds the partial sums of dz and dz * xhat that the consumer's input-gradient
+// kernel left (fixed order: the result does not depend on which workgroup finished first) and writes dbeta, dgamma
+// and the four numbers per channel from which the producer's backward kernels form their output gradient,
+//   dx = k * dz + c2 * (x - mean) - km1,   k = gamma * rstd, c2 = -k * rstd * mean(dz * xhat), km1 = k * mean(dz).
+__global__ __launch_bounds__(kBnThreads) void bn_bwd_coef_kernel(const double *__restrict__ part, int S, double count,
+                                                                 const float *__restrict__ gamma,
+                                                                 const float *__restrict__ mean,
+                                                                 const float *__restrict__ rstd,
+                                                                 float *__restrict__ coef, float *__restrict__ dgamma,
+                                                                 float *__restrict__ dbeta) {
+    const int c = blockIdx.x;
+    double s1, s2;
+    bn_reduce_partials(part, c, S, s1, s2);
+    if (threadIdx.x == 0) {
+        dbeta[c] = (float)s1;
+        dgamma[c] = (float)s2;
+        const float m1 = (float)(s1 / count), m2 = (float)(s2 / count);
+        const float rs = rstd[c], k = gamma[c] * rs;
+        reinterpret_cast<float4 *>(coef)[c] = make_float4(k, -k * rs * m2, mean[c], k * m1);
+    }
+}
+
+int launch_bn_bwd_coef(const double *part, int slots, const float *gamma, const float *mean, const float *rstd,
+                       double count, float *coef, float *dgamma, float *dbeta, int C, hipStream_t s) {
+    hipLaunchKernelGGL(bn_bwd_coef_kernel, dim3(C), dim3(kBnThreads), 0, s, part, slots, count, gamma, mean, rstd, coef,
+                       dgamma, dbeta);
+    return check_launch();
+}
+
 static int bn_splits(int N, int C, int HW4) {
     const long per_channel = (long)N * HW4;
     long s = 2048 / C;                                   // ~2048 workgroups over the chip

@@ -120,6 +120,12 @@ __device__ __forceinline__ void lds_read_strip(const float *p, float (&dst)[CNT]
     for (; e < CNT; ++e) dst[e] = p[e];
 }
 
+// The same for `CNT` consecutive floats in global memory at an address aligned to `ALIGN` floats.
+template <int CNT, int ALIGN>
+__device__ __forceinline__ void global_read_strip(const float *__restrict__ p, float (&dst)[CNT]) {
+    lds_read_strip<CNT, ALIGN>(p, dst);
+}
+
 // Sum over the 64 lanes of a wave; every lane receives the total.
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
@@ -168,13 +174,23 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
                   hipStream_t s, const float *gadd = nullptr);
 size_t grad_w_workspace_bytes(const ConvDims &d);
 int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta,
-                  void *ws, size_t ws_bytes, const ConvDims &d, hipStream_t s);
+                  void *ws, size_t ws_bytes, const ConvDims &d, hipStream_t s, const float *bn_y = nullptr,
+                  const float *bn_coef = nullptr, float *gy_out = nullptr);
+// the BatchNorm backward passes of a layer's neighbours inside the layer's backward kernels (adder_bn_links)
+int grad_x_bn_slots(const ConvDims &d);
+int launch_grad_x_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d, hipStream_t s,
+                     const float *gadd, const adder_bn_links &bn);
+bool grad_w_bn_supported(const ConvDims &d, const void *gy, const void *x, const void *bn_y, const void *bn_coef);
+int launch_bn_bwd_coef(const double *part, int slots, const float *gamma, const float *mean, const float *rstd,
+                       double count, float *coef, float *dgamma, float *dbeta, int C, hipStream_t s);
 
 // matrix-core weight gradient of the 3x3 / pad-1 layers (grad_w_mfma.hip); variant 0 = not applicable
 struct GradWMfmaPlan { int variant, slots, gy, gz, tilesH, tilesW, ntiles; };
 GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d);
 int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
                        const GradWMfmaPlan &p, hipStream_t s);
+int launch_grad_w_mfma_bn(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+                          const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s);
 
 // 1x1 / pad 0 / stride 1-2 kernels (conv1x1.hip)
 bool conv1x1_supported(const ConvDims &d, const void *a, const void *b);
@@ -202,7 +218,8 @@ int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStrea
 static constexpr int kNormBatchMax = ADDER_NORM_BATCH_MAX;
 static constexpr int kGwFinishMax = ADDER_GRAD_W_FINISH_MAX;
 int launch_grad_w_staged(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
-                         size_t ws_bytes, const ConvDims &d, adder_grad_w_stage *stage, hipStream_t s);
+                         size_t ws_bytes, const ConvDims &d, adder_grad_w_stage *stage, hipStream_t s,
+                         const float *bn_y = nullptr, const float *bn_coef = nullptr, float *gy_out = nullptr);
 size_t grad_w_finish_workspace_bytes(int count, const adder_grad_w_stage *st);
 int launch_grad_w_finish(int count, const adder_grad_w_stage *st, void *ws, hipStream_t s);
 size_t norm_scale_batched_workspace_bytes(int count);

@@ -101,16 +101,55 @@ __device__ __forceinline__ void gy_commit_m(const GyStageM<G> &st, float *buf) {
     }
 }
 
+// The gy tile of a layer that is followed by a BatchNorm, formed from the gradient dz of that BatchNorm's output
+// (already masked by the ReLU behind it), the layer's own output y and four numbers per channel,
+//   gy = k * dz + (c2 * (y - mu) - km1),      coef[channel] = {k, c2, mu, km1}
+// (k = gamma * rstd, c2 = -k * rstd * mean(dz * xhat), km1 = k * mean(dz)): the second pass of the BatchNorm
+// backward, done on the way into LDS.  gy_out (nullable): the same values go to this tensor, shaped like gy, for
+// the input-gradient kernel that runs next.  coef: the workgroup's COB channels, in LDS.
+template <class G>
+__device__ __forceinline__ void gy_commit_m_bn(const GyStageM<G> &sg, const GyStageM<G> &sy, float *buf,
+                                               const float4 *coef, float *__restrict__ gy_out, int co0, int Co, int n0,
+                                               int N, int h0, int w0, int Ho, int Wo) {
+#pragma unroll
+    for (int it = 0; it < G::GITER; ++it) {
+        const int u = threadIdx.x + it * G::NTHREADS;
+        if (G::GUNITS % G::NTHREADS == 0 || u < G::GUNITS) {
+            const int q = u % (G::TW / 4);
+            const int r = (u / (G::TW / 4)) % G::TH;
+            const int pc = u / (G::TW / 4) / G::TH;   // = img*COB + c
+            const int c = pc % G::COB, img = pc / G::COB;
+            const bool ok = n0 + img < N && co0 + c < Co && h0 + r < Ho && w0 + 4 * q < Wo;   // rows are whole groups of four
+            const float4 cf = coef[c];
+            const float4 g = sg.v[it], y = sy.v[it];
+            float4 v;
+            v.x = ok ? fmaf(cf.x, g.x, fmaf(cf.y, y.x - cf.z, -cf.w)) : 0.f;
+            v.y = ok ? fmaf(cf.x, g.y, fmaf(cf.y, y.y - cf.z, -cf.w)) : 0.f;
+            v.z = ok ? fmaf(cf.x, g.z, fmaf(cf.y, y.z - cf.z, -cf.w)) : 0.f;
+            v.w = ok ? fmaf(cf.x, g.w, fmaf(cf.y, y.w - cf.z, -cf.w)) : 0.f;
+            *reinterpret_cast<float4 *>(buf + pc * G::GPLANE + r * G::TW + 4 * q) = v;
+            if (gy_out && ok)
+                *reinterpret_cast<float4 *>(gy_out + ((((n0 + img) * Co + co0 + c) * Ho + h0 + r) * Wo + w0 + 4 * q)) = v;
+        }
+    }
+}
+
 // SUB (single tap only): x is a sampled tensor (see Subsample), read element by element at the sampled
 // positions; gy is dense.  VEC then only says how gy is read.
 // T: storage type of gy and x (float, or bf16_t for the reduced-storage mode); staged as fp32, multiplied in fp64.
-template <class G, bool VEC = true, bool SUB = false, class T = float>
+// FUSE: gy holds dz and the gy tiles are formed from (dz, bn_y, bn_coef) on the way into LDS (gy_commit_m_bn), and
+// written to gy_out (nullable) by the workgroups of the first k block; float storage, rows of whole float4 groups.
+template <class G, bool VEC = true, bool SUB = false, class T = float, bool FUSE = false>
 __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__restrict__ gy,
                                                                   const T *__restrict__ x,
                                                                   double *__restrict__ part,
                                                                   double *__restrict__ sgpart, int N, int Ci, int H,
                                                                   int W, int Co, int Ho, int Wo, int tilesH,
-                                                                  int tilesW, int ntiles, const Subsample sub) {
+                                                                  int tilesW, int ntiles, const Subsample sub,
+                                                                  const float *__restrict__ bn_y,
+                                                                  const float *__restrict__ bn_coef,
+                                                                  float *__restrict__ gy_out) {
+    static_assert(!FUSE || (VEC && !SUB && sizeof(T) == 4), "the BatchNorm link belongs to the float kernels");
     using XP = typename G::XP;
     constexpr int S = G::S, MT = G::MT, NT = G::NT;
     extern __shared__ __align__(16) float smem[];
@@ -141,7 +180,15 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
     }
 
     TileStage<XP> xs;
-    GyStageM<G> gs;
+    GyStageM<G> gs, ys;   // (ys: FUSE only)
+    const float4 *coef = reinterpret_cast<const float4 *>(smem + G::LDS_FLOATS);
+    float *const gy_dst = blockIdx.z == 0 ? gy_out : nullptr;   // every gy tile is staged once per k block
+    if constexpr (FUSE) {
+        for (int e = threadIdx.x; e < G::COB; e += G::NTHREADS)
+            reinterpret_cast<float4 *>(smem + G::LDS_FLOATS)[e] =
+                reinterpret_cast<const float4 *>(bn_coef)[min(co_blk + e, Co - 1)];
+        __syncthreads();
+    }
     int tile = blockIdx.x;
     int n0 = 0, h0 = 0, w0 = 0;
     auto decode = [&](int t) {
@@ -153,8 +200,10 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
         decode(tile);
         tile_fetch<XP, VEC && !SUB, SUB, T>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
         gy_fetch_m<G, VEC, T>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+        if constexpr (FUSE) gy_fetch_m<G, true, float>(ys, bn_y, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         tile_commit<XP>(xs, smem);
-        gy_commit_m<G>(gs, smem + XP::BUF);
+        if constexpr (FUSE) gy_commit_m_bn<G>(gs, ys, smem + XP::BUF, coef, gy_dst, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+        else gy_commit_m<G>(gs, smem + XP::BUF);
     }
     __syncthreads();
 
@@ -165,6 +214,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
             decode(next);
             tile_fetch<XP, VEC && !SUB, SUB, T>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
             gy_fetch_m<G, VEC, T>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+            if constexpr (FUSE) gy_fetch_m<G, true, float>(ys, bn_y, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         }
         const float *base = smem + cur * G::BUF;
         auto steps = [&](const int first, const int last) {
@@ -195,7 +245,11 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
         steps(0, G::WSTEPS / 2);
         if (next < ntiles) {
             tile_commit<XP>(xs, smem + (cur ^ 1) * G::BUF);
-            gy_commit_m<G>(gs, smem + (cur ^ 1) * G::BUF + XP::BUF);
+            if constexpr (FUSE)
+                gy_commit_m_bn<G>(gs, ys, smem + (cur ^ 1) * G::BUF + XP::BUF, coef, gy_dst, co_blk, Co, n0, N, h0, w0, Ho,
+                                  Wo);
+            else
+                gy_commit_m<G>(gs, smem + (cur ^ 1) * G::BUF + XP::BUF);
         }
         steps(G::WSTEPS / 2, G::WSTEPS);
         __syncthreads();
@@ -336,12 +390,15 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     return p;
 }
 
-template <class G, bool VEC, bool SUB = false, class T = float>
+template <class G, bool VEC, bool SUB = false, class T = float, bool FUSE = false>
 static int launch_one_v(const T *gy, const T *x, double *part, double *sgpart, const ConvDims &d,
-                      const GradWMfmaPlan &p, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0}) {
-    if (int rc = allow_dynamic_lds<&grad_w_mfma_kernel<G, VEC, SUB, T>>(G::LDS_BYTES)) return rc;
-    hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC, SUB, T>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), G::LDS_BYTES, s, gy, x,
-                       part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles, sub);
+                      const GradWMfmaPlan &p, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0},
+                      const float *bn_y = nullptr, const float *bn_coef = nullptr, float *gy_out = nullptr) {
+    constexpr int LDS_BYTES = G::LDS_BYTES + (FUSE ? G::COB * 16 : 0);   // + the BatchNorm coefficients of the block
+    if (int rc = allow_dynamic_lds<&grad_w_mfma_kernel<G, VEC, SUB, T, FUSE>>(LDS_BYTES)) return rc;
+    hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC, SUB, T, FUSE>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), LDS_BYTES, s,
+                       gy, x, part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles, sub, bn_y,
+                       bn_coef, gy_out);
     return check_launch();
 }
 
@@ -362,6 +419,28 @@ int launch_grad_w_mfma_bf16(const bf16_t *gy, const bf16_t *x, double *part, dou
         case 3: return launch_one<GmW8, bf16_t>(gy, x, part, sgpart, d, p, s);
         case 4: return launch_one<GmW16S2, bf16_t>(gy, x, part, sgpart, d, p, s);
         case 5: return launch_one<GmW8S2, bf16_t>(gy, x, part, sgpart, d, p, s);
+        default: return ADDER_ERR_UNSUPPORTED;
+    }
+}
+
+// The 3x3 / pad-1 variants with gy formed from (dz = gy, bn_y, bn_coef) while it is staged and left in gy_out
+// (nullable) on the way (see gy_commit_m_bn); ADDER_ERR_UNSUPPORTED for other variants and for rows that are not
+// whole float4 groups.
+int launch_grad_w_mfma_bn(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
+                          const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s) {
+    if (d.W % 4 != 0 || d.Wo % 4 != 0) return ADDER_ERR_UNSUPPORTED;
+    const Subsample none{1, 0, 0, 0};
+    switch (p.variant) {
+        case 1: return launch_one_v<GmW32, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
+                                                                           gy_out);
+        case 2: return launch_one_v<GmW16, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
+                                                                           gy_out);
+        case 3: return launch_one_v<GmW8, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
+                                                                           gy_out);
+        case 4: return launch_one_v<GmW16S2, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
+                                                                           gy_out);
+        case 5: return launch_one_v<GmW8S2, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
+                                                                           gy_out);
         default: return ADDER_ERR_UNSUPPORTED;
     }
 }

@@ -96,15 +96,21 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const T *__restrict
 // positions as one row per plane, reads x there, and stores each result together with the zeros of the
 // s x s block of input positions around it that the layer never read.
 // T: storage type of gy, x, gx and gadd (float, or bf16_t for the reduced-storage mode).
-template <class C, bool VEC = true, bool SAT = true, bool SUB = false, class T = float>
+// FUSE: the statistics pass of the backward of the BatchNorm in front of the layer is done here (the in_* fields
+// of adder_bn_links): the result is masked with x > 0 (bn.in_relu) and its per-channel sums are left in
+// bn.in_part, (Ci, gridDim.x * POSW, 2) doubles.  3x3 taps, float storage, rows of whole float4 groups.
+template <class C, bool VEC = true, bool SAT = true, bool SUB = false, class T = float, bool FUSE = false>
 __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *__restrict__ gy,
                                                                    const T *__restrict__ x,
                                                                    const float *__restrict__ w,
                                                                    T *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int tilesH,
                                                                    int tilesW, const Subsample sub,
-                                                                   const T *__restrict__ gadd) {
+                                                                   const T *__restrict__ gadd,
+                                                                   const adder_bn_links bn) {
     static_assert(!SUB || C::KS == 1, "sampling is for single-tap layers");
+    static_assert(!FUSE || (C::KS == 3 && VEC && !SUB && sizeof(T) == 4 && C::TM * C::TN <= 32),
+                  "the BatchNorm link belongs to the float 3x3 kernels");
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
 
@@ -150,6 +156,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
         }
     }
     const int xplane = SUB ? sub.plane : H * W;
+    unsigned xpos = 0;   // FUSE: bit m * TN + t = (x > 0) of the own positions
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
@@ -159,8 +166,12 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
             const float xv = ldf(src + xoff[t]);
             cr[m][t] = SAT ? fmaf(-0.5f, xv, 0.5f) : xv;
             acc[m][t] = tot[m][t] = 0.f;
+            if constexpr (FUSE) xpos |= (xv > 0.f ? 1u : 0u) << (m * TN + t);
         }
     }
+    // (pinned here: left alone, the compiler moves the comparisons down to where the bits are used and keeps all
+    // the x values in registers through the main loop for that)
+    if constexpr (FUSE) asm volatile("" : "+v"(xpos));
     // per tile position, the sum of gy over all output channels: every thread owns GITER elements of the
     // plane and adds them up in double in registers (one conversion and one add per chunk -- the sum is taken
     // off a sum of the same size at the end, so its rounding counts), the plane itself is written once
@@ -321,6 +332,31 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
         __syncthreads();
     }
 
+    // FUSE: what the epilogue needs from memory is asked for now, behind the last barrier of the main loop, so that
+    // it arrives while the correction below is worked out (the main loop's registers are free from here on).
+    // The strips' offset is formed from values the compiler cannot connect with the loads of x at the top -- it would
+    // keep their sixteen 64-bit addresses in registers through the whole main loop.  Rows are whole strips here; a
+    // strip beyond the row (a tile wider than the tensor) reads the row's last one.  Every lane loads, from inside
+    // the tensor; invalid lanes are dropped when the sums are taken.
+    float bx[FUSE ? TM : 1][TN], ga[FUSE ? TM : 1][TN];
+    if constexpr (FUSE) {
+        if (bn.in_part) {
+            static_assert(!FUSE || TN == 2 || TN == 4, "the strips are read as one float2 / float4");
+            int pofs = (nc * Ci + ci_base) * (H * W) + hc * W + min(wi0, W - TN);
+            asm volatile("" : "+v"(pofs));
+#pragma unroll
+            for (int m = 0; m < TM; ++m) {
+                global_read_strip<TN, TN>(bn.in_x + pofs + m * (H * W), bx[m]);
+                if (gadd) {
+                    global_read_strip<TN, TN>(reinterpret_cast<const float *>(gadd) + pofs + m * (H * W), ga[m]);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < TN; ++t) ga[m][t] = 0.f;
+                }
+            }
+        }
+    }
+
     // sum over (co, taps) of the gy values a position met = box sum of the channel-sum plane
     if constexpr (SAT) {
 #pragma unroll
@@ -343,6 +379,36 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
                 for (int j = 0; j < KS; ++j) sg += gs[i][t + j];
 #pragma unroll
             for (int m = 0; m < TM; ++m) tot[m][t] = fmaf(2.f, tot[m][t], -sg);
+        }
+    }
+
+    if constexpr (FUSE) {
+        if (bn.in_part) {
+            // x = relu(bn(in_x) [+ residual]): what leaves here is the gradient of the BatchNorm's output before
+            // the ReLU, dz = (gx + gadd) * [x > 0], and per channel and position wave the sums of dz and dz * xhat
+            // in the partial-sum layout of the BatchNorm kernels (a wave's 64 * TN terms in fp32, the rest in fp64)
+            const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+#pragma unroll
+            for (int m = 0; m < TM; ++m) {
+                const int ci = ci_base + m;
+                const float mu = bn.in_mean[ci], rs = bn.in_rstd[ci];
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    const bool valid = pos_ok && wi0 + t < W && ci >= ci_first;
+                    float v = tot[m][t] + ga[m][t];
+                    if (bn.in_relu && !((xpos >> (m * TN + t)) & 1u)) v = 0.f;
+                    tot[m][t] = v;
+                    s1 += valid ? v : 0.f;
+                    s2 = fmaf(valid ? v : 0.f, (bx[m][t] - mu) * rs, s2);
+                }
+                const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2);
+                if (lane == 0 && ci >= ci_first) {
+                    bn.in_part[((size_t)ci * slots + slot) * 2] = d1;
+                    bn.in_part[((size_t)ci * slots + slot) * 2 + 1] = d2;
+                }
+            }
+            gadd = nullptr;   // already added
         }
     }
 
@@ -394,19 +460,31 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
 // and carries the full magnitude (512 -> 2048 @7x7 at batch 64 had one element in 1e5 at 1.2 of the tolerance).
 static constexpr int kSatMaxTerms = 2304, kSatMaxTerms1x1 = 1024;
 
-template <class C, bool VEC, bool SAT, bool SUB = false, class T = float>
+static const adder_bn_links kNoLinks{};
+
+template <class C, bool VEC, bool SAT, bool SUB = false, class T = float, bool FUSE = false>
 static int launch_grad_x_3x3s1_v(const T *gy, const T *x, const float *w, T *gx,
                                const ConvDims &d, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0},
-                               const T *gadd = nullptr) {
+                               const T *gadd = nullptr, const adder_bn_links &bn = kNoLinks) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
+    if (FUSE && bn.in_part && bn.in_slots != gxd * C::POSW) return ADDER_ERR_BAD_SHAPE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
-    if (int rc = allow_dynamic_lds<&grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T>>(LDS_BYTES)) return rc;
-    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
-                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW, sub, gadd);
+    if (int rc = allow_dynamic_lds<&grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T, FUSE>>(LDS_BYTES)) return rc;
+    hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T, FUSE>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS),
+                       LDS_BYTES, s, gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, tilesH, tilesW, sub, gadd, bn);
     return check_launch();
+}
+
+// the same with the in_* half of adder_bn_links (float tensors with rows of whole float4 groups)
+template <class C>
+static int launch_grad_x_3x3s1_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
+                                  hipStream_t s, const float *gadd, const adder_bn_links &bn) {
+    if (d.Co * C::KK > kSatMaxTerms)
+        return launch_grad_x_3x3s1_v<C, true, false, false, float, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd, bn);
+    return launch_grad_x_3x3s1_v<C, true, true, false, float, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd, bn);
 }
 
 // picks the element-wise tile loads (rows of the staged tensor that are not whole float4 groups) and the
@@ -448,15 +526,18 @@ struct GradX3x3S2Cfg {
     static_assert(TNW % 2 == 0 && TH % 2 == 0, "lanes own 2 x 2 parity blocks");
 };
 
-template <class C, bool VEC = true, bool SAT = true, class T = float>
+// FUSE, bn: as in the stride-1 kernel.
+template <class C, bool VEC = true, bool SAT = true, class T = float, bool FUSE = false>
 __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__restrict__ gy,
                                                                    const T *__restrict__ x,
                                                                    const float *__restrict__ w,
                                                                    T *__restrict__ gx, int N, int Ci,
                                                                    int H, int W, int Co, int Ho, int Wo,
                                                                    int tilesH, int tilesW,
-                                                                   const T *__restrict__ gadd) {
+                                                                   const T *__restrict__ gadd,
+                                                                   const adder_bn_links bn) {
     constexpr int TNW = C::TNW, TM = C::TM, GSTRIP = C::GSTRIP;
+    static_assert(!FUSE || (VEC && sizeof(T) == 4 && TM * 2 * TNW <= 32), "the BatchNorm link belongs to the float kernels");
     extern __shared__ __align__(16) float smem[];
 
     int b = blockIdx.x;
@@ -483,6 +564,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
     const int nc = min(n, N - 1);
 
     float cr[TM][2][TNW], acc[TM][2][TNW], tot[TM][2][TNW];   // cr = 0.5 - 0.5 x, as in the stride-1 kernel
+    unsigned xpos = 0;   // FUSE: bit (m * 2 + rp) * TNW + t = (x > 0) of the own positions
 #pragma unroll
     for (int m = 0; m < TM; ++m) {
         const int ci = ci_base + m;
@@ -494,9 +576,11 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
                 const float xv = ldf(src + min(wi0 + t, W - 1));
                 cr[m][rp][t] = SAT ? fmaf(-0.5f, xv, 0.5f) : xv;
                 acc[m][rp][t] = tot[m][rp][t] = 0.f;
+                if constexpr (FUSE) xpos |= (xv > 0.f ? 1u : 0u) << ((m * 2 + rp) * TNW + t);
             }
         }
     }
+    if constexpr (FUSE) asm volatile("" : "+v"(xpos));   // pinned here, as in the stride-1 kernel
     constexpr int GN = C::NIMG * C::PLANE, GITER = ceil_div(GN, C::NTHREADS);
     float *gplane = smem + 2 * C::BUF;   // per tile position, the sum of gy over all output channels
     double gsum[GITER];                  // ... collected in double in registers, as in the stride-1 kernel
@@ -600,6 +684,29 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
         __syncthreads();
     }
 
+    // FUSE: the epilogue's loads, issued here as in the stride-1 kernel
+    float bx[FUSE ? TM : 1][2][TNW], ga[FUSE ? TM : 1][2][TNW];
+    if constexpr (FUSE) {
+        if (bn.in_part) {
+            static_assert(!FUSE || TNW == 2, "the strips are read as one float2");
+#pragma unroll
+            for (int rp = 0; rp < 2; ++rp) {
+                int pofs = ((nc * Ci + ci_base) * H + min(hi0 + rp, H - 1)) * W + min(wi0, W - TNW);
+                asm volatile("" : "+v"(pofs));
+#pragma unroll
+                for (int m = 0; m < TM; ++m) {
+                    global_read_strip<TNW, TNW>(bn.in_x + pofs + m * (H * W), bx[m][rp]);
+                    if (gadd) {
+                        global_read_strip<TNW, TNW>(reinterpret_cast<const float *>(gadd) + pofs + m * (H * W), ga[m][rp]);
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < TNW; ++t) ga[m][rp][t] = 0.f;
+                    }
+                }
+            }
+        }
+    }
+
     // clamp = 2 * sat - 1: take off the sum of the gy values each position met (same taps as above)
     if constexpr (SAT) {
 #pragma unroll
@@ -629,6 +736,36 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
             for (int rp = 0; rp < 2; ++rp)
 #pragma unroll
                 for (int t = 0; t < TNW; ++t) tot[m][rp][t] = fmaf(2.f, tot[m][rp][t], -sg[rp][t]);
+    }
+
+    if constexpr (FUSE) {
+        if (bn.in_part) {   // dz = (gx + gadd) * [x > 0] and its per-channel sums, as in the stride-1 kernel
+            const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+#pragma unroll
+            for (int m = 0; m < TM; ++m) {
+                const int ci = ci_base + m;
+                const float mu = bn.in_mean[ci], rs = bn.in_rstd[ci];
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int rp = 0; rp < 2; ++rp) {
+#pragma unroll
+                    for (int t = 0; t < TNW; ++t) {
+                        const bool valid = lane_ok && n < N && hi0 + rp < H && wi0 + t < W && ci >= ci_first;
+                        float v = tot[m][rp][t] + ga[m][rp][t];
+                        if (bn.in_relu && !((xpos >> ((m * 2 + rp) * TNW + t)) & 1u)) v = 0.f;
+                        tot[m][rp][t] = v;
+                        s1 += valid ? v : 0.f;
+                        s2 = fmaf(valid ? v : 0.f, (bx[m][rp][t] - mu) * rs, s2);
+                    }
+                }
+                const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2);
+                if (lane == 0 && ci >= ci_first) {
+                    bn.in_part[((size_t)ci * slots + slot) * 2] = d1;
+                    bn.in_part[((size_t)ci * slots + slot) * 2 + 1] = d2;
+                }
+            }
+            gadd = nullptr;   // already added
+        }
     }
 
     if (lane_ok && n < N) {
@@ -662,18 +799,26 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
     }
 }
 
-template <class C, bool VEC, bool SAT, class T = float>
+template <class C, bool VEC, bool SAT, class T = float, bool FUSE = false>
 static int launch_grad_x_3x3s2_v(const T *gy, const T *x, const float *w, T *gx,
-                               const ConvDims &d, hipStream_t s, const T *gadd) {
+                               const ConvDims &d, hipStream_t s, const T *gadd, const adder_bn_links &bn = kNoLinks) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
+    if (FUSE && bn.in_part && bn.in_slots != gxd * C::POSW) return ADDER_ERR_BAD_SHAPE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
-    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
-                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, gadd);
+    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T, FUSE>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
+                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, gadd, bn);
     return check_launch();
+}
+
+template <class C>
+static int launch_grad_x_3x3s2_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
+                                  hipStream_t s, const float *gadd, const adder_bn_links &bn) {
+    if (d.Co * 4 > kSatMaxTerms) return launch_grad_x_3x3s2_v<C, true, false, float, true>(gy, x, w, gx, d, s, gadd, bn);
+    return launch_grad_x_3x3s2_v<C, true, true, float, true>(gy, x, w, gx, d, s, gadd, bn);
 }
 
 template <class C, class T = float>
@@ -761,6 +906,49 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
     hipLaunchKernelGGL(grad_x_generic_kernel<TM>, dim3((unsigned)ceil_div_l(total, 256), ceil_div(d.Ci, TM)),
                        dim3(256), 0, s, gy, x, w, gx, d);
     return check_launch();
+}
+
+// Which tiled kernel carries the BatchNorm link for this layer: 1 GxW32, 2 GxW16, 3 GxW8 (stride 1), 4 GxS2W32,
+// 5 GxS2W16 (stride 2); 0: none (other kernel sizes, rows that are not whole float4 groups, fewer than TM channels).
+static int grad_x_bn_variant(const ConvDims &d) {
+    if (d.kh != 3 || d.kw != 3 || d.pad != 1 || d.Ci < GxW32::TM) return 0;
+    if (d.stride == 1 && d.W % 4 == 0) return d.W > 16 ? 1 : (d.W > 8 ? 2 : 3);
+    if (d.stride == 2 && d.W % 4 == 0 && d.Wo % 4 == 0) return d.W > 16 ? 4 : 5;
+    return 0;
+}
+
+template <class C>
+static int bn_slots_of(const ConvDims &d) {
+    return ceil_div(d.N, C::NIMG) * ceil_div(d.H, C::TH) * ceil_div(d.W, C::TW) * C::POSW;
+}
+
+// partial-sum slots per input channel that launch_grad_x_bn writes into bn.in_part; 0: no such kernel for the layer
+int grad_x_bn_slots(const ConvDims &d) {
+    switch (grad_x_bn_variant(d)) {
+        case 1: return bn_slots_of<GxW32>(d);
+        case 2: return bn_slots_of<GxW16>(d);
+        case 3: return bn_slots_of<GxW8>(d);
+        case 4: return bn_slots_of<GxS2W32>(d);
+        case 5: return bn_slots_of<GxS2W16>(d);
+        default: return 0;
+    }
+}
+
+// launch_grad_x with the statistics pass of the BatchNorm in front of the layer folded in (the in_* fields of
+// adder_bn_links); ADDER_ERR_UNSUPPORTED where the layer has no such kernel or a tensor is not 16-byte aligned
+int launch_grad_x_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d, hipStream_t s,
+                     const float *gadd, const adder_bn_links &bn) {
+    const uintptr_t align = reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx) |
+                            reinterpret_cast<uintptr_t>(gadd) | reinterpret_cast<uintptr_t>(bn.in_x);
+    if (align & 15) return ADDER_ERR_UNSUPPORTED;
+    switch (grad_x_bn_variant(d)) {
+        case 1: return launch_grad_x_3x3s1_bn<GxW32>(gy, x, w, gx, d, s, gadd, bn);
+        case 2: return launch_grad_x_3x3s1_bn<GxW16>(gy, x, w, gx, d, s, gadd, bn);
+        case 3: return launch_grad_x_3x3s1_bn<GxW8>(gy, x, w, gx, d, s, gadd, bn);
+        case 4: return launch_grad_x_3x3s2_bn<GxS2W32>(gy, x, w, gx, d, s, gadd, bn);
+        case 5: return launch_grad_x_3x3s2_bn<GxS2W16>(gy, x, w, gx, d, s, gadd, bn);
+        default: return ADDER_ERR_UNSUPPORTED;
+    }
 }
 
 // bfloat16 storage: the tiled 3x3 / pad-1 kernels (stride 1 or 2), the generic kernel for everything else

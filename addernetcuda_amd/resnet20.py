@@ -21,6 +21,7 @@ import torch.nn.functional as F
 
 from . import adder as _adder
 from .bn_act import BatchNormAct2d
+from .unit import adder_bn_act
 
 
 class BasicBlock(nn.Module):
@@ -55,22 +56,22 @@ class BasicBlock(nn.Module):
                 residual = self.downsample(x)
             out += residual
             return self.relu(out)
-        if self.bn1.training and x.is_cuda and x.requires_grad and hasattr(self.conv1, "forward_with_stats"):
-            # x leaves conv1's autograd node a second time and feeds the shortcut from there, so that the
-            # shortcut's gradient is added to conv1's input gradient by the kernel that computes it, not by
-            # a launch of its own
-            out, stats, shortcut = self.conv1.forward_with_stats(x, with_shortcut=True)
-            out = self.bn1(out, stats=stats)
-            if self.downsample is not None:
-                ds = self.downsample
-                if isinstance(ds, nn.Sequential) and len(ds) == 2 and isinstance(ds[1], BatchNormAct2d):
-                    shortcut = self._conv_bn(ds[0], ds[1], shortcut)   # statistics from the 1x1 kernel's epilogue
-                else:
-                    shortcut = ds(shortcut)
-            return self._conv_bn(self.conv2, self.bn2, out, shortcut)
-        out = self._conv_bn(self.conv1, self.bn1, x)                    # bn + relu
-        shortcut = x if self.downsample is None else self.downsample(x)
-        return self._conv_bn(self.conv2, self.bn2, out, shortcut)       # bn + residual + relu
+        # every conv -> bn (-> + shortcut) -> relu group is one autograd node (unit.py): the BatchNorm statistics
+        # come out of the adder kernel's epilogue, and in the backward pass the BatchNorm's own two passes are
+        # folded into the adder kernels on either side of it
+        if self.bn1.training and x.is_cuda and x.requires_grad:
+            # x leaves conv1's node a second time and feeds the shortcut from there, so that the shortcut's
+            # gradient is added to conv1's input gradient by the kernel that computes it, not by a launch of its own
+            out, shortcut = adder_bn_act(self.conv1, self.bn1, x, with_shortcut=True)
+        else:
+            out, shortcut = adder_bn_act(self.conv1, self.bn1, x), x
+        if self.downsample is not None:
+            ds = self.downsample
+            if isinstance(ds, nn.Sequential) and len(ds) == 2 and isinstance(ds[1], BatchNormAct2d):
+                shortcut = adder_bn_act(ds[0], ds[1], shortcut)
+            else:
+                shortcut = ds(shortcut)
+        return adder_bn_act(self.conv2, self.bn2, out, residual=shortcut)
 
 
 class _conv2d_matrix_grad(torch.autograd.Function):

@@ -265,6 +265,67 @@ ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsign
                                    float *dx, float *dresidual, float *dgamma, float *dbeta, int relu,
                                    int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);
 
+/* ------------------------------------------------------------------------
+ * The BatchNorm backward passes folded into the adder layers' backward kernels.  No counterpart in the
+ * reference, where bn -> relu and the adder layer are separate autograd nodes (resnet20.py:28-39) and the
+ * BatchNorm backward is two passes of its own over every activation gradient.  In a chain
+ *     ... -> adder A -> BatchNorm P -> (+ residual) -> ReLU -> adder B -> BatchNorm Q -> ...
+ * the backward of B already holds what P's backward needs.  Its grad_X kernel has x = relu(...) and its own
+ * result in registers, so it can write dz = (grad_X [+ gx_add]) * [x > 0], the gradient of P's output before
+ * the ReLU (which is also the gradient of the residual), and P's per-channel sums of dz and dz * xhat (the
+ * first pass of P's backward).  And A's grad_W kernel can form its gy = dP_input from (dz, A's output y, four
+ * numbers per channel) while it stages gy into LDS (the second pass):
+ *     gy = k * dz + c2 * (y - mean) - km1,   k = gamma * rstd, c2 = -k * rstd * mean(dz * xhat), km1 = k * mean(dz),
+ * and leave the result in memory for A's grad_X kernel, which runs after it.  P's backward is then one tiny
+ * launch (adder_bn_bwd_coef_f32) instead of two passes over the activation gradient.
+ *
+ *   adder_bn_links: what a layer's backward is told about its two neighbours; either half may be absent (NULL).
+ *     out_x, out_coef, out_gy   the BatchNorm BEHIND the layer: out_x = the layer's output y (N, Co, Ho, Wo),
+ *                      out_coef = 4 floats per output channel {k, c2, mean, km1} from adder_bn_bwd_coef_f32;
+ *                      the `gy` argument is then dz, not the gradient of y; out_gy (N, Co, Ho, Wo) receives the
+ *                      gradient of y from the grad_W kernel.
+ *     in_x, in_mean, in_rstd, in_part, in_slots, in_relu   the BatchNorm IN FRONT of the layer, whose output
+ *                      (after the residual add and, if in_relu, the ReLU) is the layer's x: in_x = that
+ *                      BatchNorm's input (N, Ci, H, W), its saved mean / rstd (Ci); in_part receives
+ *                      (Ci, in_slots, 2) doubles, in_slots = adder_conv2d_bwd_bn_slots; gx receives dz.
+ *   adder_conv2d_bwd_bn_slots: partial-sum slots per channel for in_part; 0 = this layer has no such kernels
+ *     (they exist for 3x3 / pad 1 / stride 1 or 2 layers whose rows are whole groups of four floats).
+ *   adder_conv2d_bwd_bn_f32: adder_conv2d_bwd_add_f32 (gx_add nullable here) with the links.  With the out_*
+ *     half gw must be requested (the grad_W kernel is the one that forms gy); a caller that stages grad_W
+ *     (adder_conv2d_grad_w_staged_bn_f32) calls this afterwards with gy = its out_gy and without the out_* half.
+ *     ADDER_ERR_UNSUPPORTED, nothing launched, where adder_conv2d_bwd_bn_slots is 0 or a tensor is not
+ *     16-byte aligned.
+ *   adder_conv2d_grad_w_staged_bn_f32: adder_conv2d_grad_w_staged_f32 with the out_* half of the links
+ *     (out_gy nullable).
+ *   adder_bn_bwd_coef_f32: sums the slots of `part` (C, slots, 2) in a fixed order and writes coef (C, 4),
+ *     dgamma and dbeta (C); count = N * H * W of the BatchNorm.
+ * ---------------------------------------------------------------------- */
+typedef struct adder_bn_links {
+    const float *out_x;
+    const float *out_coef;
+    float *out_gy;
+    const float *in_x;
+    const float *in_mean;
+    const float *in_rstd;
+    double *in_part;
+    int in_slots;
+    int in_relu;
+} adder_bn_links;
+ADDER_API int adder_conv2d_bwd_bn_slots(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad,
+                                        int *slots);
+ADDER_API int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, const float *gx_add,
+                         float *gx, float *gw, float eta,
+                         void *ws, size_t ws_bytes,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, const adder_bn_links *links, void *stream);
+ADDER_API int adder_conv2d_grad_w_staged_bn_f32(const float *gy, const float *x, const float *w, float *gw, float eta,
+                         void *ws, size_t ws_bytes,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, const adder_bn_links *links, adder_grad_w_stage *stage, void *stream);
+ADDER_API int adder_bn_bwd_coef_f32(const double *part, int slots, const float *gamma, const float *save_mean,
+                                    const float *save_rstd, double count, float *coef, float *dgamma, float *dbeta,
+                                    int C, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
