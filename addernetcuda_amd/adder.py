@@ -391,11 +391,14 @@ def plain_conv2d_forward(X, W, stride, padding):
     return y, stats
 
 
-def conv2d_weight_grad(grad_out, X, W, stride, padding):
+def conv2d_weight_grad(grad_out, X, W, stride, padding, out_link=None):
     """Weight gradient of an *ordinary* convolution ``F.conv2d(X, W, None, stride, padding)``, i.e. the
     ``sum x * gy`` half of the adder layer's weight gradient, from the same fp64 matrix-core kernel (the slab
     finalize leaves the ``- w * sum gy`` term out).  Inside a ``batched_eta_scaling()`` block it is finished
-    together with the adder layers' gradients.  Returns None where the geometry has no such kernel."""
+    together with the adder layers' gradients.  Returns None where the geometry has no such kernel.
+    ``out_link``: a BnLink whose ``coef`` is ready -- ``grad_out`` is then dz of the BatchNorm behind the
+    convolution, and the kernel forms the convolution's output gradient from it (None is returned, and nothing
+    launched, where the kernel cannot)."""
     grad_out, X = grad_out.contiguous(), X.contiguous()
     require_gpu_f32(grad_out, "grad_output")
     require_gpu_f32(X, "X")
@@ -405,8 +408,15 @@ def conv2d_weight_grad(grad_out, X, W, stride, padding):
     with on_device(dev):
         ws, nbytes = conv2d_bwd_workspace(dims, dev)
         stage = GradWStage()
-        status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), None, ptr(gw), 0.0, ptr(ws), nbytes, *dims,
-                                                    ctypes.byref(stage), stream_ptr(dev))
+        if out_link is not None:
+            links = BnLinks()
+            links.out_x, links.out_coef = ptr(out_link.bn_x), ptr(out_link.coef)
+            status = lib.adder_conv2d_grad_w_staged_bn_f32(ptr(grad_out), ptr(X), None, ptr(gw), 0.0, ptr(ws), nbytes,
+                                                           *dims, ctypes.byref(links), ctypes.byref(stage),
+                                                           stream_ptr(dev))
+        else:
+            status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), None, ptr(gw), 0.0, ptr(ws), nbytes,
+                                                        *dims, ctypes.byref(stage), stream_ptr(dev))
         if status == -7:
             return None
         check(status, "adder_conv2d_grad_w_staged_f32")

@@ -20,7 +20,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import adder as _adder
-from .bn_act import BatchNormAct2d
+from .bn_act import BatchNormAct2d, bn_forward, bn_backward
 from .unit import adder_bn_act
 
 
@@ -107,6 +107,49 @@ class _conv2d_matrix_grad(torch.autograd.Function):
         return gx, gw, None, None
 
 
+class _conv_bn_act(torch.autograd.Function):
+    """``relu(bn(conv(x)))`` for an ordinary convolution as one autograd node, the counterpart of unit.py for the
+    stem (resnet20.py:49-51, 81-83): when the adder layer that consumes the output has left the BatchNorm's
+    backward sums (``BnLink``), the weight-gradient kernel forms the convolution's output gradient itself and the
+    BatchNorm's two backward passes are not run.  The input is an image batch: no input gradient on that path."""
+
+    @staticmethod
+    def forward(ctx, x, w, gamma, beta, running_mean, running_var, num_batches, momentum, eps, relu, stride, padding):
+        x, w = x.contiguous(), w.contiguous()
+        conv_out, stats = _adder.plain_conv2d_forward(x, w, stride, padding)
+        if conv_out is None:   # no tiled kernel for this geometry
+            conv_out, stats = F.conv2d(x, w, None, stride, padding), None
+        y, mean, rstd, mask = bn_forward(conv_out, gamma, beta, None, running_mean, running_var, num_batches, momentum,
+                                         eps, relu, stats)
+        ctx.save_for_backward(x, w, conv_out, y if relu and mask is None else None, gamma, mean, rstd, mask)
+        ctx.conf, ctx.relu = (stride, padding), relu
+        ctx.out_link = _adder.BnLink(conv_out, mean, rstd, gamma, relu)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w, conv_out, y, gamma, mean, rstd, mask = ctx.saved_tensors
+        stride, padding = ctx.conf
+        dy = dy.contiguous()
+        link, ctx.out_link = ctx.out_link, None
+        gx = gw = dgamma = dbeta = None
+        if (not ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and link.claims(dy) and link.coef is not None
+                and all(t.data_ptr() % 16 == 0 for t in (x, conv_out, dy))):
+            gw = _adder.conv2d_weight_grad(dy, x, w, stride, padding, out_link=link)   # None: not with this kernel
+            if gw is not None:
+                dgamma, dbeta = link.dgamma, link.dbeta
+        link.dz = None
+        if gw is None:
+            gy, _, dgamma, dbeta = bn_backward(dy, y, mask, conv_out, gamma, mean, rstd, ctx.relu, False)
+            if ctx.needs_input_grad[0]:
+                gx = torch.nn.grad.conv2d_input(x.shape, w, gy, stride, padding)
+            if ctx.needs_input_grad[1]:
+                gw = _adder.conv2d_weight_grad(gy, x, w, stride, padding)
+                if gw is None:
+                    gw = torch.nn.grad.conv2d_weight(x, w.shape, gy, stride, padding)
+        return gx, gw, dgamma, dbeta, None, None, None, None, None, None, None, None
+
+
 class StemConv2d(nn.Conv2d):
     """``nn.Conv2d`` (resnet20.py:49) with the same parameters and state_dict; on the GPU in training its
     weight gradient -- a sum over N*H*W positions into 16 x 27 values, which the vendor library spends six
@@ -121,6 +164,27 @@ class StemConv2d(nn.Conv2d):
         if not plain:
             return super().forward(x)
         return _conv2d_matrix_grad.apply(x, self.weight, self.stride[0], self.padding[0])[0]
+
+    def _plain(self, x):
+        return (x.is_cuda and x.dtype == torch.float32 and self.bias is None and self.groups == 1
+                and self.dilation == (1, 1) and self.padding_mode == "zeros" and torch.is_grad_enabled()
+                and self.stride[0] == self.stride[1] and isinstance(self.padding[0], int)
+                and self.padding[0] == self.padding[1])
+
+    def forward_bn_act(self, x, bn):
+        """``bn(self(x))`` with the ReLU of ``bn`` (a ``BatchNormAct2d``) as one autograd node where that is possible
+        (see ``_conv_bn_act``), else as the separate modules."""
+        if not (self._plain(x) and isinstance(bn, BatchNormAct2d) and bn._fusable(x)):
+            out, stats = self.forward_with_stats(x)
+            return bn(out, stats=stats) if isinstance(bn, BatchNormAct2d) else bn(out)
+        rm = bn.running_mean if bn.track_running_stats else None
+        rv = bn.running_var if bn.track_running_stats else None
+        nb = bn.num_batches_tracked if bn.track_running_stats else None
+        out = _conv_bn_act.apply(x, self.weight, bn.weight.contiguous(), bn.bias.contiguous(), rm, rv, nb, bn.momentum,
+                                 bn.eps, bn.relu, self.stride[0], self.padding[0])
+        if out.grad_fn is not None and hasattr(out.grad_fn, "out_link"):
+            out.grad_fn.out_link.attach(out)
+        return out
 
     def forward_with_stats(self, x):
         """(output, stats) like ``adder2d.forward_with_stats``: the BatchNorm partial sums of the output from the
@@ -177,7 +241,9 @@ class ResNet(nn.Module):
             x = self.avgpool(self.layer3(self.layer2(self.layer1(x))))
             x = self.bn2(self.fc(x))
             return x.view(x.size(0), -1)
-        if self.bn1.training and x.is_cuda and hasattr(self.conv1, "forward_with_stats"):
+        if self.bn1.training and x.is_cuda and hasattr(self.conv1, "forward_bn_act"):
+            x = self.conv1.forward_bn_act(x, self.bn1)
+        elif self.bn1.training and x.is_cuda and hasattr(self.conv1, "forward_with_stats"):
             x, stats = self.conv1.forward_with_stats(x)
             x = self.bn1(x, stats=stats)
         else:

@@ -193,3 +193,21 @@ def test_batched_eta_scaling_with_units(gpu):
     assert torch.equal(grads[0][0], grads[1][0])
     for name in grads[0][1]:
         assert_close(grads[0][1][name], grads[1][1][name], name, rtol=1e-6, atol=1e-7)
+
+
+def test_resnet20_runs_three_batchnorm_backwards_of_its_own(gpu, monkeypatch):
+    """Of the 21 BatchNorms behind convolutions in ResNet-20, 18 have their backward folded into the adder kernels
+    around them (the stem's included); the two downsample BatchNorms (1x1 layers, no such kernels) and the last one
+    (its gradient comes from the pooling layer) run their own two passes."""
+    from addernetcuda_amd import unit, resnet20 as r20
+    calls = []
+    for mod in (unit, r20):
+        real = mod.bn_backward
+        monkeypatch.setattr(mod, "bn_backward", lambda *a, _real=real, **k: (calls.append(1), _real(*a, **k))[1])
+    torch.manual_seed(0)
+    net = r20.resnet20(eta=0.1).to(gpu).train()
+    x = torch.randn(8, 3, 32, 32, device=gpu)
+    F.cross_entropy(net(x), torch.randint(0, 10, (8,), device=gpu)).backward()
+    torch.cuda.synchronize()
+    assert len(calls) == 3
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in net.parameters())
