@@ -37,6 +37,7 @@ import torch.nn.functional as F
 from . import adder as _adder
 from .bn_act import BatchNormAct2d
 from .resnet20 import BasicBlock
+from .unit import adder_bn_act
 
 _conv_bn = BasicBlock._conv_bn   # conv -> BatchNorm (+ residual) (+ ReLU), statistics from the conv's epilogue
 
@@ -172,7 +173,7 @@ class VGGSmall(nn.Module):
                 if isinstance(mods[i], nn.MaxPool2d):
                     x, i = mods[i](x), i + 1
                 else:
-                    x, i = _conv_bn(mods[i], mods[i + 1], x), i + 2   # conv, BatchNorm + ReLU
+                    x, i = adder_bn_act(mods[i], mods[i + 1], x), i + 2   # conv, BatchNorm + ReLU
         return self.classifier(x.reshape(x.size(0), -1))
 
 
@@ -238,7 +239,7 @@ class VGG(nn.Module):
                 if isinstance(mods[i], nn.MaxPool2d):
                     x, i = mods[i](x), i + 1
                 else:
-                    x, i = _conv_bn(mods[i], mods[i + 1], x), i + 3   # adder layer, BatchNorm + ReLU, (ReLU placeholder)
+                    x, i = adder_bn_act(mods[i], mods[i + 1], x), i + 3   # adder layer, BatchNorm + ReLU, (ReLU placeholder)
         return self.classifier(x.view(x.size(0), -1))
 
 

@@ -27,7 +27,7 @@ import torch
 from torch.autograd import Function
 
 from . import adder as _adder
-from ._lib import require_gpu_f32
+from ._lib import require_gpu_f32, bwd_bn_slots
 from .bn_act import BatchNormAct2d, bn_forward, bn_backward
 
 
@@ -45,7 +45,8 @@ class _adder_bn_act(Function):
         ctx.save_for_backward(X, W, conv_out, y if relu and mask is None else None, gamma, mean, rstd, mask)
         ctx.dims, ctx.eta, ctx.relu, ctx.has_res = dims, eta, relu, residual is not None
         ctx.in_link = in_link
-        ctx.out_link = _adder.BnLink(conv_out, mean, rstd, gamma, relu)
+        # (a layer without the kernels that take the link could not use what its consumer would prepare)
+        ctx.out_link = _adder.BnLink(conv_out, mean, rstd, gamma, relu) if bwd_bn_slots(dims) > 0 else None
         ctx.set_materialize_grads(False)
         if with_shortcut:
             # X again, as an output of this node: see adder._adder_nchw.forward
@@ -65,7 +66,7 @@ class _adder_bn_act(Function):
         usable = _adder.bn_links_usable(ctx.dims, X, W, conv_out, dy, grad_short)
         out_link, in_link = ctx.out_link, ctx.in_link
         ctx.out_link = ctx.in_link = None
-        if usable and need_w and out_link.claims(dy) and out_link.coef is not None:
+        if usable and need_w and out_link is not None and out_link.claims(dy) and out_link.coef is not None:
             # dy is dz, written by the consumer's kernel together with this BatchNorm's sums
             gy, dres, dgamma, dbeta = dy, (dy if ctx.has_res else None), out_link.dgamma, out_link.dbeta
         else:
@@ -107,7 +108,7 @@ def adder_bn_act(conv, bn, x, residual=None, with_shortcut=False):
                               bn.momentum, bn.eps, bn.relu, int(conv.stride), int(conv.padding), conv.eta,
                               bool(with_shortcut), _adder.BnLink.of(x))
     out = res[0] if with_shortcut else res
-    link = out.grad_fn.out_link if out.grad_fn is not None and hasattr(out.grad_fn, "out_link") else None
+    link = getattr(out.grad_fn, "out_link", None)
     if link is not None:
         link.attach(out)
     return res

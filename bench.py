@@ -34,8 +34,8 @@ PEAK_VALU_ISSUE = 2 * 256 * 64 * 2.4e9
 BATCH = 256
 ETA = 0.1
 # HBM bytes per launch of the dominant kernel, from the rocprofv3 counter passes kept under profiles/
-# (34.9 MB fetched + 16.8 MB written; cannot be read without the profiler attached)
-DOMINANT_TRAFFIC_BYTES = 51.6e6
+# (54.8 MB fetched + 22.2 MB written; cannot be read without the profiler attached)
+DOMINANT_TRAFFIC_BYTES = 77.0e6
 
 # distinct adder-layer shapes of ResNet-20 at 32x32 input: (count, Ci, H, W, Co, k, stride, pad)
 RESNET20_LAYERS = [
@@ -101,7 +101,7 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
     nx, ny, nw = 4 * x.numel(), 4 * y.numel(), 4 * w.numel()
     # algorithmic HBM bytes of each call: every tensor it reads or writes crosses HBM once
     nbytes = {"fwd": nx + nw + ny, "grad_x": 2 * nx + ny + nw, "grad_w": nx + ny + 2 * nw}
-    keep = (x, w, y, gy, gx, gw, ws)
+    keep = [x, w, y, gy, gx, gw, ws]
     ops = {
         "fwd": lambda: check(lib.adder_conv2d_fwd_f32(ptr(x), ptr(w), ptr(y), *dims, st), "fwd"),
         "grad_x": lambda: check(lib.adder_conv2d_bwd_f32(ptr(gy), ptr(x), ptr(w), ptr(gx), None, 0.0, None, 0,
@@ -109,6 +109,28 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
         "grad_w": lambda: check(lib.adder_conv2d_bwd_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gw), ETA, ptr(ws),
                                                          need.value, *dims, st), "grad_w"),
     }
+    # The calls as the training step makes them for a layer between two BatchNorms (unit.py): grad_W forms the
+    # layer's output gradient from (dz, the layer's output, 4 coefficients per channel) and leaves it in memory,
+    # grad_X reads it, masks its result with x > 0 and leaves the sums of the BatchNorm in front of the layer.
+    from addernetcuda_amd._lib import BnLinks, bwd_bn_slots
+    slots = bwd_bn_slots(dims)
+    if slots > 0:
+        bn_in = torch.randn(N, Ci, H, W, device=dev, generator=g) * 20 - 90
+        mean, rstd = bn_in.mean((0, 2, 3)), 1.0 / bn_in.std((0, 2, 3))
+        part = torch.empty(Ci, slots, 2, dtype=torch.float64, device=dev)
+        coef = torch.randn(Co, 4, device=dev, generator=g) * 0.01
+        yo = torch.randn(N, Co, Ho, Wo, device=dev, generator=g) * 20 - 90
+        gyo = torch.empty_like(gy)
+        lx = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(part), slots, 1)
+        lw = BnLinks(ptr(yo), ptr(coef), ptr(gyo), None, None, None, None, 0, 0)
+        keep += [bn_in, mean, rstd, part, coef, yo, gyo, lx, lw]
+        ops["grad_x_bn"] = lambda: check(lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gx), None, 0.0,
+                                                                      None, 0, *dims, ctypes.byref(lx), st), "grad_x_bn")
+        ops["grad_w_bn"] = lambda: check(lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), None, None, ptr(gw), ETA,
+                                                                      ptr(ws), need.value, *dims, ctypes.byref(lw), st),
+                                         "grad_w_bn")
+        nbytes["grad_x_bn"] = nbytes["grad_x"] + nx + 16 * Ci * slots   # + the BatchNorm's input, + the partial sums
+        nbytes["grad_w_bn"] = nbytes["grad_w"] + 2 * ny                 # + the layer's output, + the formed gradient
     return E, ops, keep, nbytes
 
 
@@ -119,7 +141,7 @@ def bench_layers(dev, warmup=5, iters=20, which="resnet20"):
         E, ops, keep, nbytes = layer_ops(batch, Ci, H, W, Co, k, s, p, dev)
         for name, fn in ops.items():
             t = event_time(fn, warmup, iters)
-            flop, slots = OPS[name]
+            flop, slots = OPS[name[:-3] if name.endswith("_bn") else name]
             row = {
                 "layer": f"{Ci}->{Co} k{k} s{s} p{p} @{H}x{W}", "count": cnt, "op": name, "us": round(t * 1e6, 2),
                 "tflops": round(flop * E / t / 1e12, 2),
@@ -127,7 +149,7 @@ def bench_layers(dev, warmup=5, iters=20, which="resnet20"):
                 "hbm_gbs": round(nbytes[name] / t / 1e9, 1),
                 "frac_hbm_peak": round(nbytes[name] / t / 1e9 / PEAK_HBM_GBS, 4),
             }
-            if name == "grad_w" and k == 3:   # fp64 matrix-core kernel (+ finalize and scaling launches)
+            if name in ("grad_w", "grad_w_bn") and k == 3:   # fp64 matrix-core kernel (+ finalize and scaling launches)
                 row["frac_fp64_mfma_peak"] = round(2 * E / t / 1e12 / PEAK_FP64_MFMA_TFLOPS, 4)
             else:
                 row["valu_issue_util"] = round(slots * E / t / PEAK_VALU_ISSUE, 4)
@@ -173,26 +195,35 @@ def bench_col(dev, warmup=3, iters=10):
 
 
 def dominant_kernel(dev, steps):
-    """grad_x of the 16->16 3x3 @32x32 layer: the kernel with the largest share of a training step."""
+    """grad_x of the 16->16 3x3 @32x32 layer, as the training step launches it (with the statistics of the
+    BatchNorm in front of the layer in its epilogue): the kernel with the largest share of a training step.
+    `plain_kernel` repeats the figures for the same kernel without that epilogue (adder_conv2d_bwd_f32)."""
     cnt, Ci, H, W, Co, k, s, p = RESNET20_LAYERS[0]
-    E, ops, keep, _ = layer_ops(BATCH, Ci, H, W, Co, k, s, p, dev)
-    t = event_time(ops["grad_x"], 5, max(20, steps))
+    E, ops, keep, nbytes = layer_ops(BATCH, Ci, H, W, Co, k, s, p, dev)
+    t = event_time(ops["grad_x_bn"], 5, max(20, steps))
+    t_plain = event_time(ops["grad_x"], 5, max(20, steps))
     flop = OPS["grad_x"][0] * E
     achieved = flop / t / 1e12
     return {
-        "bound": "valu", "kernel": "adder::grad_x_3x3s1_kernel (16->16, 3x3 s1 p1, 32x32, batch 256)",
+        "plain_kernel": {"avg_launch_us": round(t_plain * 1e6, 2), "achieved": round(flop / t_plain / 1e12, 2),
+                         "frac": round(flop / t_plain / 1e12 / PEAK_FP32_TFLOPS, 4),
+                         "algorithmic_bytes": nbytes["grad_x"]},
+        "bound": "valu", "kernel": "adder::grad_x_3x3s1_kernel<..., FUSE = true> (16->16, 3x3 s1 p1, 32x32, batch 256; "
+                                   "masks its result and sums it for the BatchNorm in front of the layer)",
         "achieved": round(achieved, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_FP32_TFLOPS, 4), "traffic": DOMINANT_TRAFFIC_BYTES,
         "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy: "
                           "profiles/grad_x_3x3s1_resnet20_16to16_32x32_bs256.md",
-        "algorithmic_bytes": 4 * (2 * BATCH * Ci * H * W + BATCH * Co * H * W + Co * Ci * k * k),
+        "algorithmic_bytes": nbytes["grad_x_bn"],
         "avg_launch_us": round(t * 1e6, 2), "flop_per_launch": flop,
         "valu_issue_util": round(OPS["grad_x"][1] * E / t / PEAK_VALU_ISSUE, 4),
         "note": "fp32 VALU-bound (|a-b| accumulation has no FMA/MFMA form). The 157.3 TFLOP/s peak needs an FMA "
                 "in each of the two vector issue slots a SIMD has per 4 cycles; this op spends 2 instructions "
                 "(v_fma with the clamp modifier, v_fmac) on the 4 flop of a term (sub, clamp, mul, add), so the "
                 "peak itself is its ceiling. valu_issue_util is the share of the two-slot issue rate taken by "
-                "those 2 instructions per term.",
+                "those 2 instructions per term. The flop count is the adder layer's alone: the epilogue (mask, two "
+                "sums per channel, one more tensor read) is the first pass of a BatchNorm backward that no longer "
+                "runs as a kernel of its own.",
     }
 
 
@@ -284,7 +315,9 @@ def graph_matches_eager(dev, replays=4, which="resnet20", fused=True):
 
 def layer_set_summary(rows):
     """Adder-kernel time per training step of a layer set and the flop-weighted fraction of the fp32 vector peak
-    over all of its adder kernels (forward 2, grad_X 4, grad_W 3 flop per term)."""
+    over all of its adder kernels (forward 2, grad_X 4, grad_W 3 flop per term), from the rows of the plain entry
+    points (the *_bn rows time the same layers' backward calls with the BatchNorm links)."""
+    rows = [r for r in rows if not r["op"].endswith("_bn")]
     t = sum(r["us"] * r["count"] for r in rows) * 1e-6
     flop = sum(r["tflops"] * 1e12 * r["us"] * 1e-6 * r["count"] for r in rows)
     return {"adder_kernel_ms_per_step": round(t * 1e3, 3), "adder_kernels_tflops": round(flop / t / 1e12, 2),
@@ -442,9 +475,10 @@ def main():
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ResNet-20 AdderNet, batch 256, 3x32x32, 10 classes, SGD momentum 0.9 lr 0.1 wd 5e-4, "
                                "adaptive eta 0.1, fwd+bwd+optimizer; BatchNorm / ReLU / residual add run as this "
-                               "library's fused kernels (BatchNormAct2d) and the regular 3->16 stem convolution "
-                               "through the tiled forward / slab weight-gradient kernels (StemConv2d); the same step "
-                               "with stock torch modules is other_configs[0]",
+                               "library's fused kernels (BatchNormAct2d), the BatchNorm backward passes inside the "
+                               "adder backward kernels on either side of each BatchNorm (unit.py), and the regular "
+                               "3->16 stem convolution through the tiled forward / slab weight-gradient kernels "
+                               "(StemConv2d); the same step with stock torch modules is other_configs[0]",
                    "step_mode": mode},
         "images_per_s": round(BATCH / ms * 1e3, 1),
         "roofline": dominant_kernel(dev, args.steps),
