@@ -423,13 +423,13 @@ int launch_grad_w_mfma_bf16(const bf16_t *gy, const bf16_t *x, double *part, dou
     }
 }
 
-// The 3x3 / pad-1 variants with gy formed from (dz = gy, bn_y, bn_coef) while it is staged and left in gy_out
-// (nullable) on the way (see gy_commit_m_bn); ADDER_ERR_UNSUPPORTED for other variants and for rows that are not
-// whole float4 groups.
+// The 3x3 / pad-1 and the stride-1 1x1 variants with gy formed from (dz = gy, bn_y, bn_coef) while it is staged and
+// left in gy_out (nullable) on the way (see gy_commit_m_bn); ADDER_ERR_UNSUPPORTED for other variants and for rows
+// (planes, for 1x1 layers) that are not whole float4 groups.
 int launch_grad_w_mfma_bn(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
                           const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s) {
-    if (d.W % 4 != 0 || d.Wo % 4 != 0) return ADDER_ERR_UNSUPPORTED;
     const Subsample none{1, 0, 0, 0};
+    if (p.variant >= 1 && p.variant <= 5 && (d.W % 4 != 0 || d.Wo % 4 != 0)) return ADDER_ERR_UNSUPPORTED;
     switch (p.variant) {
         case 1: return launch_one_v<GmW32, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
                                                                            gy_out);
@@ -441,6 +441,16 @@ int launch_grad_w_mfma_bn(const float *gy, const float *x, double *part, double 
                                                                            gy_out);
         case 5: return launch_one_v<GmW8S2, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
                                                                            gy_out);
+        default: break;
+    }
+    // 1x1 stride-1 layers: whole planes as rows
+    const ConvDims f = mfma_one_row(d);
+    if (d.stride != 1 || f.W % 4 != 0) return ADDER_ERR_UNSUPPORTED;
+    switch (p.variant) {
+        case 6: return launch_one_v<Gm1x1, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
+        case 7: return launch_one_v<Gm1x1s, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
+        case 10: return launch_one_v<Gm1x1b, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
+        case 12: return launch_one_v<Gm1x1c, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
         default: return ADDER_ERR_UNSUPPORTED;
     }
 }

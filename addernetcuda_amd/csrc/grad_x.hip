@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const T *__restrict
 // T: storage type of gy, x, gx and gadd (float, or bf16_t for the reduced-storage mode).
 // FUSE: the statistics pass of the backward of the BatchNorm in front of the layer is done here (the in_* fields
 // of adder_bn_links): the result is masked with x > 0 (bn.in_relu) and its per-channel sums are left in
-// bn.in_part, (Ci, gridDim.x * POSW, 2) doubles.  3x3 taps, float storage, rows of whole float4 groups.
+// bn.in_part, (Ci, gridDim.x * POSW, 2) doubles.  Float storage, rows of whole float4 groups, no sampling.
 template <class C, bool VEC = true, bool SAT = true, bool SUB = false, class T = float, bool FUSE = false>
 __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *__restrict__ gy,
                                                                    const T *__restrict__ x,
@@ -109,8 +109,8 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
                                                                    const T *__restrict__ gadd,
                                                                    const adder_bn_links bn) {
     static_assert(!SUB || C::KS == 1, "sampling is for single-tap layers");
-    static_assert(!FUSE || (C::KS == 3 && VEC && !SUB && sizeof(T) == 4 && C::TM * C::TN <= 32),
-                  "the BatchNorm link belongs to the float 3x3 kernels");
+    static_assert(!FUSE || (VEC && !SUB && sizeof(T) == 4 && C::TM * C::TN <= 32),
+                  "the BatchNorm link belongs to the float kernels that read whole rows");
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
 
@@ -482,7 +482,7 @@ static int launch_grad_x_3x3s1_v(const T *gy, const T *x, const float *w, T *gx,
 template <class C>
 static int launch_grad_x_3x3s1_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                                   hipStream_t s, const float *gadd, const adder_bn_links &bn) {
-    if (d.Co * C::KK > kSatMaxTerms)
+    if (d.Co * C::KK > (C::KS == 1 ? kSatMaxTerms1x1 : kSatMaxTerms))
         return launch_grad_x_3x3s1_v<C, true, false, false, float, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd, bn);
     return launch_grad_x_3x3s1_v<C, true, true, false, float, true>(gy, x, w, gx, d, s, Subsample{1, 0, 0, 0}, gadd, bn);
 }
@@ -908,9 +908,22 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
     return check_launch();
 }
 
-// Which tiled kernel carries the BatchNorm link for this layer: 1 GxW32, 2 GxW16, 3 GxW8 (stride 1), 4 GxS2W32,
-// 5 GxS2W16 (stride 2); 0: none (other kernel sizes, rows that are not whole float4 groups, fewer than TM channels).
+// a 1x1 stride-1 layer seen as images of one row of H * W positions
+static ConvDims one_row(const ConvDims &d) {
+    ConvDims f = d;
+    f.H = f.Ho = 1;
+    f.W = f.Wo = d.H * d.W;
+    return f;
+}
+
+// Which tiled kernel carries the BatchNorm link for this layer: 1 GxW32, 2 GxW16, 3 GxW8 (3x3 stride 1), 4 GxS2W32,
+// 5 GxS2W16 (3x3 stride 2), 6 Gx1x1, 7 Gx1x1t, 8 Gx1x1s (1x1 stride 1 from 64 input / 48 output channels); 0: none
+// (other kernel sizes, rows or planes that are not whole float4 groups, too few channels).
 static int grad_x_bn_variant(const ConvDims &d) {
+    if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 48 && (d.H * d.W) % 4 == 0) {
+        const ConvDims f = one_row(d);
+        return f.W > 64 ? 6 : (small_plane_tile(f) ? 7 : 8);
+    }
     if (d.kh != 3 || d.kw != 3 || d.pad != 1 || d.Ci < GxW32::TM) return 0;
     if (d.stride == 1 && d.W % 4 == 0) return d.W > 16 ? 1 : (d.W > 8 ? 2 : 3);
     if (d.stride == 2 && d.W % 4 == 0 && d.Wo % 4 == 0) return d.W > 16 ? 4 : 5;
@@ -930,6 +943,9 @@ int grad_x_bn_slots(const ConvDims &d) {
         case 3: return bn_slots_of<GxW8>(d);
         case 4: return bn_slots_of<GxS2W32>(d);
         case 5: return bn_slots_of<GxS2W16>(d);
+        case 6: return bn_slots_of<Gx1x1>(one_row(d));
+        case 7: return bn_slots_of<Gx1x1t>(one_row(d));
+        case 8: return bn_slots_of<Gx1x1s>(one_row(d));
         default: return 0;
     }
 }
@@ -947,6 +963,9 @@ int launch_grad_x_bn(const float *gy, const float *x, const float *w, float *gx,
         case 3: return launch_grad_x_3x3s1_bn<GxW8>(gy, x, w, gx, d, s, gadd, bn);
         case 4: return launch_grad_x_3x3s2_bn<GxS2W32>(gy, x, w, gx, d, s, gadd, bn);
         case 5: return launch_grad_x_3x3s2_bn<GxS2W16>(gy, x, w, gx, d, s, gadd, bn);
+        case 6: return launch_grad_x_3x3s1_bn<Gx1x1>(gy, x, w, gx, one_row(d), s, gadd, bn);
+        case 7: return launch_grad_x_3x3s1_bn<Gx1x1t>(gy, x, w, gx, one_row(d), s, gadd, bn);
+        case 8: return launch_grad_x_3x3s1_bn<Gx1x1s>(gy, x, w, gx, one_row(d), s, gadd, bn);
         default: return ADDER_ERR_UNSUPPORTED;
     }
 }

@@ -36,10 +36,7 @@ import torch.nn.functional as F
 
 from . import adder as _adder
 from .bn_act import BatchNormAct2d
-from .resnet20 import BasicBlock
 from .unit import adder_bn_act
-
-_conv_bn = BasicBlock._conv_bn   # conv -> BatchNorm (+ residual) (+ ReLU), statistics from the conv's epilogue
 
 
 def _bn(channels, relu, fused):
@@ -73,16 +70,15 @@ class Bottleneck(nn.Module):
                 identity = self.downsample(x)
             out = out + identity
             return self.relu(out)
-        if self.bn1.training and x.is_cuda and x.requires_grad and hasattr(self.conv1, "forward_with_stats"):
-            # the shortcut leaves through conv1's autograd node, see BasicBlock.forward
-            out, stats, shortcut = self.conv1.forward_with_stats(x, with_shortcut=True)
-            out = self.bn1(out, stats=stats)
+        # every conv -> bn (-> + shortcut) -> relu group is one autograd node (unit.py), see BasicBlock.forward
+        if self.bn1.training and x.is_cuda and x.requires_grad:
+            out, shortcut = adder_bn_act(self.conv1, self.bn1, x, with_shortcut=True)
         else:
-            out, shortcut = _conv_bn(self.conv1, self.bn1, x), x
-        out = _conv_bn(self.conv2, self.bn2, out)
+            out, shortcut = adder_bn_act(self.conv1, self.bn1, x), x
+        out = adder_bn_act(self.conv2, self.bn2, out)
         if self.downsample is not None:
-            shortcut = _conv_bn(self.downsample[0], self.downsample[1], shortcut)
-        return _conv_bn(self.conv3, self.bn3, out, shortcut)       # bn + residual + relu
+            shortcut = adder_bn_act(self.downsample[0], self.downsample[1], shortcut)
+        return adder_bn_act(self.conv3, self.bn3, out, residual=shortcut)       # bn + residual + relu
 
 
 class ResNet50(nn.Module):

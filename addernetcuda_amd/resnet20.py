@@ -39,14 +39,6 @@ class BasicBlock(nn.Module):
         self.downsample = downsample
         self.stride = stride
 
-    @staticmethod
-    def _conv_bn(conv, bn, x, residual=None):
-        # the adder kernels sum their output per channel on the way out, which saves the BatchNorm its own pass
-        if bn.training and hasattr(conv, "forward_with_stats") and x.is_cuda:
-            out, stats = conv.forward_with_stats(x)
-            return bn(out, residual=residual, stats=stats)
-        return bn(conv(x), residual=residual)
-
     def forward(self, x):
         if not self.fused:   # the module sequence of resnet20.py:28-39, stock torch modules around the adder layers
             residual = x

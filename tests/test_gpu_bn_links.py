@@ -16,21 +16,30 @@ from tests.util import assert_close
 
 pytestmark = pytest.mark.gpu
 
-# (N, Ci, H, W, Co, stride)
+# (N, Ci, H, W, Co, stride[, kernel size = 3]); 3x3 layers have pad 1, 1x1 layers pad 0
 CASES = [(8, 16, 32, 32, 16, 1), (6, 16, 32, 32, 32, 2), (8, 32, 16, 16, 32, 1), (8, 32, 16, 16, 64, 2),
          (8, 64, 8, 8, 64, 1), (3, 20, 16, 16, 24, 1), (5, 12, 32, 32, 40, 1), (3, 6, 24, 40, 9, 2),
-         (2, 5, 12, 20, 3, 1), (4, 8, 8, 8, 260, 1)]   # the last one: the three-instruction grad_X form (2340 terms)
+         (2, 5, 12, 20, 3, 1), (4, 8, 8, 8, 260, 1),   # the last one: the three-instruction grad_X form (2340 terms)
+         # 1x1 layers: planes of 196 and 784 positions, planes of 64 (few and many workgroups), 128-channel blocks
+         (4, 64, 14, 14, 256, 1, 1), (2, 256, 28, 28, 64, 1, 1), (8, 64, 8, 8, 64, 1, 1), (40, 72, 8, 8, 64, 1, 1),
+         (3, 128, 8, 8, 128, 1, 1), (2, 128, 14, 14, 136, 1, 1), (2, 64, 6, 6, 1100, 1, 1)]
+
+
+def _geom(case):
+    N, Ci, H, W, Co, s = case[:6]
+    k = case[6] if len(case) > 6 else 3
+    return N, Ci, H, W, Co, s, k, k // 2
 
 
 def _make(case, seed):
-    N, Ci, H, W, Co, s = case
+    N, Ci, H, W, Co, s, k, pad = _geom(case)
     g = torch.Generator().manual_seed(seed)
     xp = torch.randn(N, Ci, H, W, generator=g) * 20 - 90            # an adder layer's output: large negative mean
     res = torch.randn(N, Ci, H, W, generator=g)
     gamma_p = torch.rand(Ci, generator=g) + 0.5
     beta_p = torch.randn(Ci, generator=g) * 0.3
-    w = torch.randn(Co, Ci, 3, 3, generator=g) * 0.5
-    Ho, Wo = (H - 1) // s + 1, (W - 1) // s + 1
+    w = torch.randn(Co, Ci, k, k, generator=g) * 0.5
+    Ho, Wo = (H - k + 2 * pad) // s + 1, (W - k + 2 * pad) // s + 1
     dzq = torch.randn(N, Co, Ho, Wo, generator=g)
     dzq = dzq * (torch.rand(dzq.shape, generator=g) > 0.4)          # a ReLU-masked gradient
     gamma_q = torch.rand(Co, generator=g) + 0.5
@@ -58,9 +67,9 @@ def _bn_input_grad(dz, x, gamma, mean, rstd):
 def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, gpu):
     from addernetcuda_amd._lib import lib, check, ptr, stream_ptr, BnLinks, bwd_bn_slots, conv_dims, conv2d_bwd_workspace
     from oracle import adder_oracle
-    N, Ci, H, W, Co, s = case
+    N, Ci, H, W, Co, s, k, pad = _geom(case)
     xp, res, gamma_p, beta_p, w, dzq, gamma_q, gx_add = _make(case, 17 + sum(case))
-    dims, Ho, Wo = conv_dims((N, Ci, H, W), w.shape, s, 1)
+    dims, Ho, Wo = conv_dims((N, Ci, H, W), w.shape, s, pad)
     slots = bwd_bn_slots(dims)
     assert slots > 0
 
@@ -70,13 +79,13 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, gpu
     # x as float32 would hold it (the kernels read the float32 tensor, and its sign is the ReLU gate)
     mean_p32, rstd_p32 = mean_p.float(), rstd_p.float()
     x = torch.relu((xp - b(mean_p32)) * b(rstd_p32 * gamma_p) + b(beta_p) + res)
-    y = adder_oracle.conv2d_forward(x.double(), w.double(), s, 1)
+    y = adder_oracle.conv2d_forward(x.double(), w.double(), s, pad)
     y32 = y.float()
     mean_q, rstd_q = _stats(y32.double())
     mean_q32, rstd_q32 = mean_q.float(), rstd_q.float()
     gy, dgamma_q, dbeta_q = _bn_input_grad(dzq.double(), y32.double(), gamma_q.double(), mean_q32.double(),
                                            rstd_q32.double())
-    gx, gw_raw, gw_scaled = adder_oracle.conv2d_backward(gy, x.double(), w.double(), s, 1, 0.2)
+    gx, gw_raw, gw_scaled = adder_oracle.conv2d_backward(gy, x.double(), w.double(), s, pad, 0.2)
     if with_add:
         gx = gx + gx_add.double()
     dz = gx * (x > 0)
@@ -142,13 +151,14 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, gpu
     assert torch.equal(gx2, gxg)
 
 
-@pytest.mark.parametrize("case", [(8, 16, 32, 32, 16, 1), (8, 32, 16, 16, 64, 2), (3, 20, 16, 16, 24, 1)], ids=str)
+@pytest.mark.parametrize("case", [(8, 16, 32, 32, 16, 1), (8, 32, 16, 16, 64, 2), (3, 20, 16, 16, 24, 1),
+                                  (4, 64, 14, 14, 96, 1, 1)], ids=str)
 def test_each_half_of_the_links_alone(case, gpu):
     """Only in-links (a plain gy) against the library's own unfused kernels, with and without the ReLU gate."""
     from addernetcuda_amd._lib import lib, check, ptr, stream_ptr, BnLinks, bwd_bn_slots, conv_dims, conv2d_bwd_workspace
-    N, Ci, H, W, Co, s = case
+    N, Ci, H, W, Co, s, k, pad = _geom(case)
     xp, res, gamma_p, beta_p, w, dzq, gamma_q, gx_add = _make(case, 5 + sum(case))
-    dims, Ho, Wo = conv_dims((N, Ci, H, W), w.shape, s, 1)
+    dims, Ho, Wo = conv_dims((N, Ci, H, W), w.shape, s, pad)
     slots = bwd_bn_slots(dims)
     st = stream_ptr(gpu)
     d = lambda t: t.to(gpu).contiguous()
@@ -183,7 +193,11 @@ def test_each_half_of_the_links_alone(case, gpu):
 def test_refusals(gpu):
     from addernetcuda_amd._lib import lib, ptr, stream_ptr, BnLinks, bwd_bn_slots, conv_dims
     dims, _, _ = conv_dims((2, 16, 8, 8), (16, 16, 1, 1), 1, 0)
-    assert bwd_bn_slots(dims) == 0                       # no fused kernels for 1x1 layers
+    assert bwd_bn_slots(dims) == 0                       # no fused kernels for 1x1 layers with fewer than 64 channels
+    dims49, _, _ = conv_dims((2, 64, 7, 7), (64, 64, 1, 1), 1, 0)
+    assert bwd_bn_slots(dims49) == 0                     # ... nor for planes that are not whole groups of four
+    dims_s2, _, _ = conv_dims((2, 64, 8, 8), (64, 64, 1, 1), 2, 0)
+    assert bwd_bn_slots(dims_s2) == 0                    # ... nor for strided 1x1 layers
     dims7, _, _ = conv_dims((2, 16, 7, 7), (16, 16, 3, 3), 1, 1)
     assert bwd_bn_slots(dims7) == 0                      # rows that are not whole groups of four
     t = torch.zeros(2 * 16 * 8 * 8, device=gpu)
