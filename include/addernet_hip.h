@@ -289,7 +289,8 @@ ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsign
  *                      BatchNorm's input (N, Ci, H, W), its saved mean / rstd (Ci); in_part receives
  *                      (Ci, in_slots, 2) doubles, in_slots = adder_conv2d_bwd_bn_slots; gx receives dz.
  *   adder_conv2d_bwd_bn_slots: partial-sum slots per channel for in_part; 0 = this layer has no such kernels
- *     (they exist for 3x3 / pad 1 / stride 1 or 2 layers whose rows are whole groups of four floats).
+ *     (they exist for 3x3 / pad 1 / stride 1 or 2 layers whose rows are whole groups of four floats, and for 1x1 /
+ *     stride 1 layers with at least 64 input and output channels whose planes are whole groups of four floats).
  *   adder_conv2d_bwd_bn_f32: adder_conv2d_bwd_add_f32 (gx_add nullable here) with the links.  With the out_*
  *     half gw must be requested (the grad_W kernel is the one that forms gy); a caller that stages grad_W
  *     (adder_conv2d_grad_w_staged_bn_f32) calls this afterwards with gy = its out_gy and without the out_* half.
