@@ -89,11 +89,19 @@ __global__ __launch_bounds__(256) void grad_w_generic_kernel(const ST *__restric
 // chain is slots/kFinLanes long.
 // ---------------------------------------------------------------------------
 static constexpr int kFinOut = 16, kFinLanes = 16;   // a wave reads four full 64-byte runs per slot row
+static constexpr int kFinThreads = kFinOut * kFinLanes;
+// The batched finalize picks the block shape per layer: layers with few slabs give a workgroup more outputs (32 x 8
+// or 64 x 4 threads), so that every thread still has a few loads in flight and a layer with 16 slabs does not need
+// four times the workgroups of one with 256.
+__host__ __device__ inline int fin_out_for(int slots) { return slots >= 128 ? 16 : (slots >= 32 ? 32 : 64); }
 // ACC: the result is added to gw (the column-matrix entry points accumulate, as the reference's atomicAdd does).
+// fo: outputs per workgroup (16, 32 or 64); kFinThreads / fo threads share the slots of an output.
 template <typename PT, bool ACC = false>
 __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ part, const PT *__restrict__ sgpart,
                                                       const float *__restrict__ w, float *__restrict__ gw,
-                                                      double *__restrict__ ss, int slots, int Co, int K, int block) {
+                                                      double *__restrict__ ss, int slots, int Co, int K, int block,
+                                                      const int fo = kFinOut) {
+    const int kFinOut = fo, kFinLanes = kFinThreads / fo;   // (the names of the fixed shape, for this workgroup's)
     const int o = threadIdx.x % kFinOut, sl = threadIdx.x / kFinOut;
     const int total = Co * K;
     const int idx = block * kFinOut + o;
@@ -117,14 +125,13 @@ __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ par
         s4[0] += (double)sgpart[(size_t)p * Co + co];
     }
     const double a = (a4[0] + a4[1]) + (a4[2] + a4[3]), sgs = (s4[0] + s4[1]) + (s4[2] + s4[3]);
-    __shared__ double ra[kFinLanes][kFinOut + 1], rs[kFinLanes][kFinOut + 1];
-    ra[sl][o] = a;
-    rs[sl][o] = sgs;
+    __shared__ double ra[kFinThreads + 16], rs[kFinThreads + 16];   // [lane][output], rows one element apart in banks
+    ra[sl * (kFinOut + 1) + o] = a;
+    rs[sl * (kFinOut + 1) + o] = sgs;
     __syncthreads();
     if (threadIdx.x < kFinOut) {
         double ta = 0.0, ts = 0.0;
-#pragma unroll 8
-        for (int k = 0; k < kFinLanes; ++k) { ta += ra[k][o]; ts += rs[k][o]; }
+        for (int k = 0; k < kFinLanes; ++k) { ta += ra[k * (kFinOut + 1) + o]; ts += rs[k * (kFinOut + 1) + o]; }
         double v = 0.0;
         if (idx < total) {
             float r = (float)(w ? ta - (double)w[idx] * ts : ta);   // no weights: the plain sum of x * gy
@@ -132,7 +139,6 @@ __device__ __forceinline__ void grad_w_finalize_block(const PT *__restrict__ par
             gw[idx] = r;
             v = (double)r * (double)r;
         }
-#pragma unroll
         for (int off = kFinOut / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
         if (threadIdx.x == 0 && ss) ss[block] = v;
     }
@@ -145,13 +151,13 @@ __global__ __launch_bounds__(kFinOut * kFinLanes) void grad_w_finalize_kernel(co
                                                                               float *__restrict__ gw,
                                                                               double *__restrict__ ss, int slots,
                                                                               int Co, int K) {
-    grad_w_finalize_block<PT, ACC>(part, sgpart, w, gw, ss, slots, Co, K, blockIdx.x);
+    grad_w_finalize_block<PT, ACC>(part, sgpart, w, gw, ss, slots, Co, K, blockIdx.x, fin_out_for(slots));
 }
 
 // gw (+)= sum of `slots` fp64 slabs - w * sum of the gy partials: the finalize on its own, for the column-matrix path
 int launch_grad_w_slab_finalize(const double *part, const double *sgpart, const float *w, float *gw, int slots, int Co,
                                 int K, bool accumulate, hipStream_t s) {
-    const int nb = (int)ceil_div_l((long)Co * K, kFinOut);
+    const int nb = (int)ceil_div_l((long)Co * K, fin_out_for(slots));
     if (accumulate)
         hipLaunchKernelGGL((grad_w_finalize_kernel<double, true>), dim3(nb), dim3(kFinOut * kFinLanes), 0, s, part, sgpart,
                            w, gw, nullptr, slots, Co, K);
@@ -178,12 +184,13 @@ __global__ __launch_bounds__(kFinOut * kFinLanes) void batch_finalize_kernel(con
     const adder_grad_w_stage &it = b.it[t];
     const int block = blockIdx.x - b.first[t];
     double *mine = ss + b.first[t];
+    const int fo = fin_out_for(it.slots);
     if (it.fp64)
         grad_w_finalize_block<double>(static_cast<const double *>(it.part), static_cast<const double *>(it.sgpart), it.w,
-                                      it.gw, mine, it.slots, it.Co, it.K, block);
+                                      it.gw, mine, it.slots, it.Co, it.K, block, fo);
     else
         grad_w_finalize_block<float>(static_cast<const float *>(it.part), static_cast<const float *>(it.sgpart), it.w,
-                                     it.gw, mine, it.slots, it.Co, it.K, block);
+                                     it.gw, mine, it.slots, it.Co, it.K, block, fo);
 }
 
 __global__ __launch_bounds__(256) void batch_finish_scale_kernel(const GwStageBatch b, const double *__restrict__ ss,
@@ -389,7 +396,7 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
     const int K = d.K();
     const long n = (long)d.Co * K;
     if (p.variant) {
-        const int nb = (int)ceil_div_l(n, kFinOut);
+        const int nb = (int)ceil_div_l(n, fin_out_for(p.slots));
         const bool fused_norm = eta > 0.f && nb <= kNormBlocksMax;
         int rc;
         if (p.variant == 2) {
@@ -445,7 +452,7 @@ int launch_grad_w_bf16(const bf16_t *gy, const bf16_t *x, const float *w, float 
         double *part = reinterpret_cast<double *>(ss + kNormBlocksMax);
         double *sgpart = part + (size_t)p.slots * d.Co * K;
         if (int rc = launch_grad_w_mfma_bf16(gy, x, part, sgpart, d, p.mfma, s)) return rc;
-        const int nb = (int)ceil_div_l(n, kFinOut);
+        const int nb = (int)ceil_div_l(n, fin_out_for(p.slots));
         hipLaunchKernelGGL(grad_w_finalize_kernel<double>, dim3(nb), dim3(kFinOut * kFinLanes), 0, s, part, sgpart, w, gw,
                            nullptr, p.slots, d.Co, K);
     } else {
@@ -506,7 +513,7 @@ int launch_grad_w_staged(const float *gy, const float *x, const float *w, float 
 
 static long finish_blocks(int count, const adder_grad_w_stage *st) {
     long total = 0;
-    for (int t = 0; t < count; ++t) total += ceil_div(st[t].Co * st[t].K, kFinOut);
+    for (int t = 0; t < count; ++t) total += ceil_div(st[t].Co * st[t].K, fin_out_for(st[t].slots));
     return total;
 }
 
@@ -520,7 +527,7 @@ int launch_grad_w_finish(int count, const adder_grad_w_stage *st, void *ws, hipS
     b.count = count;
     for (int t = 0; t < count; ++t) {
         b.it[t] = st[t];
-        b.first[t + 1] = b.first[t] + ceil_div(st[t].Co * st[t].K, kFinOut);
+        b.first[t + 1] = b.first[t] + ceil_div(st[t].Co * st[t].K, fin_out_for(st[t].slots));
         const long n = (long)st[t].Co * st[t].K;
         most_n = n > most_n ? n : most_n;
     }
