@@ -168,11 +168,14 @@ class BnLink:
     and the partial sums of the BatchNorm's backward, a small kernel turns those into ``coef`` / ``dgamma`` /
     ``dbeta``, and the node of the BatchNorm, when it is handed exactly that ``dz`` tensor, skips its own two
     passes."""
-    __slots__ = ("bn_x", "mean", "rstd", "gamma", "relu", "out_ptr", "out_shape", "out_version", "dz", "dz_version",
-                 "coef", "dgamma", "dbeta")
+    __slots__ = ("bn_x", "mean", "rstd", "gamma", "beta", "beta_version", "relu", "out_ptr", "out_shape", "out_version", "dz",
+                 "dz_version", "coef", "dgamma", "dbeta")
 
-    def __init__(self, bn_x, mean, rstd, gamma, relu):
-        self.bn_x, self.mean, self.rstd, self.gamma, self.relu = bn_x, mean, rstd, gamma, relu
+    def __init__(self, bn_x, mean, rstd, gamma, relu, beta=None):
+        """``beta``: the BatchNorm's bias, given only when nothing was added to the BatchNorm's output (no residual):
+        the consumer's kernel can then recover xhat from its own input instead of reading ``bn_x``."""
+        self.bn_x, self.mean, self.rstd, self.gamma, self.beta, self.relu = bn_x, mean, rstd, gamma, beta, relu
+        self.beta_version = None if beta is None else (beta._version, gamma._version)
         self.out_ptr = self.out_shape = self.out_version = None
         self.dz = self.dz_version = self.coef = self.dgamma = self.dbeta = None
 
@@ -225,6 +228,8 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
             part = torch.empty((X.size(1), slots, 2), device=dev, dtype=torch.float64)
             links.in_x, links.in_mean, links.in_rstd = ptr(in_link.bn_x), ptr(in_link.mean), ptr(in_link.rstd)
             links.in_part, links.in_slots, links.in_relu = ptr(part), slots, int(in_link.relu)
+            if in_link.beta is not None and in_link.beta_version == (in_link.beta._version, in_link.gamma._version):
+                links.in_gamma, links.in_beta = ptr(in_link.gamma), ptr(in_link.beta)
     if _eta_batch is not None and need_w and any(W is entry[0] for entry in _eta_batch):
         raise RuntimeError("batched_eta_scaling: this weight already has a pending gradient in the block "
                            "(one backward pass per block, no weight shared between layers)")

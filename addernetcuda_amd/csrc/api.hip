@@ -398,6 +398,7 @@ int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, con
     if ((bn.out_x == nullptr) != (bn.out_coef == nullptr) || (bn.out_gy && !bn.out_x)) return ADDER_ERR_NULL_POINTER;
     if (bn.out_x && gx && !bn.out_gy) return ADDER_ERR_NULL_POINTER;   // grad_X reads the gradient grad_W leaves there
     if (bn.in_part && (!bn.in_x || !bn.in_mean || !bn.in_rstd || !gx)) return ADDER_ERR_NULL_POINTER;
+    if ((bn.in_gamma == nullptr) != (bn.in_beta == nullptr)) return ADDER_ERR_NULL_POINTER;
     ConvDims d;
     if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
     const int slots = grad_w_bn_supported(d, nullptr, nullptr, nullptr, nullptr) ? grad_x_bn_slots(d) : 0;

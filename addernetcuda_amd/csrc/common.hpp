@@ -157,6 +157,26 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// The same sum for a caller that needs it in one lane only: the row sums travel on with two row broadcasts
+// (lane 15 of each row into the next row, lane 31 into the upper half) instead of through scalar registers.
+// The result is valid in lanes 48..63.
+__device__ __forceinline__ float wave_sum_top_row(float v) {
+    int t;
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true);   // row_half_mirror
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true);   // row_mirror
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1, 3
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2, 3
+    v += __int_as_float(t);
+    return v;
+}
+
 struct ConvDims {
     int N, Ci, H, W, Co, kh, kw, stride, pad, Ho, Wo;
     __host__ __device__ int K() const { return Ci * kh * kw; }

@@ -338,22 +338,34 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
     // keep their sixteen 64-bit addresses in registers through the whole main loop.  Rows are whole strips here; a
     // strip beyond the row (a tile wider than the tensor) reads the row's last one.  Every lane loads, from inside
     // the tensor; invalid lanes are dropped when the sums are taken.
+    // With bn.in_gamma / in_beta (a BatchNorm whose output went through nothing but the ReLU, x = relu(gamma * xhat +
+    // beta)) the BatchNorm's input is not read at all: where the ReLU passed, xhat = (x - beta) / gamma comes from the
+    // x this lane holds, and where it did not, dz is zero.  Channels whose |gamma| is too small for that division
+    // (below max(1, |beta|) / 64) read the input after all, in the epilogue.
+    // The per-channel constants come through the scalar cache (nothing writes them while the kernel runs), also
+    // asked for here: as vector loads in the epilogue they would share the counter of the stores there, and every
+    // channel's loads would wait for the previous channel's sums to reach memory.
     float bx[FUSE ? TM : 1][TN], ga[FUSE ? TM : 1][TN];
+    float bn_mu[FUSE ? TM : 1], bn_rs[FUSE ? TM : 1], bn_g[FUSE ? TM : 1], bn_be[FUSE ? TM : 1];
+    int pofs = 0;
     if constexpr (FUSE) {
-        if (bn.in_part) {
-            static_assert(!FUSE || TN == 2 || TN == 4, "the strips are read as one float2 / float4");
-            int pofs = (nc * Ci + ci_base) * (H * W) + hc * W + min(wi0, W - TN);
-            asm volatile("" : "+v"(pofs));
+        static_assert(!FUSE || TN == 2 || TN == 4, "the strips are read as one float2 / float4");
+        pofs = (nc * Ci + ci_base) * (H * W) + hc * W + min(wi0, W - TN);
+        asm volatile("" : "+v"(pofs));
 #pragma unroll
-            for (int m = 0; m < TM; ++m) {
+        for (int m = 0; m < TM; ++m) {
+            bn_mu[m] = as_uniform(bn.in_mean)[ci_base + m];
+            bn_rs[m] = as_uniform(bn.in_rstd)[ci_base + m];
+            bn_g[m] = bn.in_gamma ? as_uniform(bn.in_gamma)[ci_base + m] : 0.f;
+            bn_be[m] = bn.in_gamma ? as_uniform(bn.in_beta)[ci_base + m] : 0.f;
+            if (!bn.in_gamma) {
                 global_read_strip<TN, TN>(bn.in_x + pofs + m * (H * W), bx[m]);
-                if (gadd) {
-                    global_read_strip<TN, TN>(reinterpret_cast<const float *>(gadd) + pofs + m * (H * W), ga[m]);
-                } else {
+            } else {
+                // (x, as this lane holds it, in the place of the BatchNorm's input: no registers of its own)
 #pragma unroll
-                    for (int t = 0; t < TN; ++t) ga[m][t] = 0.f;
-                }
+                for (int t = 0; t < TN; ++t) bx[m][t] = cr[m][t];
             }
+            if (gadd) global_read_strip<TN, TN>(reinterpret_cast<const float *>(gadd) + pofs + m * (H * W), ga[m]);
         }
     }
 
@@ -383,35 +395,93 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
     }
 
     if constexpr (FUSE) {
-        if (bn.in_part) {
-            // x = relu(bn(in_x) [+ residual]): what leaves here is the gradient of the BatchNorm's output before
-            // the ReLU, dz = (gx + gadd) * [x > 0], and per channel and position wave the sums of dz and dz * xhat
-            // in the partial-sum layout of the BatchNorm kernels (a wave's 64 * TN terms in fp32, the rest in fp64)
-            const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+        // x = relu(bn(in_x) [+ residual]): what leaves here is the gradient of the BatchNorm's output before the
+        // ReLU, dz = (gx + gadd) * [x > 0], and per channel and position wave the sums of dz and dz * xhat in the
+        // partial-sum layout of the BatchNorm kernels (a wave's 64 * TN terms in fp32, the rest in fp64).
+        // With one round of workgroups on the chip nothing overlaps this epilogue, so it is kept short: one mask bit
+        // per position decides what counts (inside the tensor, an own channel, the ReLU passed); per term one
+        // select, one add, one subtract and one multiply-add; the scale of xhat is applied to the wave's sum.
+        const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+        unsigned keep = 0;
+#pragma unroll
+        for (int t = 0; t < TN; ++t) keep |= (pos_ok && wi0 + t < W ? 1u : 0u) << t;
+        {
+            unsigned all = 0;
+#pragma unroll
+            for (int m = 0; m < TM; ++m) all |= (ci_base + m >= ci_first ? keep : 0u) << (m * TN);
+            keep = bn.in_relu ? all & xpos : all;
+        }
+        if (gadd) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m)
+#pragma unroll
+                for (int t = 0; t < TN; ++t) tot[m][t] += ga[m][t];
+        }
+        float s1[TM], s2[TM];
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            // |gamma| large enough that the rounding of x - beta stays ~1e-5 of xhat
+            const bool from_x = bn.in_gamma && fabsf(bn_g[m]) >= 0x1p-6f * fmaxf(1.f, fabsf(bn_be[m]));
+            if (bn.in_gamma && !from_x) global_read_strip<TN, TN>(bn.in_x + pofs + m * (H * W), bx[m]);
+            // xhat = (bx - off) * scale, with bx = cr where xhat comes from x (x = 1 - 2 cr in the two-instruction
+            // form: xhat = (cr - (1 - beta) / 2) * (-2 / gamma))
+            const float off = from_x ? (SAT ? 0.5f - 0.5f * bn_be[m] : bn_be[m]) : bn_mu[m];
+            const float scale = from_x ? (SAT ? -2.f : 1.f) * __builtin_amdgcn_rcpf(bn_g[m]) : bn_rs[m];
+            float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                // (what is zeroed for being outside the tensor or another group's channel is not stored below)
+                const int bit = __builtin_amdgcn_sbfe((int)keep, m * TN + t, 1);   // 0 or all ones
+                const float v = __int_as_float(__float_as_int(tot[m][t]) & bit);
+                tot[m][t] = v;
+                a1 += v;
+                a2 = fmaf(v, bx[m][t] - off, a2);
+            }
+            s1[m] = wave_sum_top_row(a1);
+            s2[m] = wave_sum_top_row(a2 * scale);
+        }
+        // Only stores from here on, and nothing that would have to be waited for between them: loads and stores
+        // share one counter, in order, so a wait for any later load is a wait for every store before it -- a round
+        // trip to memory per channel.
+        if (lane == 63) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m)
+                if (ci_base + m >= ci_first)
+                    *reinterpret_cast<double2 *>(bn.in_part + ((size_t)(ci_base + m) * slots + slot) * 2) =
+                        make_double2((double)s1[m], (double)s2[m]);
+        }
+        if (pos_ok && wi0 < W) {
 #pragma unroll
             for (int m = 0; m < TM; ++m) {
-                const int ci = ci_base + m;
-                const float mu = bn.in_mean[ci], rs = bn.in_rstd[ci];
-                float s1 = 0.f, s2 = 0.f;
-#pragma unroll
-                for (int t = 0; t < TN; ++t) {
-                    const bool valid = pos_ok && wi0 + t < W && ci >= ci_first;
-                    float v = tot[m][t] + ga[m][t];
-                    if (bn.in_relu && !((xpos >> (m * TN + t)) & 1u)) v = 0.f;
-                    tot[m][t] = v;
-                    s1 += valid ? v : 0.f;
-                    s2 = fmaf(valid ? v : 0.f, (bx[m][t] - mu) * rs, s2);
-                }
-                const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2);
-                if (lane == 0 && ci >= ci_first) {
-                    bn.in_part[((size_t)ci * slots + slot) * 2] = d1;
-                    bn.in_part[((size_t)ci * slots + slot) * 2 + 1] = d2;
-                }
+                if (ci_base + m < ci_first) continue;
+                float *dst = reinterpret_cast<float *>(gx) + pofs + m * (H * W);
+                if constexpr (TN == 4) stf4(dst, make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]));
+                else stf2(dst, make_float2(tot[m][0], tot[m][1]));
             }
-            gadd = nullptr;   // already added
         }
+        return;
     }
 
+    // A second gradient of the same tensor (a residual shortcut) is added on the way out -- all of it is read before
+    // the first store: loads and stores share one counter, in order, so a wait for a load behind a store is a wait
+    // for the store's round trip to memory as well.
+    if (gadd && pos_ok) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const T *src = gadd + (((size_t)n * Ci + ci_base + m) * H + hi) * W + wi0;
+            if (TN % 4 == 0 && (W & 3) == 0 && wi0 + TN <= W) {
+#pragma unroll
+                for (int t = 0; t < TN; t += 4) {
+                    const float4 a = ldf4(src + t);
+                    tot[m][t] += a.x; tot[m][t + 1] += a.y; tot[m][t + 2] += a.z; tot[m][t + 3] += a.w;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < TN; ++t)
+                    if (wi0 + t < W) tot[m][t] += ldf(src + t);
+            }
+        }
+    }
     if (pos_ok) {
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
@@ -434,18 +504,12 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
                 T *dst = gx + o;
                 if (TN % 4 == 0 && (W & 3) == 0 && wi0 + TN <= W) {
 #pragma unroll
-                    for (int t = 0; t < TN; t += 4) {
-                        float4 v = make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]);
-                        if (gadd) {   // a second gradient of the same tensor (a residual shortcut), added on the way out
-                            const float4 a = ldf4(gadd + o + t);
-                            v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
-                        }
-                        stf4(dst + t, v);
-                    }
+                    for (int t = 0; t < TN; t += 4)
+                        stf4(dst + t, make_float4(tot[m][t], tot[m][t + 1], tot[m][t + 2], tot[m][t + 3]));
                 } else {
 #pragma unroll
                     for (int t = 0; t < TN; ++t)
-                        if (wi0 + t < W) stf(dst + t, gadd ? tot[m][t] + ldf(gadd + o + t) : tot[m][t]);
+                        if (wi0 + t < W) stf(dst + t, tot[m][t]);
                 }
             }
         }
@@ -470,7 +534,7 @@ static int launch_grad_x_3x3s1_v(const T *gy, const T *x, const float *w, T *gx,
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    if (FUSE && bn.in_part && bn.in_slots != gxd * C::POSW) return ADDER_ERR_BAD_SHAPE;
+    if (FUSE && (!bn.in_part || bn.in_slots != gxd * C::POSW)) return ADDER_ERR_BAD_SHAPE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     if (int rc = allow_dynamic_lds<&grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T, FUSE>>(LDS_BYTES)) return rc;
     hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T, FUSE>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS),
@@ -686,23 +750,18 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
 
     // FUSE: the epilogue's loads, issued here as in the stride-1 kernel
     float bx[FUSE ? TM : 1][2][TNW], ga[FUSE ? TM : 1][2][TNW];
+    int pofs[2] = {0, 0};
     if constexpr (FUSE) {
-        if (bn.in_part) {
-            static_assert(!FUSE || TNW == 2, "the strips are read as one float2");
+        static_assert(!FUSE || TNW == 2, "the strips are read as one float2");
 #pragma unroll
-            for (int rp = 0; rp < 2; ++rp) {
-                int pofs = ((nc * Ci + ci_base) * H + min(hi0 + rp, H - 1)) * W + min(wi0, W - TNW);
-                asm volatile("" : "+v"(pofs));
+        for (int rp = 0; rp < 2; ++rp) {
+            pofs[rp] = ((nc * Ci + ci_base) * H + min(hi0 + rp, H - 1)) * W + min(wi0, W - TNW);
+            asm volatile("" : "+v"(pofs[rp]));
 #pragma unroll
-                for (int m = 0; m < TM; ++m) {
-                    global_read_strip<TNW, TNW>(bn.in_x + pofs + m * (H * W), bx[m][rp]);
-                    if (gadd) {
-                        global_read_strip<TNW, TNW>(reinterpret_cast<const float *>(gadd) + pofs + m * (H * W), ga[m][rp]);
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < TNW; ++t) ga[m][rp][t] = 0.f;
-                    }
-                }
+            for (int m = 0; m < TM; ++m) {
+                global_read_strip<TNW, TNW>(bn.in_x + pofs[rp] + m * (H * W), bx[m][rp]);
+                if (gadd)
+                    global_read_strip<TNW, TNW>(reinterpret_cast<const float *>(gadd) + pofs[rp] + m * (H * W), ga[m][rp]);
             }
         }
     }
@@ -739,35 +798,82 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
     }
 
     if constexpr (FUSE) {
-        if (bn.in_part) {   // dz = (gx + gadd) * [x > 0] and its per-channel sums, as in the stride-1 kernel
-            const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+        // dz = (gx + gadd) * [x > 0] and its per-channel sums, as in the stride-1 kernel (one mask bit per position,
+        // every load before the first store)
+        const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+        unsigned keep = 0;
 #pragma unroll
-            for (int m = 0; m < TM; ++m) {
-                const int ci = ci_base + m;
-                const float mu = bn.in_mean[ci], rs = bn.in_rstd[ci];
-                float s1 = 0.f, s2 = 0.f;
+        for (int rp = 0; rp < 2; ++rp)
 #pragma unroll
-                for (int rp = 0; rp < 2; ++rp) {
+            for (int t = 0; t < TNW; ++t)
+                keep |= (lane_ok && n < N && hi0 + rp < H && wi0 + t < W ? 1u : 0u) << (rp * TNW + t);
+        {
+            unsigned all = 0;
 #pragma unroll
-                    for (int t = 0; t < TNW; ++t) {
-                        const bool valid = lane_ok && n < N && hi0 + rp < H && wi0 + t < W && ci >= ci_first;
-                        float v = tot[m][rp][t] + ga[m][rp][t];
-                        if (bn.in_relu && !((xpos >> ((m * 2 + rp) * TNW + t)) & 1u)) v = 0.f;
-                        tot[m][rp][t] = v;
-                        s1 += valid ? v : 0.f;
-                        s2 = fmaf(valid ? v : 0.f, (bx[m][rp][t] - mu) * rs, s2);
-                    }
-                }
-                const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2);
-                if (lane == 0 && ci >= ci_first) {
-                    bn.in_part[((size_t)ci * slots + slot) * 2] = d1;
-                    bn.in_part[((size_t)ci * slots + slot) * 2 + 1] = d2;
+            for (int m = 0; m < TM; ++m) all |= (ci_base + m >= ci_first ? keep : 0u) << (m * 2 * TNW);
+            keep = bn.in_relu ? all & xpos : all;
+        }
+        float s1[TM], s2[TM];
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            const float mu = as_uniform(bn.in_mean)[ci_base + m], rs = as_uniform(bn.in_rstd)[ci_base + m];
+            float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+            for (int rp = 0; rp < 2; ++rp) {
+#pragma unroll
+                for (int t = 0; t < TNW; ++t) {
+                    const int bit = __builtin_amdgcn_sbfe((int)keep, (m * 2 + rp) * TNW + t, 1);   // 0 or all ones
+                    const float g = gadd ? tot[m][rp][t] + ga[m][rp][t] : tot[m][rp][t];
+                    const float v = __int_as_float(__float_as_int(g) & bit);
+                    tot[m][rp][t] = v;
+                    a1 += v;
+                    a2 = fmaf(v, bx[m][rp][t] - mu, a2);
                 }
             }
-            gadd = nullptr;   // already added
+            s1[m] = wave_sum_top_row(a1);
+            s2[m] = wave_sum_top_row(a2 * rs);
         }
+        if (lane == 63) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m)
+                if (ci_base + m >= ci_first)
+                    *reinterpret_cast<double2 *>(bn.in_part + ((size_t)(ci_base + m) * slots + slot) * 2) =
+                        make_double2((double)s1[m], (double)s2[m]);
+        }
+        if (lane_ok && n < N && wi0 < W) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m) {
+                if (ci_base + m < ci_first) continue;
+#pragma unroll
+                for (int rp = 0; rp < 2; ++rp)
+                    if (hi0 + rp < H)
+                        stf2(reinterpret_cast<float *>(gx) + pofs[rp] + m * (H * W), make_float2(tot[m][rp][0], tot[m][rp][1]));
+            }
+        }
+        return;
     }
 
+    // (a second gradient of the same tensor is read before the first store, as in the stride-1 kernel)
+    if (gadd && lane_ok && n < N) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m)
+#pragma unroll
+            for (int rp = 0; rp < 2; ++rp) {
+                if (hi0 + rp >= H) continue;
+                const T *src = gadd + (((size_t)n * Ci + ci_base + m) * H + hi0 + rp) * W + wi0;
+                if ((W & 1) == 0 && wi0 + TNW <= W) {
+#pragma unroll
+                    for (int t = 0; t < TNW; t += 2) {
+                        const float2 a = ldf2(src + t);
+                        tot[m][rp][t] += a.x; tot[m][rp][t + 1] += a.y;
+                    }
+                } else {
+#pragma unroll
+                    for (int t = 0; t < TNW; ++t)
+                        if (wi0 + t < W) tot[m][rp][t] += ldf(src + t);
+                }
+            }
+    }
     if (lane_ok && n < N) {
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
@@ -781,18 +887,11 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
                 T *dst = gx + o;
                 if ((W & 1) == 0 && wi0 + TNW <= W) {
 #pragma unroll
-                    for (int t = 0; t < TNW; t += 2) {
-                        float2 v = make_float2(tot[m][rp][t], tot[m][rp][t + 1]);
-                        if (gadd) {   // a second gradient of the same tensor, added on the way out
-                            const float2 a = ldf2(gadd + o + t);
-                            v.x += a.x; v.y += a.y;
-                        }
-                        stf2(dst + t, v);
-                    }
+                    for (int t = 0; t < TNW; t += 2) stf2(dst + t, make_float2(tot[m][rp][t], tot[m][rp][t + 1]));
                 } else {
 #pragma unroll
                     for (int t = 0; t < TNW; ++t)
-                        if (wi0 + t < W) stf(dst + t, gadd ? tot[m][rp][t] + ldf(gadd + o + t) : tot[m][rp][t]);
+                        if (wi0 + t < W) stf(dst + t, tot[m][rp][t]);
                 }
             }
         }
@@ -806,7 +905,7 @@ static int launch_grad_x_3x3s2_v(const T *gy, const T *x, const float *w, T *gx,
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    if (FUSE && bn.in_part && bn.in_slots != gxd * C::POSW) return ADDER_ERR_BAD_SHAPE;
+    if (FUSE && (!bn.in_part || bn.in_slots != gxd * C::POSW)) return ADDER_ERR_BAD_SHAPE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
     hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T, FUSE>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
@@ -857,8 +956,8 @@ static bool small_plane_tile(const ConvDims &f) {
 static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
               "the launcher checks Ci against one TM per stride");
 
-// gadd (nullable): a tensor shaped like gx that is added to the result (tiled 3x3 / pad 1 kernels only;
-// ADDER_ERR_UNSUPPORTED elsewhere)
+// gadd (nullable): a tensor shaped like gx that is added to the result (tiled 3x3 / pad 1 kernels and the tiled
+// 1x1 stride-1 kernels only; ADDER_ERR_UNSUPPORTED elsewhere)
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s, const float *gadd) {
     const bool k3s1p1 = d.kh == 3 && d.kw == 3 && d.stride == 1 && d.pad == 1;
@@ -875,18 +974,19 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
         if (d.W > 16) return launch_grad_x_3x3s2<GxS2W32>(gy, x, w, gx, d, s, gadd);
         return launch_grad_x_3x3s2<GxS2W16>(gy, x, w, gx, d, s, gadd);
     }
-    if (gadd) return ADDER_ERR_UNSUPPORTED;
-        // (from 48 output channels on the tiled kernel is ahead of the plain one: DenseNet's 48-channel bottlenecks)
+    // (from 48 output channels on the tiled kernel is ahead of the plain one: DenseNet's 48-channel bottlenecks)
     if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride == 1 && d.Ci >= 64 && d.Co >= 48) {
         ConvDims f = d;   // every (H, W) plane as one row of H*W positions
         f.H = f.Ho = 1;
         f.W = f.Wo = d.H * d.W;
-        if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0) {
-            if (f.W > 64) return launch_grad_x_3x3s1<Gx1x1>(gy, x, w, gx, f, s);
-            return small_plane_tile(f) ? launch_grad_x_3x3s1<Gx1x1t>(gy, x, w, gx, f, s)
-                                       : launch_grad_x_3x3s1<Gx1x1s>(gy, x, w, gx, f, s);
+        if (f.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx) |
+                              reinterpret_cast<uintptr_t>(gadd)) & 15) == 0) {
+            if (f.W > 64) return launch_grad_x_3x3s1<Gx1x1>(gy, x, w, gx, f, s, gadd);
+            return small_plane_tile(f) ? launch_grad_x_3x3s1<Gx1x1t>(gy, x, w, gx, f, s, gadd)
+                                       : launch_grad_x_3x3s1<Gx1x1s>(gy, x, w, gx, f, s, gadd);
         }
     }
+    if (gadd) return ADDER_ERR_UNSUPPORTED;
     if (d.kh == 1 && d.kw == 1 && d.pad == 0 && d.stride > 1 && d.Ci >= 64 && d.Co >= 64) {
         ConvDims f = d;   // the sampled positions of every plane as one row; x and gx are read / written in place
         f.H = f.Ho = 1;
@@ -955,8 +1055,10 @@ int grad_x_bn_slots(const ConvDims &d) {
 int launch_grad_x_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d, hipStream_t s,
                      const float *gadd, const adder_bn_links &bn) {
     const uintptr_t align = reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx) |
-                            reinterpret_cast<uintptr_t>(gadd) | reinterpret_cast<uintptr_t>(bn.in_x);
+                            reinterpret_cast<uintptr_t>(gadd) | reinterpret_cast<uintptr_t>(bn.in_x) |
+                            reinterpret_cast<uintptr_t>(bn.in_part);
     if (align & 15) return ADDER_ERR_UNSUPPORTED;
+    if (!bn.in_part) return launch_grad_x(gy, x, w, gx, d, s, gadd);   // nothing to leave for a BatchNorm in front
     switch (grad_x_bn_variant(d)) {
         case 1: return launch_grad_x_3x3s1_bn<GxW32>(gy, x, w, gx, d, s, gadd, bn);
         case 2: return launch_grad_x_3x3s1_bn<GxW16>(gy, x, w, gx, d, s, gadd, bn);

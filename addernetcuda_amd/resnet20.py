@@ -115,7 +115,7 @@ class _conv_bn_act(torch.autograd.Function):
                                          eps, relu, stats)
         ctx.save_for_backward(x, w, conv_out, y if relu and mask is None else None, gamma, mean, rstd, mask)
         ctx.conf, ctx.relu = (stride, padding), relu
-        ctx.out_link = _adder.BnLink(conv_out, mean, rstd, gamma, relu)
+        ctx.out_link = _adder.BnLink(conv_out, mean, rstd, gamma, relu, beta)
         return y
 
     @staticmethod

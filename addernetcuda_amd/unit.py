@@ -46,7 +46,8 @@ class _adder_bn_act(Function):
         ctx.dims, ctx.eta, ctx.relu, ctx.has_res = dims, eta, relu, residual is not None
         ctx.in_link = in_link
         # (a layer without the kernels that take the link could not use what its consumer would prepare)
-        ctx.out_link = _adder.BnLink(conv_out, mean, rstd, gamma, relu) if bwd_bn_slots(dims) > 0 else None
+        ctx.out_link = (_adder.BnLink(conv_out, mean, rstd, gamma, relu, None if residual is not None else beta)
+                        if bwd_bn_slots(dims) > 0 else None)
         ctx.set_materialize_grads(False)
         if with_shortcut:
             # X again, as an output of this node: see adder._adder_nchw.forward

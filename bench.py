@@ -121,15 +121,19 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
         coef = torch.randn(Co, 4, device=dev, generator=g) * 0.01
         yo = torch.randn(N, Co, Ho, Wo, device=dev, generator=g) * 20 - 90
         gyo = torch.empty_like(gy)
-        lx = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(part), slots, 1)
+        # (the BatchNorm in front with its weight and bias, as for a unit whose input had no residual added: the
+        # stride-1 3x3 and 1x1 kernels then take xhat from x and do not read bn_in; 2 of 3 launches of a ResNet step)
+        gamma, beta = torch.ones(Ci, device=dev), torch.zeros(Ci, device=dev)
+        lx = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(part), slots, 1, ptr(gamma), ptr(beta))
         lw = BnLinks(ptr(yo), ptr(coef), ptr(gyo), None, None, None, None, 0, 0)
-        keep += [bn_in, mean, rstd, part, coef, yo, gyo, lx, lw]
+        keep += [bn_in, mean, rstd, part, coef, yo, gyo, lx, lw, gamma, beta]
         ops["grad_x_bn"] = lambda: check(lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gx), None, 0.0,
                                                                       None, 0, *dims, ctypes.byref(lx), st), "grad_x_bn")
         ops["grad_w_bn"] = lambda: check(lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), None, None, ptr(gw), ETA,
                                                                       ptr(ws), need.value, *dims, ctypes.byref(lw), st),
                                          "grad_w_bn")
-        nbytes["grad_x_bn"] = nbytes["grad_x"] + nx + 16 * Ci * slots   # + the BatchNorm's input, + the partial sums
+        # + the partial sums, + the BatchNorm's input where the kernel reads it (stride 2)
+        nbytes["grad_x_bn"] = nbytes["grad_x"] + 16 * Ci * slots + (nx if stride != 1 else 0)
         nbytes["grad_w_bn"] = nbytes["grad_w"] + 2 * ny                 # + the layer's output, + the formed gradient
     return E, ops, keep, nbytes
 
@@ -222,7 +226,7 @@ def dominant_kernel(dev, steps):
                 "(v_fma with the clamp modifier, v_fmac) on the 4 flop of a term (sub, clamp, mul, add), so the "
                 "peak itself is its ceiling. valu_issue_util is the share of the two-slot issue rate taken by "
                 "those 2 instructions per term. The flop count is the adder layer's alone: the epilogue (mask, two "
-                "sums per channel, one more tensor read) is the first pass of a BatchNorm backward that no longer "
+                "sums per channel; xhat comes from the x the lanes hold) is the first pass of a BatchNorm backward that no longer "
                 "runs as a kernel of its own.",
     }
 

@@ -64,11 +64,18 @@ def _bn_input_grad(dz, x, gamma, mean, rstd):
 
 @pytest.mark.parametrize("case", CASES, ids=str)
 @pytest.mark.parametrize("with_add", [False, True])
-def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, gpu):
+@pytest.mark.parametrize("from_x", [False, True], ids=["reads_bn_input", "xhat_from_x"])
+def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, from_x, gpu):
+    """``from_x``: P's output went through nothing but the ReLU, and the links carry P's weight and bias so that the
+    kernel may take xhat from x; two channels are then outside what it accepts for that (a tiny and a negative
+    weight: the first must read P's input after all, the second divides by a negative number)."""
     from addernetcuda_amd._lib import lib, check, ptr, stream_ptr, BnLinks, bwd_bn_slots, conv_dims, conv2d_bwd_workspace
     from oracle import adder_oracle
     N, Ci, H, W, Co, s, k, pad = _geom(case)
     xp, res, gamma_p, beta_p, w, dzq, gamma_q, gx_add = _make(case, 17 + sum(case))
+    if from_x:
+        res = torch.zeros_like(res)
+        gamma_p[0], gamma_p[1], beta_p[0] = 1e-3, -0.7, 0.2
     dims, Ho, Wo = conv_dims((N, Ci, H, W), w.shape, s, pad)
     slots = bwd_bn_slots(dims)
     assert slots > 0
@@ -110,7 +117,9 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, gpu
 
     part = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float64, device=gpu)
     gy_out = torch.full_like(dzqg, float("nan"))
-    links = BnLinks(ptr(y32g), ptr(coef), ptr(gy_out), ptr(xpg), ptr(mean_pg), ptr(rstd_pg), ptr(part), slots, 1)
+    gamma_pg, beta_pg = (d(gamma_p), d(beta_p)) if from_x else (None, None)
+    links = BnLinks(ptr(y32g), ptr(coef), ptr(gy_out), ptr(xpg), ptr(mean_pg), ptr(rstd_pg), ptr(part), slots, 1,
+                    ptr(gamma_pg), ptr(beta_pg))
     gxg, gwg = torch.empty_like(xg), torch.empty_like(wg)
     ws, nbytes = conv2d_bwd_workspace(dims, gpu)
     check(lib.adder_conv2d_bwd_bn_f32(ptr(dzqg), ptr(xg), ptr(wg), ptr(addg), ptr(gxg), ptr(gwg), 0.2, ptr(ws), nbytes,
@@ -143,7 +152,8 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, gpu
     assert torch.equal(gw2, gwg), "staged and one-call weight gradients differ"
     assert torch.equal(gy_out2, gy_out)
     # ... and the input gradient from what it left, with the in-links alone (the order a caller that stages uses)
-    links_x = BnLinks(None, None, None, ptr(xpg), ptr(mean_pg), ptr(rstd_pg), ptr(part), slots, 1)
+    links_x = BnLinks(None, None, None, ptr(xpg), ptr(mean_pg), ptr(rstd_pg), ptr(part), slots, 1, ptr(gamma_pg),
+                      ptr(beta_pg))
     gx2 = torch.empty_like(xg)
     check(lib.adder_conv2d_bwd_bn_f32(ptr(gy_out2), ptr(xg), ptr(wg), ptr(addg), ptr(gx2), None, 0.0, None, 0, *dims,
                                       ctypes.byref(links_x), st), "adder_conv2d_bwd_bn_f32")
@@ -206,6 +216,12 @@ def test_refusals(gpu):
                                      stream_ptr(gpu))
     assert rc == -7
     dims3, _, _ = conv_dims((2, 16, 8, 8), (16, 16, 3, 3), 1, 1)
+    slots3 = bwd_bn_slots(dims3)
+    part = torch.empty(16 * slots3 * 2, dtype=torch.float64, device=gpu)
+    links = BnLinks(None, None, None, ptr(t), ptr(t), ptr(t), ptr(part), slots3, 1, ptr(t), None)   # weight, no bias
+    rc = lib.adder_conv2d_bwd_bn_f32(ptr(t), ptr(t), ptr(t), None, ptr(t), None, 0.0, None, 0, *dims3, ctypes.byref(links),
+                                     stream_ptr(gpu))
+    assert rc == -1
     links = BnLinks(ptr(t), None, None, None, None, None, None, 0, 0)     # out_x without out_coef
     rc = lib.adder_conv2d_bwd_bn_f32(ptr(t), ptr(t), ptr(t), None, ptr(t), None, 0.0, None, 0, *dims3, ctypes.byref(links),
                                      stream_ptr(gpu))
