@@ -83,3 +83,66 @@ def test_full_batch_layer(layer, gpu):
     if s == 2:                                                                     # unsampled pixels stay exactly 0
         if k == 1:
             assert (xg.grad[:, :, 1::2, :] == 0).all() and (xg.grad[:, :, :, 1::2] == 0).all()
+
+
+# the layer shapes above whose kernels carry the BatchNorm links (3x3 / pad 1, and 1x1 stride 1 from 64 channels on
+# planes of whole float4 groups), at their full batch
+LINKED = [l for l in RESNET20 if l[5] == 3] + [(64, 64, 56, 56, 256, 1, 1, 0), (64, 256, 56, 56, 64, 1, 1, 0),
+                                               (64, 512, 28, 28, 128, 1, 1, 0)]
+
+
+@pytest.mark.parametrize("from_x", [False, True], ids=["reads_bn_input", "xhat_from_x"])
+@pytest.mark.parametrize("layer", LINKED, ids=str)
+def test_full_batch_links(layer, from_x, gpu):
+    """The backward with both BatchNorm links at full batch (slot counts and grids depend on it), against the
+    library's plain kernels -- which the test above holds to the oracle -- and float64 BatchNorm arithmetic on the
+    GPU: the output gradient the weight-gradient kernel forms, both gradients, the partial sums of the BatchNorm in
+    front."""
+    import ctypes
+    from addernetcuda_amd._lib import lib, check, ptr, stream_ptr, BnLinks, bwd_bn_slots, conv_dims, conv2d_bwd_workspace
+    N, Ci, H, W, Co, k, s, p = layer
+    g = torch.Generator(device=gpu).manual_seed(7 + Ci + Co + k + s)
+    b = lambda v: v[None, :, None, None]
+    bn_in = torch.randn(N, Ci, H, W, device=gpu, generator=g) * 20 - 90
+    mean, rstd = bn_in.mean((0, 2, 3)), 1.0 / bn_in.std((0, 2, 3))
+    gamma, beta = torch.rand(Ci, device=gpu, generator=g) + 0.5, torch.randn(Ci, device=gpu, generator=g) * 0.3
+    x = (bn_in - b(mean)) * b(rstd * gamma) + b(beta)
+    if not from_x:
+        x = x + torch.randn(x.shape, device=gpu, generator=g)          # a residual: xhat cannot come from x
+    x = torch.relu(x)
+    w = torch.randn(Co, Ci, k, k, device=gpu, generator=g) * math.sqrt(2.0 / (Ci * k * k))
+    dims, Ho, Wo = conv_dims(x.shape, w.shape, s, p)
+    slots = bwd_bn_slots(dims)
+    assert slots > 0
+    y = torch.randn(N, Co, Ho, Wo, device=gpu, generator=g) * 20 - 90
+    dz = torch.randn(N, Co, Ho, Wo, device=gpu, generator=g) * (torch.rand(N, Co, Ho, Wo, device=gpu, generator=g) > 0.4)
+    coef = torch.randn(Co, 4, device=gpu, generator=g) * torch.tensor([1.0, 0.01, 0.0, 0.1], device=gpu)
+    coef[:, 2] = y.mean((0, 2, 3))
+    gadd = torch.randn(x.shape, device=gpu, generator=g)
+    st = stream_ptr(gpu)
+    ws, nbytes = conv2d_bwd_workspace(dims, gpu)
+
+    part = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float64, device=gpu)
+    gy_out = torch.empty_like(dz)
+    links = BnLinks(ptr(y), ptr(coef), ptr(gy_out), ptr(bn_in), ptr(mean), ptr(rstd), ptr(part), slots, 1,
+                    ptr(gamma) if from_x else None, ptr(beta) if from_x else None)
+    gx, gw = torch.empty_like(x), torch.empty_like(w)
+    check(lib.adder_conv2d_bwd_bn_f32(ptr(dz), ptr(x), ptr(w), ptr(gadd), ptr(gx), ptr(gw), 0.1, ptr(ws), nbytes, *dims,
+                                      ctypes.byref(links), st), "adder_conv2d_bwd_bn_f32")
+    torch.cuda.synchronize()
+
+    c = coef.double()
+    want_gy = b(c[:, 0]) * dz.double() + b(c[:, 1]) * (y.double() - b(c[:, 2])) - b(c[:, 3])
+    assert_close(gy_out, want_gy, f"formed gy {layer}", rtol=1e-5, atol=1e-5)
+    # the same kernels without the links, on the gradient that was formed
+    gx0, gw0 = torch.empty_like(x), torch.empty_like(w)
+    check(lib.adder_conv2d_bwd_f32(ptr(gy_out), ptr(x), ptr(w), ptr(gx0), ptr(gw0), 0.1, ptr(ws), nbytes, *dims, st),
+          "adder_conv2d_bwd_f32")
+    torch.cuda.synchronize()
+    assert torch.equal(gw, gw0)
+    assert torch.equal(gx, (gx0 + gadd) * (x > 0))
+    xhat = (bn_in.double() - b(mean.double())) * b(rstd.double())
+    want = torch.stack([gx.double().sum((0, 2, 3)), (gx.double() * xhat).sum((0, 2, 3))], 1)
+    assert torch.isfinite(part).all()
+    scale = max(1.0, float(want.abs().max()))
+    assert_close(part.sum(1) / scale, want / scale, f"sums of dz, dz * xhat {layer}", rtol=1e-5, atol=1e-5)
