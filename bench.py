@@ -34,8 +34,8 @@ PEAK_VALU_ISSUE = 2 * 256 * 64 * 2.4e9
 BATCH = 256
 ETA = 0.1
 # HBM bytes per launch of the dominant kernel, from the rocprofv3 counter passes kept under profiles/
-# (54.8 MB fetched + 22.2 MB written; cannot be read without the profiler attached)
-DOMINANT_TRAFFIC_BYTES = 77.0e6
+# (37.0 MB fetched + 19.1 MB written; cannot be read without the profiler attached)
+DOMINANT_TRAFFIC_BYTES = 56.1e6
 
 # distinct adder-layer shapes of ResNet-20 at 32x32 input: (count, Ci, H, W, Co, k, stride, pad)
 RESNET20_LAYERS = [

@@ -313,8 +313,8 @@ typedef struct adder_bn_links {
     int in_relu;
     /* optional, both or neither, and only for a BatchNorm whose output reached the layer through nothing but the
        ReLU (no residual added): its weight and bias (Ci).  The stride-1 kernels then take xhat = (x - beta) / gamma
-       from the x they hold instead of reading in_x (which must still be given: channels with |gamma| < max(1, |beta|) / 64 and
-       the stride-2 kernels read it). */
+       from the x they hold instead of reading in_x (which must still be given: channels with
+       |gamma| < max(1, |beta|) / 64 and the stride-2 kernels read it). */
     const float *in_gamma;
     const float *in_beta;
 } adder_bn_links;
