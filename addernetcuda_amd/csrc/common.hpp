@@ -177,6 +177,50 @@ __device__ __forceinline__ float wave_sum_top_row(float v) {
     return v;
 }
 
+// K sums over the 64 lanes at once (K = 4, 8 or 16) for a caller that needs each of them in one lane only: a
+// reduce-scatter.  In each of the first log2(K) steps a lane keeps half of its values, hands the other half to its
+// partner and adds what the partner hands over, so that the values halve while the lanes per sum double (partners: lane
+// ^ 1, lane ^ 2, then the lanes 4 and 8 further round the row of 16, which pairs the quads just as well); what is left
+// of the four in-row steps are plain sums, and the four rows are added lane by lane through the LDS crossbar (two
+// ds_bpermute; the row broadcasts of DPP hand on lane 15 only).  K + K/2 + ... additions instead of 6 K.
+// Returns, in every lane, the sum of v[j] over the wave with j = wave_sum_scatter_index<K>(lane); v is used up.
+template <int CTRL>
+__device__ __forceinline__ float dpp_row_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int K>
+__device__ __forceinline__ int wave_sum_scatter_index(int lane) {
+    constexpr int BITS = K == 16 ? 4 : (K == 8 ? 3 : 2);
+    return (int)(__brev((unsigned)lane) >> (32 - BITS));   // step s splits on bit s of the lane and on bit BITS-1-s of j
+}
+template <int K, int S, int CTRL>
+__device__ __forceinline__ void wave_sum_scatter_step(float (&v)[K], int lane) {
+    constexpr int n = (K >> S) > 1 ? (K >> S) : 1;   // values still held before this step
+    if constexpr (n > 1) {
+        constexpr int h = n / 2;
+        const bool up = (lane >> S) & 1;
+#pragma unroll
+        for (int i = 0; i < h; ++i) {
+            const float keep = up ? v[i + h] : v[i], send = up ? v[i] : v[i + h];
+            v[i] = keep + dpp_row_move<CTRL>(send);
+        }
+    } else {
+        v[0] += dpp_row_move<CTRL>(v[0]);
+    }
+}
+template <int K>
+__device__ __forceinline__ float wave_sum_scatter(float (&v)[K], int lane) {
+    static_assert(K == 4 || K == 8 || K == 16, "4, 8 or 16 sums");
+    wave_sum_scatter_step<K, 0, 0xB1>(v, lane);    // quad_perm [1,0,3,2]
+    wave_sum_scatter_step<K, 1, 0x4E>(v, lane);    // quad_perm [2,3,0,1]
+    wave_sum_scatter_step<K, 2, 0x124>(v, lane);   // row_ror:4
+    wave_sum_scatter_step<K, 3, 0x128>(v, lane);   // row_ror:8
+    float r = v[0];
+    r += __shfl_xor(r, 16, 64);
+    r += __shfl_xor(r, 32, 64);
+    return r;
+}
+
 struct ConvDims {
     int N, Ci, H, W, Co, kh, kw, stride, pad, Ho, Wo;
     __host__ __device__ int K() const { return Ci * kh * kw; }

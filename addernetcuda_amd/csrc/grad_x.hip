@@ -417,7 +417,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
 #pragma unroll
                 for (int t = 0; t < TN; ++t) tot[m][t] += ga[m][t];
         }
-        float s1[TM], s2[TM];
+        float sums[2 * TM];   // per channel: dz, dz * xhat
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
             // |gamma| large enough that the rounding of x - beta stays ~1e-5 of xhat
@@ -437,18 +437,17 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
                 a1 += v;
                 a2 = fmaf(v, bx[m][t] - off, a2);
             }
-            s1[m] = wave_sum_top_row(a1);
-            s2[m] = wave_sum_top_row(a2 * scale);
+            sums[2 * m] = a1;
+            sums[2 * m + 1] = a2 * scale;
         }
+        // all 2 TM wave sums at once; lane l ends with the one numbered wave_sum_scatter_index(l)
+        const float total = wave_sum_scatter<2 * TM>(sums, lane);
         // Only stores from here on, and nothing that would have to be waited for between them: loads and stores
         // share one counter, in order, so a wait for any later load is a wait for every store before it -- a round
         // trip to memory per channel.
-        if (lane == 63) {
-#pragma unroll
-            for (int m = 0; m < TM; ++m)
-                if (ci_base + m >= ci_first)
-                    *reinterpret_cast<double2 *>(bn.in_part + ((size_t)(ci_base + m) * slots + slot) * 2) =
-                        make_double2((double)s1[m], (double)s2[m]);
+        if (lane < 2 * TM) {
+            const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
+            if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = (double)total;
         }
         if (pos_ok && wi0 < W) {
 #pragma unroll
@@ -813,7 +812,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
             for (int m = 0; m < TM; ++m) all |= (ci_base + m >= ci_first ? keep : 0u) << (m * 2 * TNW);
             keep = bn.in_relu ? all & xpos : all;
         }
-        float s1[TM], s2[TM];
+        float sums[2 * TM];   // per channel: dz, dz * xhat
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
             const float mu = as_uniform(bn.in_mean)[ci_base + m], rs = as_uniform(bn.in_rstd)[ci_base + m];
@@ -830,15 +829,13 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
                     a2 = fmaf(v, bx[m][rp][t] - mu, a2);
                 }
             }
-            s1[m] = wave_sum_top_row(a1);
-            s2[m] = wave_sum_top_row(a2 * rs);
+            sums[2 * m] = a1;
+            sums[2 * m + 1] = a2 * rs;
         }
-        if (lane == 63) {
-#pragma unroll
-            for (int m = 0; m < TM; ++m)
-                if (ci_base + m >= ci_first)
-                    *reinterpret_cast<double2 *>(bn.in_part + ((size_t)(ci_base + m) * slots + slot) * 2) =
-                        make_double2((double)s1[m], (double)s2[m]);
+        const float total = wave_sum_scatter<2 * TM>(sums, lane);
+        if (lane < 2 * TM) {
+            const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
+            if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = (double)total;
         }
         if (lane_ok && n < N && wi0 < W) {
 #pragma unroll
