@@ -315,20 +315,22 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
 }
 
 // ---- host side ------------------------------------------------------------------
-// One blocking for every layer: a workgroup of eight waves owns 16 output channels x 16 input channels
-// (one accumulator row of nine 16x16 fp64 tiles per wave = 72 registers) and 256 positions per staged
-// tile.  Small (co, k) blocks keep the partial slabs at Co*K values per position split whatever the layer.
+// One blocking for every layer: a workgroup of twelve waves owns 16 output channels x 16 input channels (nine
+// 16x16 fp64 accumulator tiles: three k waves with three tiles each, times four position waves) and 256 positions
+// per staged tile.  Small (co, k) blocks keep the partial slabs at Co*K values per position split whatever the layer.
+// (Eight position waves with all nine tiles each were 1.5-3 us per launch slower: a three-round fold of 72
+// registers per lane through LDS at the end, against two rounds of 24.)
 //                            S  TH  TW NIMG MT NT MW NW PW
-using GmW32   = GwMfmaCfg<1, 8, 32, 1, 1, 9, 1, 1, 8>;   // outputs 32 wide: 8 rows of one image
-using GmW16   = GwMfmaCfg<1, 16, 16, 1, 1, 9, 1, 1, 8>;  // outputs 16 wide: one image
-using GmW8    = GwMfmaCfg<1, 8, 8, 4, 1, 9, 1, 1, 8>;    // outputs 8 wide:  four images
-using GmW16S2 = GwMfmaCfg<2, 8, 16, 1, 1, 9, 1, 1, 8>;   // stride 2, outputs 16 wide: half an image
-using GmW8S2  = GwMfmaCfg<2, 8, 8, 2, 1, 9, 1, 1, 8>;    // stride 2, outputs 8 wide: two images
+using GmW32   = GwMfmaCfg<1, 8, 32, 1, 1, 3, 1, 3, 4>;   // outputs 32 wide: 8 rows of one image
+using GmW16   = GwMfmaCfg<1, 16, 16, 1, 1, 3, 1, 3, 4>;  // outputs 16 wide: one image
+using GmW8    = GwMfmaCfg<1, 8, 8, 4, 1, 3, 1, 3, 4>;    // outputs 8 wide:  four images
+using GmW16S2 = GwMfmaCfg<2, 8, 16, 1, 1, 3, 1, 3, 4>;   // stride 2, outputs 16 wide: half an image
+using GmW8S2  = GwMfmaCfg<2, 8, 8, 2, 1, 3, 1, 3, 4>;    // stride 2, outputs 8 wide: two images
 // 1x1, stride 1: a plain (Co x positions) x (positions x Ci) product; (H, W) planes walked as one row.
-// 64 output channels x 64 input channels per workgroup (sixteen accumulator tiles per wave), 128 positions
-// per staged tile; every wave does four steps of 16 MFMAs on 4 + 4 LDS reads per tile.
-using Gm1x1   = GwMfmaCfg<1, 1, 128, 1, 4, 4, 1, 1, 8, 1>;
-using Gm1x1s  = GwMfmaCfg<1, 1, 64, 2, 4, 4, 1, 1, 8, 1>;    // planes of <= 64 positions: two images
+// 64 output channels x 64 input channels per workgroup (two k waves with eight accumulator tiles each, times four
+// position waves), 128 positions per staged tile; every wave does eight steps of 8 MFMAs on 4 + 2 LDS reads per tile.
+using Gm1x1   = GwMfmaCfg<1, 1, 128, 1, 4, 2, 1, 2, 4, 1>;
+using Gm1x1s  = GwMfmaCfg<1, 1, 64, 2, 4, 2, 1, 2, 4, 1>;    // planes of <= 64 positions: two images
 // From 128 channels on either side: 128 x 128 channels per workgroup (2 x 2 waves of 64 x 64 and two position
 // waves), 64 positions per staged tile.  The 64 x 64 blocking reads every x tile Co / 64 times and every gy tile
 // Ci / 64 times, which is what bounds it on the wide layers; this one halves that (5-15 % less time).
@@ -344,8 +346,8 @@ static void plan_one(const ConvDims &d, GradWMfmaPlan &p) {
     p.ntiles = ceil_div(d.N, G::NIMG) * p.tilesH * p.tilesW;
     p.gy = ceil_div(d.Co, G::COB);
     p.gz = ceil_div(d.Ci * G::KK, G::KB);
-    // ~2048 waves over the chip (two per SIMD; a workgroup's staged tiles fill a good part of a CU's LDS)
-    int want = ceil_div(2048 / (G::NTHREADS / 64), p.gy * p.gz);
+    // one workgroup per CU (a workgroup's two staged tiles fill half of a CU's LDS and more)
+    int want = ceil_div(256, p.gy * p.gz);
     p.slots = want < p.ntiles ? want : p.ntiles;
     if (p.slots < 1) p.slots = 1;
 }
