@@ -218,7 +218,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
         }
         const float *base = smem + cur * G::BUF;
         auto steps = [&](const int first, const int last) {
-#pragma unroll 4
+#pragma unroll 8
             for (int ws = first; ws < last; ++ws) {
                 const int st = pw + ws * G::PW;                 // wave-uniform step: (img, row, column group)
                 const int c4 = st % (G::TW / 4);
