@@ -192,7 +192,11 @@ def test_random_shapes_match_oracle(case, gpu):
 
 @pytest.mark.parametrize("case", [(3, 16, 32, 32, 16, 3, 1, 1), (2, 32, 16, 16, 32, 3, 1, 1), (5, 64, 8, 8, 64, 3, 1, 1),
                                   (2, 9, 10, 18, 8, 3, 1, 1), (2, 16, 14, 14, 24, 1, 1, 0), (2, 6, 14, 24, 10, 3, 2, 1),
-                                  (2, 16, 32, 32, 32, 3, 2, 1), (3, 32, 16, 16, 64, 3, 2, 1), (2, 5, 12, 20, 7, 3, 2, 1)],
+                                  (2, 16, 32, 32, 32, 3, 2, 1), (3, 32, 16, 16, 64, 3, 2, 1), (2, 5, 12, 20, 7, 3, 2, 1),
+                                  # the tiled 1x1 kernels (from 64 input channels): large and small planes, planes that
+                                  # are not whole groups of four
+                                  (2, 64, 14, 14, 64, 1, 1, 0), (4, 64, 8, 8, 256, 1, 1, 0), (2, 128, 7, 7, 128, 1, 1, 0),
+                                  (3, 256, 6, 6, 64, 1, 1, 0), (40, 72, 8, 8, 56, 1, 1, 0)],
                          ids=str)
 def test_shortcut_gradient_is_added_to_grad_x(case, gpu):
     """with_shortcut: x leaves the layer's autograd node a second time; what is back-propagated into that output
