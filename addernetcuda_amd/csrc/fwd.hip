@@ -226,22 +226,57 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
 #pragma unroll
         for (int t = 0; t < TN; ++t) cnt += (row_ok && wo + t < Wo) ? 1.f : 0.f;
         const double count = (double)wave_sum_dpp(cnt);
+        if constexpr (TM == 2 || TM == 4 || TM == 8) {
+            // all 2 TM sums of the wave in one reduce-scatter: lane l < 2 TM ends with sum number j(l) (channel j / 2,
+            // first or second moment j % 2), fetches the other moment of its channel from the lane that holds it,
+            // and moves its own one back to the origin
+            float sums[2 * TM], pivot[TM];
 #pragma unroll
-        for (int m = 0; m < TM; ++m) {
-            const float pivot = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(tot[m][0])));
-            float s1 = 0.f, s2 = 0.f;
+            for (int m = 0; m < TM; ++m) {
+                pivot[m] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(tot[m][0])));
+                float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-            for (int t = 0; t < TN; ++t)
-                if (row_ok && wo + t < Wo) {
-                    const float dv = tot[m][t] - pivot;
-                    s1 += dv;
-                    s2 = fmaf(dv, dv, s2);
-                }
-            const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2), c = (double)pivot;
+                for (int t = 0; t < TN; ++t)
+                    if (row_ok && wo + t < Wo) {
+                        const float dv = tot[m][t] - pivot[m];
+                        s1 += dv;
+                        s2 = fmaf(dv, dv, s2);
+                    }
+                sums[2 * m] = s1;
+                sums[2 * m + 1] = s2;
+            }
+            const float mine = wave_sum_scatter<2 * TM>(sums, lane);
+            constexpr int TOP = TM;   // lane bit that j % 2 comes from: j is the bit reversal of the lane
+            const float other = __shfl_xor(mine, TOP, 64);
+            const int j = wave_sum_scatter_index<2 * TM>(lane), m = j >> 1;
+            float piv = pivot[0];
+#pragma unroll
+            for (int k = 1; k < TM; ++k) piv = m == k ? pivot[k] : piv;
+            const double c = (double)piv;
             const int co = co_base + m;
-            if (lane == 0 && co < Co) {
-                stats[((size_t)co * slots + slot) * 2] = d1 + count * c;
-                stats[((size_t)co * slots + slot) * 2 + 1] = d2 + 2.0 * c * d1 + count * c * c;
+            if (lane < 2 * TM && co < Co) {
+                // j % 2 == 0: sum of y = d1 + n c;  else: sum of y*y = d2 + 2 c d1 + n c*c
+                const double v = (j & 1) ? (double)mine + 2.0 * c * (double)other + count * c * c : (double)mine + count * c;
+                stats[((size_t)co * slots + slot) * 2 + (j & 1)] = v;
+            }
+        } else {
+#pragma unroll
+            for (int m = 0; m < TM; ++m) {
+                const float pivot = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(tot[m][0])));
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int t = 0; t < TN; ++t)
+                    if (row_ok && wo + t < Wo) {
+                        const float dv = tot[m][t] - pivot;
+                        s1 += dv;
+                        s2 = fmaf(dv, dv, s2);
+                    }
+                const double d1 = (double)wave_sum_dpp(s1), d2 = (double)wave_sum_dpp(s2), c = (double)pivot;
+                const int co = co_base + m;
+                if (lane == 0 && co < Co) {
+                    stats[((size_t)co * slots + slot) * 2] = d1 + count * c;
+                    stats[((size_t)co * slots + slot) * 2 + 1] = d2 + 2.0 * c * d1 + count * c * c;
+                }
             }
         }
     }
