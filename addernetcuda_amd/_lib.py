@@ -26,6 +26,7 @@ _SIGNATURES = {
     "adder_out_dim": (_i, [_i, _i, _i, _i]),
     "adder_conv2d_fwd_f32": (_i, [_p, _p, _p] + [_i] * 9 + [_p]),
     "adder_conv2d_fwd_stats_slots": (_i, [_i] * 9 + [ctypes.POINTER(ctypes.c_int)]),
+    "adder_conv2d_fwd_pair_stats_f32": (_i, [_p] * 7 + [_i] * 10 + [_p]),
     "adder_conv2d_fwd_stats_f32": (_i, [_p, _p, _p, _p, _i] + [_i] * 9 + [_p]),
     "adder_plain_conv2d_fwd_f32": (_i, [_p, _p, _p, _p, _i] + [_i] * 9 + [_p]),
     "adder_conv2d_bwd_workspace_bytes": (_i, [_i] * 9 + [_szp]),

@@ -158,6 +158,58 @@ def conv_forward(X, W, stride, padding, with_stats):
     return out, stats, dims
 
 
+class SideOutput:
+    """The output of a strided 1x1 layer that was computed by the strided 3x3 layer beside it (same input: the first
+    layer and the downsample layer of a residual block that halves the map; ``adder_conv2d_fwd_pair_stats_f32``).
+    Made by the 3x3 layer's node, attached to the tensor that carries x on to the 1x1 layer, and taken by that
+    layer's node in place of its own forward launch if it is asked for exactly this product."""
+    __slots__ = ("x_ptr", "x_shape", "x_version", "w_ptr", "w_version", "out", "stats")
+
+    def __init__(self, x, w, out, stats):
+        self.x_ptr, self.x_shape, self.x_version = x.data_ptr(), tuple(x.shape), x._version
+        self.w_ptr, self.w_version = w.data_ptr(), w._version
+        self.out, self.stats = out, stats
+
+    @staticmethod
+    def of(x, w, stride, padding):
+        """(out, stats) if ``x`` carries the product of exactly this 1x1 / stride-2 / pad-0 layer, else None."""
+        side = getattr(x, "_adder_side_output", None)
+        if (side is None or side.out is None or stride != 2 or padding != 0 or tuple(w.shape[2:]) != (1, 1)
+                or side.x_ptr != x.data_ptr() or side.x_shape != tuple(x.shape) or side.x_version != x._version
+                or side.w_ptr != w.data_ptr() or side.w_version != w._version or not w.is_contiguous()):
+            return None
+        out, stats = side.out, side.stats
+        side.out = side.stats = None   # taken once
+        return out, stats
+
+
+def conv_forward_pair(X, W, W_side, stride, padding):
+    """``conv_forward`` (with statistics) of a strided 3x3 layer and, in the same launch, of the strided 1x1 layer
+    ``W_side`` on the same input: (out, stats, out_side, stats_side, dims), or None where that kernel does not apply
+    (the caller then runs the two layers one after the other)."""
+    if (stride != 2 or padding != 1 or tuple(W.shape[2:]) != (3, 3) or tuple(W_side.shape) != (W.size(0), W.size(1), 1, 1)
+            or not W_side.is_cuda or W_side.dtype != torch.float32 or W_side.device != X.device):
+        return None
+    require_gpu_f32(X, "X")
+    require_gpu_f32(W, "W")
+    dev = same_device(X, W)
+    dims, Ho, Wo = conv_dims(X.shape, W.shape, stride, padding)
+    with on_device(dev):
+        slots = fwd_stats_slots(dims)
+        if slots <= 0:
+            return None
+        out = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
+        out_side = torch.empty_like(out)
+        stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64)
+        stats_side = torch.empty_like(stats)
+        status = lib.adder_conv2d_fwd_pair_stats_f32(ptr(X), ptr(W), ptr(W_side), ptr(out), ptr(out_side), ptr(stats),
+                                                     ptr(stats_side), slots, *dims, stream_ptr(dev))
+        if status == -7:
+            return None
+        check(status, "adder_conv2d_fwd_pair_stats_f32")
+    return out, stats, out_side, stats_side, dims
+
+
 class BnLink:
     """What passes between the backward of a layer and the BatchNorm on either side of it when the BatchNorm's
     backward is folded into the layer's kernels (``adder_bn_links`` of the C ABI; unit.py drives it).

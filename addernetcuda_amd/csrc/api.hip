@@ -129,6 +129,35 @@ int adder_conv2d_fwd_stats_f32(const float *x, const float *w, float *y, double 
     return launch_fwd(x, w, y, stats, d, static_cast<hipStream_t>(stream));
 }
 
+int adder_conv2d_fwd_pair_stats_f32(const float *x, const float *w, const float *w_side, float *y, float *y_side,
+                                    double *stats, double *stats_side, int stats_slots, int N, int Ci, int H, int W,
+                                    int Co, int kh, int kw, int stride, int pad, void *stream) {
+    if (!x || !w || !w_side || !y || !y_side || !stats || !stats_side) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    if (!fwd_pair_supported(d)) return ADDER_ERR_UNSUPPORTED;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) |
+                            reinterpret_cast<uintptr_t>(y_side);
+    if (align & 15) return ADDER_ERR_UNSUPPORTED;
+    const int slots = fwd_stats_slots(d);
+    if (slots == 0) return ADDER_ERR_UNSUPPORTED;
+    if (stats_slots != slots) return ADDER_ERR_BAD_SHAPE;
+    const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
+                 nws = sizeof(float) * (size_t)Co * Ci, ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo,
+                 ns = sizeof(double) * 2 * (size_t)Co * slots;
+    const void *ins[3] = {x, w, w_side};
+    const size_t in_bytes[3] = {nx, nw, nws};
+    void *outs[4] = {y, y_side, stats, stats_side};
+    const size_t out_bytes[4] = {ny, ny, ns, ns};
+    for (int o = 0; o < 4; ++o) {
+        for (int i = 0; i < 3; ++i)
+            if (overlaps(outs[o], out_bytes[o], ins[i], in_bytes[i])) return ADDER_ERR_ALIAS;
+        for (int o2 = o + 1; o2 < 4; ++o2)
+            if (overlaps(outs[o], out_bytes[o], outs[o2], out_bytes[o2])) return ADDER_ERR_ALIAS;
+    }
+    return launch_fwd_pair(x, w, w_side, y, y_side, stats, stats_side, d, static_cast<hipStream_t>(stream));
+}
+
 int adder_plain_conv2d_fwd_f32(const float *x, const float *w, float *y, double *stats, int stats_slots, int N,
                                int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, void *stream) {
     if (!x || !w || !y) return ADDER_ERR_NULL_POINTER;

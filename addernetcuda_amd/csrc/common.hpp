@@ -233,6 +233,9 @@ int check_launch();                  // hipGetLastError -> status
 // Launchers implemented in the kernel translation units.
 int launch_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s);
 int fwd_stats_slots(const ConvDims &d);
+bool fwd_pair_supported(const ConvDims &d);
+int launch_fwd_pair(const float *x, const float *w, const float *w_side, float *y, float *y_side, double *stats,
+                    double *stats_side, const ConvDims &d, hipStream_t s);
 int launch_mulconv_fwd(const float *x, const float *w, float *y, double *stats, const ConvDims &d, hipStream_t s);   // 0: no statistics epilogue for these dimensions
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s, const float *gadd = nullptr);

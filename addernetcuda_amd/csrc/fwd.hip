@@ -87,13 +87,21 @@ __global__ __launch_bounds__(256) void fwd_generic_kernel(const T *__restrict__ 
 // MUL: the same kernel as an ordinary convolution, y = sum w * x (one v_fmac per term), for the regular
 // stem layer that precedes the adder layers of a network.
 // T: storage type of x and y (float, or bf16_t for the reduced-storage mode); the arithmetic is fp32 either way.
-template <class C, bool VEC = true, bool SUB = false, bool MUL = false, class T = float>
+// PAIR (3x3 taps at stride 2 only): the strided 1x1 layer that reads the same x beside this layer (the downsample
+// branch of a residual block, resnet20.py:66-70) is computed along with it -- its one tap is the centre tap of the
+// 3x3 window, so the x values are in registers already: weights w_side (Co, Ci), output y_side and statistics
+// stats_side shaped like y and stats.
+template <class C, bool VEC = true, bool SUB = false, bool MUL = false, class T = float, bool PAIR = false>
 __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restrict__ x,
                                                                 const float *__restrict__ w,
                                                                 T *__restrict__ y,
                                                                 double *__restrict__ stats, int N, int Ci,
                                                                 int H, int W, int Co, int Ho, int Wo,
-                                                                int tilesH, int tilesW, const Subsample sub) {
+                                                                int tilesH, int tilesW, const Subsample sub,
+                                                                const float *__restrict__ w_side = nullptr,
+                                                                T *__restrict__ y_side = nullptr,
+                                                                double *__restrict__ stats_side = nullptr) {
+    static_assert(!PAIR || (C::S == 2 && C::KS == 3 && !MUL && !SUB), "the side layer is a strided 1x1 beside a strided 3x3");
     constexpr int TN = C::TN, TM = C::TM, CQ = C::CQ, S = C::S, STRIP = C::STRIP, KS = C::KS, KK = C::KK;
     extern __shared__ __align__(16) float smem[];
 
@@ -120,6 +128,17 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
 #pragma unroll
     for (int m = 0; m < TM; ++m)
         wrow[m] = __builtin_amdgcn_readfirstlane(min(co_base + m, Co - 1) * K);
+    uniform_f32_ptr wsc = as_uniform(w_side);
+    int wsrow[PAIR ? TM : 1];
+    float tots[PAIR ? TM : 1][TN];   // PAIR: the side layer's sums (Ci terms each: one level)
+    if constexpr (PAIR) {
+#pragma unroll
+        for (int m = 0; m < TM; ++m) {
+            wsrow[m] = __builtin_amdgcn_readfirstlane(min(co_base + m, Co - 1) * Ci);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) tots[m][t] = 0.f;
+        }
+    }
 
     // two-level sum: `acc` collects one channel chunk (<= 9*CC terms), `tot` the chunks, so the
     // rounding error grows with the square roots of the two lengths instead of with K
@@ -153,6 +172,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
         // operands and with the rest of the arithmetic still ahead to hide the latency.
         float xr[2][CQ][KS][STRIP];
         float wv[2][CQ * KK];
+        float wsv[2][CQ];   // PAIR: the side layer's weights, buffered like wv
 #pragma unroll
         for (int q = 0; q < CQ; ++q)
 #pragma unroll
@@ -160,6 +180,10 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
                 lds_read_strip<STRIP, C::STRIP_ALIGN>(lbase + q * C::PLANE + i * C::PITCH, xr[0][q][i]);
 #pragma unroll
         for (int e = 0; e < CQ * KK; ++e) wv[0][e] = wc[wrow[0] + ci0 * KK + e];
+        if constexpr (PAIR) {
+#pragma unroll
+            for (int q = 0; q < CQ; ++q) wsv[0][q] = wsc[wsrow[0] + ci0 + q];
+        }
 
         auto half = [&](const int cc, const int cur) {
             // cur = 0/1: which xr buffer holds channel group cc
@@ -180,9 +204,18 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
                         if (m + 1 < TM) {
 #pragma unroll
                             for (int e = 0; e < CQ * KK; ++e) wv[(m + 1) & 1][e] = wc[wrow[m + 1] + kofs + e];
+                            if constexpr (PAIR) {
+#pragma unroll
+                                for (int q2 = 0; q2 < CQ; ++q2) wsv[(m + 1) & 1][q2] = wsc[wsrow[m + 1] + ci0 + cc + q2];
+                            }
                         } else {
 #pragma unroll
                             for (int e = 0; e < CQ * KK; ++e) wv[(m + 1) & 1][e] = wc[wrow[0] + knext + e];
+                            if constexpr (PAIR) {
+#pragma unroll
+                                for (int q2 = 0; q2 < CQ; ++q2)
+                                    wsv[(m + 1) & 1][q2] = wsc[wsrow[0] + ci0 + (more ? cc + CQ : cc) + q2];
+                            }
                         }
                         if (m == 0 && more) {
 #pragma unroll
@@ -194,6 +227,12 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
                         }
                         __builtin_amdgcn_sched_barrier(0);
                     }
+                }
+                if constexpr (PAIR) {   // the centre tap (1, 1) is the strided 1x1 layer's only tap
+#pragma unroll
+                    for (int q = 0; q < CQ; ++q)
+#pragma unroll
+                        for (int t = 0; t < TN; ++t) tots[m][t] -= fabsf(wsv[m & 1][q] - xr[cur][q][1][t * S + 1]);
                 }
             }
         };
@@ -214,6 +253,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
     }
 
     const int n = n0 + img, ho = h0 + row, wo = w0 + strip * TN;
+    auto finish = [&](float (&tot)[TM][TN], T *__restrict__ y, double *__restrict__ stats) {
     if (stats) {
         // BatchNorm statistics of the layer's output on the way out: per wave and output channel the sums of
         // y and y*y over the wave's valid positions, in the partial-sum layout of the BatchNorm kernels
@@ -299,6 +339,9 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_3x3_kernel(const T *__restric
             }
         }
     }
+    };
+    finish(tot, y, stats);
+    if constexpr (PAIR) finish(tots, y_side, stats_side);
 }
 
 template <class C, bool VEC, bool SUB = false, bool MUL = false, class T = float>
@@ -390,6 +433,35 @@ static ConvDims as_one_row(const ConvDims &d) {
     return f;
 }
 static Subsample sampling_of(const ConvDims &d) { return Subsample{d.stride, d.Wo, d.W, d.H * d.W}; }
+
+// A strided 3x3 / pad 1 layer and the strided 1x1 / pad 0 layer beside it (same x, same Co, Ho, Wo) in one launch;
+// d describes the 3x3 layer.  Both outputs with their statistics (fwd_stats_slots(d) slots each).  Rows of whole
+// float4 groups only; ADDER_ERR_UNSUPPORTED otherwise.
+template <class C>
+static int launch_fwd_pair_3x3(const float *x, const float *w, const float *w_side, float *y, float *y_side,
+                               double *stats, double *stats_side, const ConvDims &d, hipStream_t s) {
+    const int tilesH = ceil_div(d.Ho, C::TH), tilesW = ceil_div(d.Wo, C::TW);
+    const long gx = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
+    const int gy = ceil_div(d.Co, C::TM * C::COW);
+    if (gx > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
+    if (int rc = allow_dynamic_lds<&fwd_3x3_kernel<C, true, false, false, float, true>>(C::LDS_BYTES)) return rc;
+    hipLaunchKernelGGL((fwd_3x3_kernel<C, true, false, false, float, true>), dim3((unsigned)gx, gy), dim3(C::NTHREADS),
+                       C::LDS_BYTES, s, x, w, y, stats, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW,
+                       Subsample{1, 0, 0, 0}, w_side, y_side, stats_side);
+    return check_launch();
+}
+
+bool fwd_pair_supported(const ConvDims &d) {
+    return d.kh == 3 && d.kw == 3 && d.pad == 1 && d.stride == 2 && d.W % 4 == 0 && d.H % 2 == 0 && d.W % 2 == 0;
+}
+
+int launch_fwd_pair(const float *x, const float *w, const float *w_side, float *y, float *y_side, double *stats,
+                    double *stats_side, const ConvDims &d, hipStream_t s) {
+    if (!fwd_pair_supported(d)) return ADDER_ERR_UNSUPPORTED;
+    if (d.Wo > 8) return launch_fwd_pair_3x3<FwdW16S2>(x, w, w_side, y, y_side, stats, stats_side, d, s);
+    return d.Ci >= 128 ? launch_fwd_pair_3x3<FwdW8S2L>(x, w, w_side, y, y_side, stats, stats_side, d, s)
+                       : launch_fwd_pair_3x3<FwdW8S2>(x, w, w_side, y, y_side, stats, stats_side, d, s);
+}
 
 int fwd_stats_slots(const ConvDims &d) {
     switch (fwd_tiled_variant(d)) {

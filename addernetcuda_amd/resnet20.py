@@ -54,7 +54,9 @@ class BasicBlock(nn.Module):
         if self.bn1.training and x.is_cuda and x.requires_grad:
             # x leaves conv1's node a second time and feeds the shortcut from there, so that the shortcut's
             # gradient is added to conv1's input gradient by the kernel that computes it, not by a launch of its own
-            out, shortcut = adder_bn_act(self.conv1, self.bn1, x, with_shortcut=True)
+            ds = self.downsample
+            side = ds[0] if isinstance(ds, nn.Sequential) and len(ds) == 2 else None   # the strided 1x1 layer beside conv1
+            out, shortcut = adder_bn_act(self.conv1, self.bn1, x, with_shortcut=True, side_conv=side)
         else:
             out, shortcut = adder_bn_act(self.conv1, self.bn1, x), x
         if self.downsample is not None:

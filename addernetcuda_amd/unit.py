@@ -27,19 +27,31 @@ import torch
 from torch.autograd import Function
 
 from . import adder as _adder
-from ._lib import require_gpu_f32, bwd_bn_slots
+from ._lib import require_gpu_f32, bwd_bn_slots, conv_dims
 from .bn_act import BatchNormAct2d, bn_forward, bn_backward
 
 
 class _adder_bn_act(Function):
     @staticmethod
     def forward(ctx, X, W, gamma, beta, residual, running_mean, running_var, num_batches, momentum, eps, relu, stride,
-                padding, eta, with_shortcut, in_link):
+                padding, eta, with_shortcut, in_link, side_weight, given):
         ctx.w_is_given = W.is_contiguous()
         X, W = X.contiguous(), W.contiguous()
         if residual is not None:
             residual = residual.contiguous()
-        conv_out, stats, dims = _adder.conv_forward(X, W, stride, padding, True)
+        ctx.side = None
+        pair = None
+        if given is not None:      # this layer's product came out of the launch of the 3x3 layer beside it
+            conv_out, stats = given
+            dims = conv_dims(X.shape, W.shape, stride, padding)[0]
+        else:
+            if side_weight is not None and with_shortcut:
+                pair = _adder.conv_forward_pair(X, W, side_weight, stride, padding)
+            if pair is not None:
+                conv_out, stats, out_side, stats_side, dims = pair
+                ctx.side = _adder.SideOutput(X, side_weight, out_side, stats_side)
+            else:
+                conv_out, stats, dims = _adder.conv_forward(X, W, stride, padding, True)
         y, mean, rstd, mask = bn_forward(conv_out, gamma, beta, residual, running_mean, running_var, num_batches,
                                          momentum, eps, relu, stats)
         ctx.save_for_backward(X, W, conv_out, y if relu and mask is None else None, gamma, mean, rstd, mask)
@@ -59,7 +71,7 @@ class _adder_bn_act(Function):
         X, W, conv_out, y, gamma, mean, rstd, mask = ctx.saved_tensors
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if dy is None:   # only the shortcut output was used
-            return (grad_short,) + (None,) * 15
+            return (grad_short,) + (None,) * 17
         dy = dy.contiguous()
         require_gpu_f32(dy, "grad_output")
         if grad_short is not None:
@@ -79,14 +91,17 @@ class _adder_bn_act(Function):
             in_link = None
         gx, gw = _adder.conv_backward(X, W, gy, grad_short, ctx.dims, ctx.eta, need_x, need_w, ctx.w_is_given,
                                       out_link=out_link, in_link=in_link)
-        return (gx, gw, dgamma, dbeta, dres) + (None,) * 11
+        return (gx, gw, dgamma, dbeta, dres) + (None,) * 13
 
 
-def adder_bn_act(conv, bn, x, residual=None, with_shortcut=False):
+def adder_bn_act(conv, bn, x, residual=None, with_shortcut=False, side_conv=None):
     """``bn(conv(x)) [+ residual]`` followed by the ReLU of ``bn`` (a ``BatchNormAct2d``), as one autograd node where
     that is possible (training on the GPU, float32, an ``adder2d`` without bias), else as the separate modules.
     ``with_shortcut``: returns (out, shortcut) with ``shortcut`` = x routed through the node, so that a residual
-    shortcut's gradient is added inside the input-gradient kernel."""
+    shortcut's gradient is added inside the input-gradient kernel.
+    ``side_conv`` (with ``with_shortcut``): the strided 1x1 ``adder2d`` that is applied to ``shortcut`` next (the
+    downsample layer of the block): where ``conv`` is a strided 3x3 layer its kernel computes that layer's output
+    too, and the call of ``adder_bn_act(side_conv, ..., shortcut)`` finds it ready."""
     ok = (isinstance(conv, _adder.adder2d) and isinstance(bn, BatchNormAct2d) and not conv.bias and bn._fusable(x)
           and torch.is_grad_enabled() and conv.adder.dtype == torch.float32
           and (residual is None or (residual.shape[1:] == (conv.output_channel,) + _out_hw(conv, x)
@@ -105,13 +120,26 @@ def adder_bn_act(conv, bn, x, residual=None, with_shortcut=False):
     rm = bn.running_mean if bn.track_running_stats else None
     rv = bn.running_var if bn.track_running_stats else None
     nb = bn.num_batches_tracked if bn.track_running_stats else None
+    side_weight = None
+    if (with_shortcut and isinstance(side_conv, _adder.adder2d) and not side_conv.bias
+            and side_conv.adder.dtype == torch.float32 and side_conv.adder.is_contiguous()):
+        side_weight = side_conv.adder.detach()
+    given = _adder.SideOutput.of(x, conv.adder, int(conv.stride), int(conv.padding)) if residual is None else None
     res = _adder_bn_act.apply(x, conv.adder, bn.weight.contiguous(), bn.bias.contiguous(), residual, rm, rv, nb,
                               bn.momentum, bn.eps, bn.relu, int(conv.stride), int(conv.padding), conv.eta,
-                              bool(with_shortcut), _adder.BnLink.of(x))
+                              bool(with_shortcut), _adder.BnLink.of(x), side_weight, given)
     out = res[0] if with_shortcut else res
     link = getattr(out.grad_fn, "out_link", None)
     if link is not None:
         link.attach(out)
+    if with_shortcut:
+        side = getattr(out.grad_fn, "side", None)
+        if side is not None:
+            out.grad_fn.side = None
+            # (the node saw x; what travels on is its second output, another tensor object on the same memory)
+            side.x_ptr, side.x_shape, side.x_version = res[1].data_ptr(), tuple(res[1].shape), res[1]._version
+            side.w_ptr, side.w_version = side_conv.adder.data_ptr(), side_conv.adder._version
+            res[1]._adder_side_output = side
     return res
 
 

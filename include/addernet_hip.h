@@ -75,6 +75,18 @@ ADDER_API int adder_conv2d_fwd_stats_f32(const float *x, const float *w, float *
                                          int N, int Ci, int H, int W, int Co, int kh, int kw,
                                          int stride, int pad, void *stream);
 
+/* A strided 3x3 / pad 1 layer and the strided 1x1 / pad 0 layer that reads the same x beside it -- the first layer and
+ * the downsample layer of a residual block that halves the map (resnet20.py:66-70, resnet50.py:84-98 build them as two
+ * adder2d modules; adder_cuda.cpp:88-93 would run ADDER_CONV twice on two unfolded copies of x) -- in one launch:
+ * the 1x1 layer's only tap is the centre tap of the 3x3 window, which the kernel holds in registers anyway.
+ * dims describe the 3x3 layer; w_side is (Co, Ci, 1, 1); y_side and stats_side are shaped like y and stats
+ * (adder_conv2d_fwd_stats_slots slots).  Rows of whole float4 groups and even H, W, 16-byte aligned tensors;
+ * ADDER_ERR_UNSUPPORTED otherwise (optional: the two separate calls give the same results). */
+ADDER_API int adder_conv2d_fwd_pair_stats_f32(const float *x, const float *w, const float *w_side, float *y,
+                         float *y_side, double *stats, double *stats_side, int stats_slots,
+                         int N, int Ci, int H, int W, int Co, int kh, int kw,
+                         int stride, int pad, void *stream);
+
 /* An ordinary convolution y = sum w * x (no bias) through the tiled kernel of the adder forward, for the
  * regular stem layer in front of the adder layers (resnet20.py:49 uses nn.Conv2d there): 3x3 / stride 1 /
  * pad 1 only, ADDER_ERR_UNSUPPORTED (nothing launched) elsewhere.  stats (nullable) / stats_slots as in
