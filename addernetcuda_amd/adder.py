@@ -163,16 +163,20 @@ class SideOutput:
     layer and the downsample layer of a residual block that halves the map; ``adder_conv2d_fwd_pair_stats_f32``).
     Made by the 3x3 layer's node, attached to the tensor that carries x on to the 1x1 layer, and taken by that
     layer's node in place of its own forward launch if it is asked for exactly this product."""
-    __slots__ = ("x_ptr", "x_shape", "x_version", "w_ptr", "w_version", "out", "stats")
+    __slots__ = ("x_ptr", "x_shape", "x_version", "w_ptr", "w_version", "out", "stats", "side_gy", "side_w")
 
     def __init__(self, x, w, out, stats):
         self.x_ptr, self.x_shape, self.x_version = x.data_ptr(), tuple(x.shape), x._version
         self.w_ptr, self.w_version = w.data_ptr(), w._version
         self.out, self.stats = out, stats
+        # backward: the 1x1 layer's node leaves its output gradient and weights here instead of computing its input
+        # gradient, and the 3x3 layer's node, which runs after it, adds that gradient to its own (conv_backward)
+        self.side_gy = self.side_w = None
 
     @staticmethod
     def of(x, w, stride, padding):
-        """(out, stats) if ``x`` carries the product of exactly this 1x1 / stride-2 / pad-0 layer, else None."""
+        """(out, stats, the SideOutput) if ``x`` carries the product of exactly this 1x1 / stride-2 / pad-0 layer,
+        else None."""
         side = getattr(x, "_adder_side_output", None)
         if (side is None or side.out is None or stride != 2 or padding != 0 or tuple(w.shape[2:]) != (1, 1)
                 or side.x_ptr != x.data_ptr() or side.x_shape != tuple(x.shape) or side.x_version != x._version
@@ -180,7 +184,7 @@ class SideOutput:
             return None
         out, stats = side.out, side.stats
         side.out = side.stats = None   # taken once
-        return out, stats
+        return out, stats, side
 
 
 def conv_forward_pair(X, W, W_side, stride, padding):
@@ -256,15 +260,38 @@ def _aligned16(*tensors):
     return all(t is None or t.data_ptr() % 16 == 0 for t in tensors)
 
 
-def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_given, out_link=None, in_link=None):
+def side_input_grad(X, side_gy, side_w):
+    """grad_X of the strided 1x1 / pad 0 layer ``side_w`` on X, from that layer's output gradient (its own kernel)."""
+    dims1 = conv_dims(X.shape, side_w.shape, 2, 0)[0]
+    gx = torch.empty_like(X)
+    with on_device(X.device):
+        check(lib.adder_conv2d_bwd_f32(ptr(side_gy), ptr(X), ptr(side_w), ptr(gx), None, 0.0, None, 0, *dims1,
+                                       stream_ptr(X.device)), "adder_conv2d_bwd_f32")
+    return gx
+
+
+def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_given, out_link=None, in_link=None,
+                  side=None):
     """The backward launches shared by the autograd nodes: (grad_X, grad_W), either None where not needed.
 
     ``grad_short``: a second gradient of X (a residual shortcut), added to grad_X by the kernel where it can.
     ``out_link``: a BnLink whose ``coef`` is ready -- ``grad_out`` is then dz of the BatchNorm behind the layer
     (the caller has checked ``bwd_bn_slots(dims)``, the alignment of the tensors and ``need_w``).
     ``in_link``: the BnLink of the BatchNorm whose output X is -- grad_X leaves as dz, and the link receives dz,
-    coef, dgamma and dbeta (same checks by the caller, and ``need_x``)."""
+    coef, dgamma and dbeta (same checks by the caller, and ``need_x``).
+    ``side``: (side_gy, side_w) of the strided 1x1 layer that reads X beside this (strided 3x3) layer and has left its
+    input gradient to this call: added inside the input-gradient kernel where that takes ``in_link``, else computed
+    by the 1x1 layer's own kernel and added like ``grad_short``."""
     dev = X.device
+    if side is not None and need_x:
+        N, Ci, H, W_ = X.shape
+        if not (in_link is not None and H % 2 == 0 and W_ % 2 == 0 and _aligned16(*side)
+                and side[0].is_contiguous() and side[1].is_contiguous()):
+            extra = side_input_grad(X, side[0].contiguous(), side[1].contiguous())
+            grad_short = extra if grad_short is None else grad_short + extra
+            side = None
+    else:
+        side = None
     gx = torch.empty_like(X) if need_x else None
     gw = torch.empty_like(W) if need_w else None
     eta = float(eta or 0.0)
@@ -282,6 +309,8 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
             links.in_part, links.in_slots, links.in_relu = ptr(part), slots, int(in_link.relu)
             if in_link.beta is not None and in_link.beta_version == (in_link.beta._version, in_link.gamma._version):
                 links.in_gamma, links.in_beta = ptr(in_link.gamma), ptr(in_link.beta)
+            if side is not None:
+                links.side_gy, links.side_w = ptr(side[0]), ptr(side[1])
     if _eta_batch is not None and need_w and any(W is entry[0] for entry in _eta_batch):
         raise RuntimeError("batched_eta_scaling: this weight already has a pending gradient in the block "
                            "(one backward pass per block, no weight shared between layers)")

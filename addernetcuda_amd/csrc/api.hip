@@ -86,7 +86,7 @@ const char *adder_strerror(int status) {
 
 const char *adder_last_hip_error(void) { return g_last_hip_error.c_str(); }
 
-int adder_abi_version(void) { return 4; }
+int adder_abi_version(void) { return 5; }
 
 int adder_out_dim(int h, int k, int pad, int stride) {
     if (h <= 0 || k <= 0 || pad < 0 || stride <= 0 || h + 2 * pad < k) return 0;
@@ -428,6 +428,9 @@ int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, con
     if (bn.out_x && gx && !bn.out_gy) return ADDER_ERR_NULL_POINTER;   // grad_X reads the gradient grad_W leaves there
     if (bn.in_part && (!bn.in_x || !bn.in_mean || !bn.in_rstd || !gx)) return ADDER_ERR_NULL_POINTER;
     if ((bn.in_gamma == nullptr) != (bn.in_beta == nullptr)) return ADDER_ERR_NULL_POINTER;
+    if ((bn.side_gy == nullptr) != (bn.side_w == nullptr)) return ADDER_ERR_NULL_POINTER;
+    if (bn.side_gy && (!bn.in_part || kh != 3 || kw != 3 || stride != 2 || pad != 1 || (H & 1) || (W & 1)))
+        return ADDER_ERR_UNSUPPORTED;
     ConvDims d;
     if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
     const int slots = grad_w_bn_supported(d, nullptr, nullptr, nullptr, nullptr) ? grad_x_bn_slots(d) : 0;

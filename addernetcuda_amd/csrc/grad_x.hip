@@ -590,7 +590,12 @@ struct GradX3x3S2Cfg {
 };
 
 // FUSE, bn: as in the stride-1 kernel.
-template <class C, bool VEC = true, bool SAT = true, class T = float, bool FUSE = false>
+// PAIR (with FUSE): the input gradient of the strided 1x1 layer that reads the same x beside this layer (the
+// downsample branch of a residual block) is added in here: bn.side_gy is that layer's output gradient (shaped like
+// gy), bn.side_w its weights (Co, Ci).  Its one tap is the centre tap of the 3x3 window, so its gradient lands on
+// the even positions -- element (0, 0) of every lane's 2 x 2 block -- and takes the gy value of the block's own
+// output position, one float per lane and output channel, read from memory one channel ahead.
+template <class C, bool VEC = true, bool SAT = true, class T = float, bool FUSE = false, bool PAIR = false>
 __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__restrict__ gy,
                                                                    const T *__restrict__ x,
                                                                    const float *__restrict__ w,
@@ -601,6 +606,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
                                                                    const adder_bn_links bn) {
     constexpr int TNW = C::TNW, TM = C::TM, GSTRIP = C::GSTRIP;
     static_assert(!FUSE || (VEC && sizeof(T) == 4 && TM * 2 * TNW <= 32), "the BatchNorm link belongs to the float kernels");
+    static_assert(!PAIR || (FUSE && TNW == 2), "the side layer rides on the linked kernel; one 2 x 2 block per lane");
     extern __shared__ __align__(16) float smem[];
 
     int b = blockIdx.x;
@@ -653,6 +659,15 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
     const int lane_off = img * C::CC * C::PLANE + brow * C::PITCH + bcol * (TNW / 2);
     const int nchunks = ceil_div(Co, C::CC);
     const int hb = h0 / 2, wb = w0 / 2;
+    // PAIR: the side layer's gy at the lane's own output position (clamped into the tensor: what lands outside is
+    // not stored), its weights for the lane's TM channels, and the sum of its gy for the correction at the end
+    uniform_f32_ptr wsc = as_uniform(bn.side_w) + ci_base;
+    const float *gdp = nullptr;
+    float gd_next = 0.f, gd_sum = 0.f;
+    if constexpr (PAIR) {
+        gdp = bn.side_gy + ((size_t)nc * Co * Ho + min(hi0 / 2, Ho - 1)) * Wo + min(wi0 / 2, Wo - 1);
+        gd_next = gdp[0];
+    }
 
     TileStage<typename C::Patch> st;
     tile_fetch<typename C::Patch, VEC, false, T>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
@@ -677,15 +692,22 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
         constexpr int RP[3] = {0, 1, 1}, RI[3] = {1, 0, 2}, RG[3] = {0, 1, 0};
         float gr[2][2][GSTRIP];
         float wv[2][HW];
+        float wsv[2][PAIR ? TM : 1];   // PAIR: the side layer's weights of this and the next output channel
 #pragma unroll
         for (int r = 0; r < 2; ++r) lds_read_strip<GSTRIP, 1>(lbase + r * C::PITCH, gr[0][r]);
 #pragma unroll
         for (int e = 0; e < HW; ++e) wv[0][e] = wc[co0 * K + e];
+        if constexpr (PAIR) {
+#pragma unroll
+            for (int m = 0; m < TM; ++m) wsv[0][m] = wsc[co0 * Ci + m];
+        }
 
         auto one_channel = [&](const int cc, const int cur) {
             const int kofs = (co0 + cc) * K;
             const bool more = cc + 1 < ccnt;
             const int knext = more ? kofs + K : kofs;
+            float gd = 0.f;
+            if constexpr (PAIR) gd = gd_next;
 #pragma unroll
             for (int h = 0; h < NU; ++h) {
 #pragma unroll
@@ -710,9 +732,26 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
                             for (int r = 0; r < 2; ++r)
                                 lds_read_strip<GSTRIP, 1>(lbase + (cc + 1) * C::PLANE + r * C::PITCH, gr[cur ^ 1][r]);
                         }
+                        if constexpr (PAIR) {
+                            if (h == 0) {   // the next output channel's side operands (the last one asks for itself again)
+                                const int cn = min(co0 + cc + 1, Co - 1);
+                                gd_next = gdp[(size_t)cn * Ho * Wo];
+#pragma unroll
+                                for (int m2 = 0; m2 < TM; ++m2) wsv[cur ^ 1][m2] = wsc[cn * Ci + m2];
+                            }
+                        }
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
+            }
+            if constexpr (PAIR) {
+#pragma unroll
+                for (int m = 0; m < TM; ++m) {
+                    const float wgt = wsv[cur][m];
+                    const float d = SAT ? sat01(fmaf(wgt, 0.5f, cr[m][0][0])) : hardtanh(wgt - cr[m][0][0]);
+                    acc[m][0][0] = fmaf(d, gd, acc[m][0][0]);
+                }
+                gd_sum += gd;
             }
         };
 #pragma unroll 1
@@ -794,6 +833,10 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
             for (int rp = 0; rp < 2; ++rp)
 #pragma unroll
                 for (int t = 0; t < TNW; ++t) tot[m][rp][t] = fmaf(2.f, tot[m][rp][t], -sg[rp][t]);
+        if constexpr (PAIR) {   // the side layer's terms met the even position only
+#pragma unroll
+            for (int m = 0; m < TM; ++m) tot[m][0][0] -= gd_sum;
+        }
     }
 
     if constexpr (FUSE) {
@@ -895,7 +938,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
     }
 }
 
-template <class C, bool VEC, bool SAT, class T = float, bool FUSE = false>
+template <class C, bool VEC, bool SAT, class T = float, bool FUSE = false, bool PAIR = false>
 static int launch_grad_x_3x3s2_v(const T *gy, const T *x, const float *w, T *gx,
                                const ConvDims &d, hipStream_t s, const T *gadd, const adder_bn_links &bn = kNoLinks) {
     const int tilesH = ceil_div(d.H, C::TH), tilesW = ceil_div(d.W, C::TW);
@@ -905,14 +948,19 @@ static int launch_grad_x_3x3s2_v(const T *gy, const T *x, const float *w, T *gx,
     if (FUSE && (!bn.in_part || bn.in_slots != gxd * C::POSW)) return ADDER_ERR_BAD_SHAPE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
-    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T, FUSE>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS), LDS_BYTES, s,
-                       gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, gadd, bn);
+    hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T, FUSE, PAIR>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS),
+                       LDS_BYTES, s, gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, gadd, bn);
     return check_launch();
 }
 
 template <class C>
 static int launch_grad_x_3x3s2_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                                   hipStream_t s, const float *gadd, const adder_bn_links &bn) {
+    if (bn.side_gy) {   // (H, W even: the two layers' outputs have one size)
+        if (d.Co * 4 > kSatMaxTerms)
+            return launch_grad_x_3x3s2_v<C, true, false, float, true, true>(gy, x, w, gx, d, s, gadd, bn);
+        return launch_grad_x_3x3s2_v<C, true, true, float, true, true>(gy, x, w, gx, d, s, gadd, bn);
+    }
     if (d.Co * 4 > kSatMaxTerms) return launch_grad_x_3x3s2_v<C, true, false, float, true>(gy, x, w, gx, d, s, gadd, bn);
     return launch_grad_x_3x3s2_v<C, true, true, float, true>(gy, x, w, gx, d, s, gadd, bn);
 }

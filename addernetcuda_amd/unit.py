@@ -39,23 +39,24 @@ class _adder_bn_act(Function):
         X, W = X.contiguous(), W.contiguous()
         if residual is not None:
             residual = residual.contiguous()
-        ctx.side = None
+        ctx.side = ctx.pair = None
         pair = None
         if given is not None:      # this layer's product came out of the launch of the 3x3 layer beside it
-            conv_out, stats = given
+            conv_out, stats, ctx.pair = given
             dims = conv_dims(X.shape, W.shape, stride, padding)[0]
         else:
             if side_weight is not None and with_shortcut:
                 pair = _adder.conv_forward_pair(X, W, side_weight, stride, padding)
             if pair is not None:
                 conv_out, stats, out_side, stats_side, dims = pair
-                ctx.side = _adder.SideOutput(X, side_weight, out_side, stats_side)
+                ctx.side = ctx.pair = _adder.SideOutput(X, side_weight, out_side, stats_side)
             else:
                 conv_out, stats, dims = _adder.conv_forward(X, W, stride, padding, True)
         y, mean, rstd, mask = bn_forward(conv_out, gamma, beta, residual, running_mean, running_var, num_batches,
                                          momentum, eps, relu, stats)
         ctx.save_for_backward(X, W, conv_out, y if relu and mask is None else None, gamma, mean, rstd, mask)
         ctx.dims, ctx.eta, ctx.relu, ctx.has_res = dims, eta, relu, residual is not None
+        ctx.with_shortcut = with_shortcut
         ctx.in_link = in_link
         # (a layer without the kernels that take the link could not use what its consumer would prepare)
         ctx.out_link = (_adder.BnLink(conv_out, mean, rstd, gamma, relu, None if residual is not None else beta)
@@ -70,7 +71,15 @@ class _adder_bn_act(Function):
     def backward(ctx, dy, grad_short=None):
         X, W, conv_out, y, gamma, mean, rstd, mask = ctx.saved_tensors
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        pair, ctx.pair = ctx.pair, None
+        side = None
+        if pair is not None and ctx.with_shortcut and pair.side_gy is not None:
+            # the strided 1x1 layer beside this one has left its input gradient to this node
+            side, pair.side_gy, pair.side_w = (pair.side_gy, pair.side_w), None, None
         if dy is None:   # only the shortcut output was used
+            if side is not None and need_x:
+                extra = _adder.side_input_grad(X, *side)
+                grad_short = extra if grad_short is None else grad_short + extra
             return (grad_short,) + (None,) * 17
         dy = dy.contiguous()
         require_gpu_f32(dy, "grad_output")
@@ -89,8 +98,12 @@ class _adder_bn_act(Function):
             out_link.dz = None   # (the tensor is kept alive by autograd for as long as it is needed)
         if not (usable and need_x and in_link is not None and X.data_ptr() == in_link.out_ptr):
             in_link = None
+        if pair is not None and not ctx.with_shortcut and need_x and X.is_contiguous():
+            # this is the 1x1 layer of the pair: its input gradient is left to the 3x3 layer's node, which runs next
+            pair.side_gy, pair.side_w = gy.contiguous(), W
+            need_x = False
         gx, gw = _adder.conv_backward(X, W, gy, grad_short, ctx.dims, ctx.eta, need_x, need_w, ctx.w_is_given,
-                                      out_link=out_link, in_link=in_link)
+                                      out_link=out_link, in_link=in_link, side=side)
         return (gx, gw, dgamma, dbeta, dres) + (None,) * 13
 
 
@@ -101,7 +114,10 @@ def adder_bn_act(conv, bn, x, residual=None, with_shortcut=False, side_conv=None
     shortcut's gradient is added inside the input-gradient kernel.
     ``side_conv`` (with ``with_shortcut``): the strided 1x1 ``adder2d`` that is applied to ``shortcut`` next (the
     downsample layer of the block): where ``conv`` is a strided 3x3 layer its kernel computes that layer's output
-    too, and the call of ``adder_bn_act(side_conv, ..., shortcut)`` finds it ready."""
+    too, and the call of ``adder_bn_act(side_conv, ..., shortcut)`` finds it ready.  In the backward pass that
+    layer's node then leaves its input gradient to this node (``adder.SideOutput``), whose strided input-gradient
+    kernel adds it on the positions the 1x1 layer read -- so ``shortcut`` is for ``side_conv`` and nothing else:
+    a gradient taken with respect to ``shortcut`` itself would miss that part."""
     ok = (isinstance(conv, _adder.adder2d) and isinstance(bn, BatchNormAct2d) and not conv.bias and bn._fusable(x)
           and torch.is_grad_enabled() and conv.adder.dtype == torch.float32
           and (residual is None or (residual.shape[1:] == (conv.output_channel,) + _out_hw(conv, x)

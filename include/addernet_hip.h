@@ -329,6 +329,12 @@ typedef struct adder_bn_links {
        |gamma| < max(1, |beta|) / 64 and the stride-2 kernels read it). */
     const float *in_gamma;
     const float *in_beta;
+    /* optional, both or neither, with the in_* half, for a 3x3 / stride 2 / pad 1 layer on a map of even height and
+       width: the strided 1x1 / pad 0 layer that reads the same x beside this one (resnet20.py:66-70).  side_gy is
+       that layer's output gradient (N, Co, Ho, Wo), side_w its weights (Co, Ci): its input gradient is added to
+       grad_X inside the kernel (before the mask and the sums), as if it had been passed as gx_add. */
+    const float *side_gy;
+    const float *side_w;
 } adder_bn_links;
 ADDER_API int adder_conv2d_bwd_bn_slots(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad,
                                         int *slots);

@@ -66,6 +66,96 @@ def test_pair_refusals(gpu):
                                                stream_ptr(gpu)) == -1
 
 
+@pytest.mark.parametrize("case", [(6, 16, 32, 32, 32), (5, 32, 16, 16, 64), (3, 128, 8, 8, 130), (2, 8, 64, 64, 8),
+                                  (4, 8, 8, 8, 600)], ids=str)   # the last one: the three-instruction form
+@pytest.mark.parametrize("with_add", [False, True])
+def test_side_input_gradient_inside_the_strided_kernel(case, with_add, gpu):
+    """adder_bn_links.side_gy / side_w: the strided 1x1 layer's input gradient added inside the strided 3x3 layer's
+    linked input-gradient kernel, against the same call with that gradient computed by the 1x1 layer's own kernel
+    (held to the oracle in test_gpu_parity_nchw.py) and passed as gx_add."""
+    from addernetcuda_amd._lib import lib, check, ptr, stream_ptr, conv_dims, BnLinks, bwd_bn_slots
+    N, Ci, H, W, Co = case
+    g = torch.Generator(device=gpu).manual_seed(sum(case))
+    b = lambda v: v[None, :, None, None]
+    bn_in = torch.randn(N, Ci, H, W, device=gpu, generator=g) * 20 - 90
+    mean, rstd = bn_in.mean((0, 2, 3)), 1.0 / bn_in.std((0, 2, 3))
+    x = torch.relu((bn_in - b(mean)) * b(rstd) + torch.randn(N, Ci, H, W, device=gpu, generator=g))
+    w = torch.randn(Co, Ci, 3, 3, device=gpu, generator=g) * 0.3
+    ws = torch.randn(Co, Ci, 1, 1, device=gpu, generator=g) * 0.3
+    dims, Ho, Wo = conv_dims(x.shape, w.shape, 2, 1)
+    dims1, _, _ = conv_dims(x.shape, ws.shape, 2, 0)
+    gy = torch.randn(N, Co, Ho, Wo, device=gpu, generator=g)
+    gyd = torch.randn(N, Co, Ho, Wo, device=gpu, generator=g)
+    more = torch.randn(x.shape, device=gpu, generator=g) if with_add else None
+    slots = bwd_bn_slots(dims)
+    assert slots > 0
+    st = stream_ptr(gpu)
+    gxd, gxa, gxb = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    pa = torch.empty(Ci, slots, 2, dtype=torch.float64, device=gpu)
+    pb = torch.full_like(pa, float("nan"))
+    la = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(pa), slots, 1)
+    lb = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(pb), slots, 1, None, None, ptr(gyd), ptr(ws))
+    check(lib.adder_conv2d_bwd_f32(ptr(gyd), ptr(x), ptr(ws), ptr(gxd), None, 0.0, None, 0, *dims1, st), "1x1 grad_X")
+    add = gxd + more if with_add else gxd
+    check(lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), ptr(add), ptr(gxa), None, 0.0, None, 0, *dims,
+                                      ctypes.byref(la), st), "gx_add")
+    check(lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), ptr(more), ptr(gxb), None, 0.0, None, 0, *dims,
+                                      ctypes.byref(lb), st), "side")
+    torch.cuda.synchronize()
+    assert_close(gxb, gxa, f"dz {case}", rtol=1e-5, atol=1e-4)
+    scale = max(1.0, float(pa.sum(1).abs().max()))
+    assert_close(pb.sum(1) / scale, pa.sum(1) / scale, f"sums {case}", rtol=1e-6, atol=1e-6)
+    # refusals: one of the two pointers, no in-links, a stride-1 layer
+    lc = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(pb), slots, 1, None, None, ptr(gyd), None)
+    assert lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gxb), None, 0.0, None, 0, *dims,
+                                       ctypes.byref(lc), st) == -1
+    ld = BnLinks(None, None, None, None, None, None, None, 0, 0, None, None, ptr(gyd), ptr(ws))
+    assert lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gxb), None, 0.0, None, 0, *dims,
+                                       ctypes.byref(ld), st) == -7
+
+
+def test_pair_in_a_chain_of_units(gpu, monkeypatch):
+    """A unit in front of a block that halves the map, so that the block's first layer has a BatchNorm link on its
+    input and the 1x1 layer's input gradient is added inside its strided kernel: gradients against the same
+    network with the pair switched off."""
+    from addernetcuda_amd import adder, resnet20
+    from addernetcuda_amd.bn_act import BatchNormAct2d
+    from addernetcuda_amd.unit import adder_bn_act
+    import torch.nn as nn
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            torch.manual_seed(5)
+            self.conv0 = adder.adder2d(8, 16, kernel_size=3, stride=1, padding=1, bias=False)
+            self.bn0 = BatchNormAct2d(16, relu=True)
+            ds = nn.Sequential(adder.adder2d(16, 32, kernel_size=1, stride=2, padding=0, bias=False),
+                               BatchNormAct2d(32, relu=False))
+            self.block = resnet20.BasicBlock(16, 32, stride=2, downsample=ds)
+
+        def forward(self, x):
+            return self.block(adder_bn_act(self.conv0, self.bn0, x))
+
+    x = torch.randn(6, 8, 16, 16, device=gpu)
+    gy = torch.randn(6, 32, 8, 8, device=gpu)
+    used = []
+    orig = adder.conv_backward
+    monkeypatch.setattr(adder, "conv_backward", lambda *a, **k: used.append(k.get("side")) or orig(*a, **k))
+    a = Net().to(gpu).train()
+    xa = x.clone().requires_grad_(True)
+    a(xa).backward(gy)
+    assert sum(u is not None for u in used) == 1          # the 3x3 layer's call carried the 1x1 layer's gradient
+    monkeypatch.setattr(adder, "conv_forward_pair", lambda *args: None)
+    used.clear()
+    b = Net().to(gpu).train()
+    xb = x.clone().requires_grad_(True)
+    b(xb).backward(gy)
+    assert all(u is None for u in used)
+    assert_close(xa.grad, xb.grad, "input gradient", rtol=1e-4, atol=1e-4)
+    for (n, p), (_, q) in zip(a.named_parameters(), b.named_parameters()):
+        assert_close(p.grad, q.grad, n, rtol=1e-4, atol=1e-4)
+
+
 def test_block_hands_the_side_output_over(gpu, monkeypatch):
     """The first block of a ResNet-20 stage: conv1's launch also computes the downsample layer's output, the
     downsample node takes it instead of launching its own kernel, and nothing changes in what the block computes."""
