@@ -174,7 +174,7 @@ class VGGSmall(nn.Module):
 
 
 def vgg_small(**kwargs):
-    """The BASELINE configuration "VGG-small-style AdderNet" (128-128-M-256-256-M-512-512-M, batch 128).  It is a
+    """The benchmark configuration "VGG-small-style AdderNet" (128-128-M-256-256-M-512-512-M, batch 128).  It is a
     harness for those layer shapes, not one of vgg.py's networks: its keys and its 8192-wide classifier match no
     reference VGG checkpoint -- for those use the ``vgg11`` ... ``vgg19_bn`` factories below."""
     return VGGSmall(**kwargs)

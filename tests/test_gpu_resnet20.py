@@ -53,7 +53,7 @@ def test_one_step_matches_the_unfold_reference_path(gpu):
     assert statistics.median(rel.values()) <= 0.02, sorted(rel.items(), key=lambda kv: -kv[1])[:5]
 
 
-BATCH, STEPS = 256, 50     # BASELINE config 3: batch 256, 50 steps, SGD momentum 0.9, eta 0.1
+BATCH, STEPS = 256, 50     # the third benchmark configuration: batch 256, 50 steps, SGD momentum 0.9, eta 0.1
 
 
 def _sgd(model):
