@@ -206,3 +206,26 @@ def test_block_hands_the_side_output_over(gpu, monkeypatch):
     assert orig(shortcut.clone(), c.downsample[0].adder, 2, 0) is None     # ... another tensor
     assert orig(shortcut, c.downsample[0].adder, 2, 0) is not None
     assert orig(shortcut, c.downsample[0].adder, 2, 0) is None             # taken once
+
+
+def test_second_backward_through_a_retained_graph(gpu):
+    """The hand-over between the two nodes is used once; a second backward pass through a retained graph takes the
+    plain path and must deliver the same gradients again."""
+    from addernetcuda_amd import adder, resnet20
+    from addernetcuda_amd.bn_act import BatchNormAct2d
+    import torch.nn as nn
+    torch.manual_seed(2)
+    ds = nn.Sequential(adder.adder2d(16, 32, kernel_size=1, stride=2, padding=0, bias=False), BatchNormAct2d(32, relu=False))
+    block = resnet20.BasicBlock(16, 32, stride=2, downsample=ds).to(gpu).train()
+    x = torch.randn(4, 16, 16, 16, device=gpu, requires_grad=True)
+    gy = torch.randn(4, 32, 8, 8, device=gpu)
+    y = block(x)
+    y.backward(gy, retain_graph=True)
+    first = [x.grad.clone()] + [p.grad.clone() for p in block.parameters()]
+    x.grad = None
+    for p in block.parameters():
+        p.grad = None
+    y.backward(gy)
+    second = [x.grad] + [p.grad for p in block.parameters()]
+    for a, b in zip(first, second):
+        assert_close(b, a, "second pass", rtol=1e-4, atol=1e-4)
