@@ -480,7 +480,8 @@ def main():
         "config": {"workload": "ResNet-20 AdderNet, batch 256, 3x32x32, 10 classes, SGD momentum 0.9 lr 0.1 wd 5e-4, "
                                "adaptive eta 0.1, fwd+bwd+optimizer; BatchNorm / ReLU / residual add run as this "
                                "library's fused kernels (BatchNormAct2d), the BatchNorm backward passes inside the "
-                               "adder backward kernels on either side of each BatchNorm (unit.py), and the regular "
+                               "adder backward kernels on either side of each BatchNorm (unit.py), the strided 1x1 downsample "
+                               "layers inside the strided 3x3 kernels beside them (forward and grad_X), and the regular "
                                "3->16 stem convolution through the tiled forward / slab weight-gradient kernels "
                                "(StemConv2d); the same step with stock torch modules is other_configs[0]",
                    "step_mode": mode},
