@@ -102,6 +102,14 @@ class _adder_bn_act(Function):
             # this is the 1x1 layer of the pair: its input gradient is left to the 3x3 layer's node, which runs next
             pair.side_gy, pair.side_w = gy.contiguous(), W
             need_x = False
+
+            def collected(pair=pair):   # runs when this backward pass is over
+                if pair.side_gy is not None:
+                    pair.side_gy = pair.side_w = None
+                    raise RuntimeError("adder_bn_act: the input gradient of a paired 1x1 layer was left to the 3x3 layer "
+                                       "beside it, whose backward did not run in this pass (differentiate with respect "
+                                       "to the block's input, not to the `shortcut` tensor between the two layers)")
+            torch.autograd.Variable._execution_engine.queue_callback(collected)
         gx, gw = _adder.conv_backward(X, W, gy, grad_short, ctx.dims, ctx.eta, need_x, need_w, ctx.w_is_given,
                                       out_link=out_link, in_link=in_link, side=side)
         return (gx, gw, dgamma, dbeta, dres) + (None,) * 13

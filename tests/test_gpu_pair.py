@@ -229,3 +229,20 @@ def test_second_backward_through_a_retained_graph(gpu):
     second = [x.grad] + [p.grad for p in block.parameters()]
     for a, b in zip(first, second):
         assert_close(b, a, "second pass", rtol=1e-4, atol=1e-4)
+
+
+def test_uncollected_side_gradient_is_an_error(gpu):
+    """Differentiating with respect to the tensor between the two layers of a pair would silently miss the 1x1
+    layer's part (it is left to the 3x3 layer's node): that must be an error, not a wrong number."""
+    from addernetcuda_amd import adder
+    from addernetcuda_amd.bn_act import BatchNormAct2d
+    from addernetcuda_amd.unit import adder_bn_act
+    torch.manual_seed(4)
+    conv1 = adder.adder2d(16, 32, kernel_size=3, stride=2, padding=1, bias=False).to(gpu)
+    side = adder.adder2d(16, 32, kernel_size=1, stride=2, padding=0, bias=False).to(gpu)
+    bn1, bns = BatchNormAct2d(32, relu=True).to(gpu).train(), BatchNormAct2d(32, relu=False).to(gpu).train()
+    x = torch.randn(4, 16, 16, 16, device=gpu, requires_grad=True)
+    out, shortcut = adder_bn_act(conv1, bn1, x, with_shortcut=True, side_conv=side)
+    ys = adder_bn_act(side, bns, shortcut)
+    with pytest.raises(RuntimeError, match="paired 1x1 layer"):
+        torch.autograd.grad(ys.sum(), shortcut)
