@@ -16,6 +16,10 @@ if not os.path.exists(LIB_PATH):
 
 lib = ctypes.CDLL(LIB_PATH)
 
+# adder_status of include/addernet_hip.h
+ADDER_OK, ADDER_ERR_NULL_POINTER, ADDER_ERR_BAD_SHAPE, ADDER_ERR_TOO_LARGE = 0, -1, -2, -3
+ADDER_ERR_WORKSPACE, ADDER_ERR_HIP, ADDER_ERR_ALIAS, ADDER_ERR_UNSUPPORTED = -4, -5, -6, -7
+
 _i, _l, _f, _p, _sz = ctypes.c_int, ctypes.c_long, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 _szp = ctypes.POINTER(ctypes.c_size_t)
 
@@ -84,7 +88,7 @@ def check(status, what):
     """Turn a negative adder_status into the RuntimeError the reference's AT_ASSERTM would raise."""
     if status != 0:
         msg = lib.adder_strerror(status).decode()
-        if status == -5:
+        if status == ADDER_ERR_HIP:
             msg += ": " + lib.adder_last_hip_error().decode()
         raise RuntimeError(f"{what}: {msg}")
 

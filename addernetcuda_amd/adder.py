@@ -19,7 +19,8 @@ from torch.autograd import Function
 
 from . import adder_cuda
 from ._lib import (lib, check, ptr, require_gpu_f32, require_gpu_bf16, same_device, stream_ptr, conv_dims,
-                   conv2d_bwd_workspace, fwd_stats_slots, on_device, GradWStage, BnLinks, bwd_bn_slots)
+                   conv2d_bwd_workspace, fwd_stats_slots, on_device, GradWStage, BnLinks, bwd_bn_slots,
+                   ADDER_OK, ADDER_ERR_UNSUPPORTED)
 
 DEFAULT_ETA = 0.2  # adder.py:78 divides by 5
 
@@ -149,7 +150,7 @@ def conv_forward(X, W, stride, padding, with_stats):
         if slots > 0:
             stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64)
             status = lib.adder_conv2d_fwd_stats_f32(ptr(X), ptr(W), ptr(out), ptr(stats), slots, *dims, stream_ptr(dev))
-            if status == -7:   # e.g. tensors that are not 16-byte aligned: the kernel that sums was turned down
+            if status == ADDER_ERR_UNSUPPORTED:   # e.g. tensors that are not 16-byte aligned: the kernel that sums was turned down
                 stats, slots = None, 0
             else:
                 check(status, "adder_conv2d_fwd_stats_f32")
@@ -208,7 +209,7 @@ def conv_forward_pair(X, W, W_side, stride, padding):
         stats_side = torch.empty_like(stats)
         status = lib.adder_conv2d_fwd_pair_stats_f32(ptr(X), ptr(W), ptr(W_side), ptr(out), ptr(out_side), ptr(stats),
                                                      ptr(stats_side), slots, *dims, stream_ptr(dev))
-        if status == -7:
+        if status == ADDER_ERR_UNSUPPORTED:
             return None
         check(status, "adder_conv2d_fwd_pair_stats_f32")
     return out, stats, out_side, stats_side, dims
@@ -329,7 +330,7 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
         if status == 0:      # slabs only; finished with all the others when the block ends
             _eta_batch.append((W, eta, stage, ws))
             staged = True
-        elif status != -7 or out_link is not None:
+        elif status != ADDER_ERR_UNSUPPORTED or out_link is not None:
             check(status, "adder_conv2d_grad_w_staged_f32")
         elif eta > 0.0:      # no slab kernel for this layer: raw gradient now, scaled when the block ends
             _eta_batch.append((W, eta, None, None))
@@ -353,7 +354,7 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
                     status = lib.adder_conv2d_bwd_add_f32(ptr(grad_out), ptr(X), ptr(W), ptr(grad_short), ptr(gx),
                                                           ptr(gw), eta, ptr(ws), nbytes, *dims, stream_ptr(dev))
                     fused = status == 0
-                    if status not in (0, -7):   # -7: this layer's grad_X kernel has no fused add
+                    if status not in (ADDER_OK, ADDER_ERR_UNSUPPORTED):   # unsupported: this layer's grad_X kernel has no fused add
                         check(status, "adder_conv2d_bwd_add_f32")
                 if not fused:
                     check(lib.adder_conv2d_bwd_f32(ptr(grad_out), ptr(X), ptr(W), ptr(gx), ptr(gw), eta, ptr(ws), nbytes,
@@ -471,7 +472,7 @@ def plain_conv2d_forward(X, W, stride, padding):
         y = torch.empty((X.size(0), W.size(0), Ho, Wo), device=dev, dtype=torch.float32)
         stats = torch.empty((W.size(0), slots, 2), device=dev, dtype=torch.float64) if slots else None
         status = lib.adder_plain_conv2d_fwd_f32(ptr(X), ptr(W), ptr(y), ptr(stats), slots, *dims, stream_ptr(dev))
-    if status == -7:
+    if status == ADDER_ERR_UNSUPPORTED:
         return None, None
     check(status, "adder_plain_conv2d_fwd_f32")
     return y, stats
@@ -503,7 +504,7 @@ def conv2d_weight_grad(grad_out, X, W, stride, padding, out_link=None):
         else:
             status = lib.adder_conv2d_grad_w_staged_f32(ptr(grad_out), ptr(X), None, ptr(gw), 0.0, ptr(ws), nbytes,
                                                         *dims, ctypes.byref(stage), stream_ptr(dev))
-        if status == -7:
+        if status == ADDER_ERR_UNSUPPORTED:
             return None
         check(status, "adder_conv2d_grad_w_staged_f32")
         if (_eta_batch is not None and W.is_leaf and W.grad is None and W.is_contiguous()

@@ -439,11 +439,15 @@ int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, con
     const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
                  ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo, np = sizeof(double) * 2 * (size_t)Ci * slots,
                  nc = 16 * (size_t)Co;
-    const void *ins[] = {gy, x, w, gx_add, bn.out_x, bn.out_coef, bn.in_x, bn.in_mean, bn.in_rstd};
-    const size_t in_bytes[] = {ny, nx, nw, nx, ny, nc, nx, 4 * (size_t)Ci, 4 * (size_t)Ci};
+    const void *ins[] = {gy, x, w, gx_add, bn.out_x, bn.out_coef, bn.in_x, bn.in_mean, bn.in_rstd,
+                         bn.in_gamma, bn.in_beta, bn.side_gy, bn.side_w};
+    const size_t in_bytes[] = {ny, nx, nw, nx, ny, nc, nx, 4 * (size_t)Ci, 4 * (size_t)Ci,
+                               4 * (size_t)Ci, 4 * (size_t)Ci, ny, sizeof(float) * (size_t)Co * Ci};
+    constexpr int kIns = sizeof(ins) / sizeof(ins[0]);
+    static_assert(kIns == sizeof(in_bytes) / sizeof(in_bytes[0]), "one size per input");
     const size_t need = gw ? grad_w_workspace_bytes(d) : 0;
     if (gw && (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255))) return ADDER_ERR_WORKSPACE;
-    for (int i = 0; i < 9; ++i)
+    for (int i = 0; i < kIns; ++i)
         if (overlaps(gx, nx, ins[i], in_bytes[i]) || overlaps(gw, nw, ins[i], in_bytes[i]) ||
             overlaps(bn.in_part, np, ins[i], in_bytes[i]) || overlaps(bn.out_gy, ny, ins[i], in_bytes[i]) ||
             (gw && overlaps(ws, need, ins[i], in_bytes[i])))

@@ -315,7 +315,9 @@ __global__ __launch_bounds__(256) void col_bwd_fused_kernel(const float *__restr
         if (active)
             *reinterpret_cast<float2 *>(gX + (size_t)(k0 + kk) * NL + c0) =
                 make_float2(old.x + fmaf(2.f, a0, -s2[0]), old.y + fmaf(2.f, a1, -s2[1]));
-        *reinterpret_cast<float2 *>(mine + (kk & 15) * kFusedPitch + 2 * lane) = xv;   // for the weight gradient
+        // for the weight gradient; idle lanes (columns past NL, re-pointed at the last two) stage zeros, so that a
+        // non-finite X there cannot reach the products of every row through 0 * Inf
+        *reinterpret_cast<float2 *>(mine + (kk & 15) * kFusedPitch + 2 * lane) = active ? xv : make_float2(0.f, 0.f);
     };
     auto ld2 = [&](const float *base, int kk) {
         return *reinterpret_cast<const float2 *>(base + (size_t)(k0 + min(kk, kcnt - 1)) * NL + c0);

@@ -399,10 +399,26 @@ using FwdW8S2L = Tile3x3Cfg<2, 4, 8, 2, 4, 8, 8, 1, 2>;
 // channels (8 weights, 64 vector instructions), eight output-channel waves share the staged x tile.
 using Fwd1x1   = Tile3x3Cfg<4, 64, 1, 1, 4, 8, 16, 8, 1, 1>;   // 256 positions of one image x 32 channels
 using Fwd1x1s  = Tile3x3Cfg<4, 16, 1, 4, 4, 8, 16, 8, 1, 1>;   // planes of <= 64 positions: four images
+// 1x1 with a stride: the tile loader gathers the sampled x element by element, which costs several times what the
+// aligned float4 loads of a stride-1 plane cost, so a workgroup takes 64 output channels per staged tile instead of
+// 32 (eight per lane, chunks of eight input channels to stay within 128 registers); ResNet-50's three downsample
+// layers at batch 64: 538 -> 319, 621 -> 376, 591 -> 374 us.  (On stride-1 planes this shape is slower.)
+using Fwd1x1sub = Tile3x3Cfg<4, 16, 1, 4, 8, 8, 8, 8, 1, 1>;   // 64 sampled positions of four images x 64 channels
 // the same two with units of four input channels, for channel counts that are multiples of 4 but not of 8
 // (DenseNet's multiples of 12)
 using Fwd1x1q  = Tile3x3Cfg<4, 64, 1, 1, 4, 8, 16, 4, 1, 1>;
 using Fwd1x1sq = Tile3x3Cfg<4, 16, 1, 4, 4, 8, 16, 4, 1, 1>;
+
+// ... the same register tile in workgroups of four waves that cover fewer rows, for maps whose height is not a
+// multiple of 16: 56 rows are 7 x 8, 28 rows 7 x 4 (ResNet-50 at batch 64: 64 -> 64 @56x56 340 -> 294 us,
+// 128 -> 128 @28x28 330 -> 298 us); on 32 rows they are no faster than FwdW32
+using FwdW32H8 = Tile3x3Cfg<4, 8, 8, 1, 4, 4, 8, 1, 1>;    // 8 rows of one image x 16 channels
+using FwdW32H4 = Tile3x3Cfg<4, 8, 4, 2, 4, 4, 8, 1, 1>;    // 4 rows of two images x 16 channels
+// rows per tile (16, 8 or 4) that pad a map of H rows least; the larger tile on a tie
+static int rows_per_tile_w32(int H) {
+    const int p16 = round_up(H, 16), p8 = round_up(H, 8), p4 = round_up(H, 4);
+    return p16 <= p8 && p16 <= p4 ? 16 : (p8 <= p4 ? 8 : 4);
+}
 
 // which tiled kernel serves these dimensions (0 = none): 1..3 3x3 stride 1 by output width, 4..5 3x3 stride 2,
 // 6..7 1x1 stride 1 by plane size, 8..9 1x1 with a stride (the sampled positions walked like a stride-1 plane),
@@ -465,15 +481,18 @@ int launch_fwd_pair(const float *x, const float *w, const float *w_side, float *
 
 int fwd_stats_slots(const ConvDims &d) {
     switch (fwd_tiled_variant(d)) {
-        case 1: return stats_slots_3x3<FwdW32>(d);
+        case 1: switch (rows_per_tile_w32(d.Ho)) {
+            case 16: return stats_slots_3x3<FwdW32>(d);
+            case 8: return stats_slots_3x3<FwdW32H8>(d);
+            default: return stats_slots_3x3<FwdW32H4>(d);
+        }
         case 2: return stats_slots_3x3<FwdW16>(d);
         case 3: return stats_slots_3x3<FwdW8>(d);
         case 4: return stats_slots_3x3<FwdW16S2>(d);
         case 5: return stats_slots_3x3<FwdW8S2>(d);
         case 6: return stats_slots_3x3<Fwd1x1>(as_one_row(d));
         case 7: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
-        case 8: return stats_slots_3x3<Fwd1x1>(as_one_row(d));
-        case 9: return stats_slots_3x3<Fwd1x1s>(as_one_row(d));
+        case 8: case 9: return stats_slots_3x3<Fwd1x1sub>(as_one_row(d));
         case 10: return stats_slots_3x3<Fwd1x1q>(as_one_row(d));
         case 11: return stats_slots_3x3<Fwd1x1sq>(as_one_row(d));
         case 12: return stats_slots_3x3<Fwd1x1q>(as_one_row(d));
@@ -493,8 +512,7 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
     if (strided) {   // x is read element by element; y is a dense row per plane
         const ConvDims f = as_one_row(d);
         if (f.Wo % 4 != 0 || (reinterpret_cast<uintptr_t>(y) & 15) == 0) switch (variant) {
-            case 8: return launch_fwd_3x3_v<Fwd1x1, false, true>(x, w, y, stats, f, s, sampling_of(d));
-            case 9: return launch_fwd_3x3_v<Fwd1x1s, false, true>(x, w, y, stats, f, s, sampling_of(d));
+            case 8: case 9: return launch_fwd_3x3_v<Fwd1x1sub, false, true>(x, w, y, stats, f, s, sampling_of(d));
             case 12: return launch_fwd_3x3_v<Fwd1x1q, false, true>(x, w, y, stats, f, s, sampling_of(d));
             default: return launch_fwd_3x3_v<Fwd1x1sq, false, true>(x, w, y, stats, f, s, sampling_of(d));
         }
@@ -509,7 +527,11 @@ int launch_fwd(const float *x, const float *w, float *y, double *stats, const Co
     }
     if (k3p1) {
         switch (variant) {
-            case 1: return launch_fwd_3x3<FwdW32>(x, w, y, stats, d, s);
+            case 1: switch (rows_per_tile_w32(d.Ho)) {
+                case 16: return launch_fwd_3x3<FwdW32>(x, w, y, stats, d, s);
+                case 8: return launch_fwd_3x3<FwdW32H8>(x, w, y, stats, d, s);
+                default: return launch_fwd_3x3<FwdW32H4>(x, w, y, stats, d, s);
+            }
             case 2: return launch_fwd_3x3<FwdW16>(x, w, y, stats, d, s);
             case 3: return launch_fwd_3x3<FwdW8>(x, w, y, stats, d, s);
             case 4: return launch_fwd_3x3<FwdW16S2>(x, w, y, stats, d, s);
@@ -562,7 +584,11 @@ int launch_mulconv_fwd(const float *x, const float *w, float *y, double *stats, 
                     (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0);
     if (!ok) return ADDER_ERR_UNSUPPORTED;
     switch (fwd_tiled_variant(d)) {
-        case 1: return launch_mulconv_3x3<FwdW32>(x, w, y, stats, d, s);
+        case 1: switch (rows_per_tile_w32(d.Ho)) {   // (the statistics slots are counted per tile shape)
+            case 16: return launch_mulconv_3x3<FwdW32>(x, w, y, stats, d, s);
+            case 8: return launch_mulconv_3x3<FwdW32H8>(x, w, y, stats, d, s);
+            default: return launch_mulconv_3x3<FwdW32H4>(x, w, y, stats, d, s);
+        }
         case 2: return launch_mulconv_3x3<FwdW16>(x, w, y, stats, d, s);
         case 3: return launch_mulconv_3x3<FwdW8>(x, w, y, stats, d, s);
         default: return ADDER_ERR_UNSUPPORTED;

@@ -998,6 +998,15 @@ using Gx1x1t = Tile3x3Cfg<2, 32, 1, 2, 4, 8, 16, 8, 1, 1>;    // ... two images 
 static bool small_plane_tile(const ConvDims &f) {
     return (long)ceil_div(f.N, Gx1x1s::NIMG) * ceil_div(f.Ci, Gx1x1s::TM * Gx1x1s::COW) <= 256;
 }
+// ... in workgroups of four waves that cover fewer rows, for maps whose height is not a multiple of 16 (56 = 7 x 8,
+// 28 = 7 x 4: ResNet-50 at batch 64, 64 -> 64 @56x56 366 -> 321 us, 128 -> 128 @28x28 345 -> 332 us)
+using GxW32H8 = Tile3x3Cfg<4, 8, 8, 1, 4, 4, 8, 1>;    // 8 rows of one image x 16 channels
+using GxW32H4 = Tile3x3Cfg<4, 8, 4, 2, 4, 4, 8, 1>;    // 4 rows of two images x 16 channels
+// rows per tile (16, 8 or 4) that pad a map of H rows least; the larger tile on a tie
+static int rows_per_tile_w32(int H) {
+    const int p16 = round_up(H, 16), p8 = round_up(H, 8), p4 = round_up(H, 4);
+    return p16 <= p8 && p16 <= p4 ? 16 : (p8 <= p4 ? 8 : 4);
+}
 static_assert(GxW32::TM == GxW16::TM && GxW16::TM == GxW8::TM && GxS2W32::TM == GxS2W16::TM,
               "the launcher checks Ci against one TM per stride");
 
@@ -1009,7 +1018,11 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
     if (k3s1p1 && d.Ci >= GxW32::TM &&
         (d.W % 4 != 0 || ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(gx) |
                            reinterpret_cast<uintptr_t>(gadd)) & 15) == 0)) {
-        if (d.W > 16) return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s, gadd);
+        if (d.W > 16) switch (rows_per_tile_w32(d.H)) {
+            case 16: return launch_grad_x_3x3s1<GxW32>(gy, x, w, gx, d, s, gadd);
+            case 8: return launch_grad_x_3x3s1<GxW32H8>(gy, x, w, gx, d, s, gadd);
+            default: return launch_grad_x_3x3s1<GxW32H4>(gy, x, w, gx, d, s, gadd);
+        }
         if (d.W > 8) return launch_grad_x_3x3s1<GxW16>(gy, x, w, gx, d, s, gadd);
         return launch_grad_x_3x3s1<GxW8>(gy, x, w, gx, d, s, gadd);
     }
@@ -1083,7 +1096,11 @@ static int bn_slots_of(const ConvDims &d) {
 // partial-sum slots per input channel that launch_grad_x_bn writes into bn.in_part; 0: no such kernel for the layer
 int grad_x_bn_slots(const ConvDims &d) {
     switch (grad_x_bn_variant(d)) {
-        case 1: return bn_slots_of<GxW32>(d);
+        case 1: switch (rows_per_tile_w32(d.H)) {
+            case 16: return bn_slots_of<GxW32>(d);
+            case 8: return bn_slots_of<GxW32H8>(d);
+            default: return bn_slots_of<GxW32H4>(d);
+        }
         case 2: return bn_slots_of<GxW16>(d);
         case 3: return bn_slots_of<GxW8>(d);
         case 4: return bn_slots_of<GxS2W32>(d);
@@ -1105,7 +1122,11 @@ int launch_grad_x_bn(const float *gy, const float *x, const float *w, float *gx,
     if (align & 15) return ADDER_ERR_UNSUPPORTED;
     if (!bn.in_part) return launch_grad_x(gy, x, w, gx, d, s, gadd);   // nothing to leave for a BatchNorm in front
     switch (grad_x_bn_variant(d)) {
-        case 1: return launch_grad_x_3x3s1_bn<GxW32>(gy, x, w, gx, d, s, gadd, bn);
+        case 1: switch (rows_per_tile_w32(d.H)) {
+            case 16: return launch_grad_x_3x3s1_bn<GxW32>(gy, x, w, gx, d, s, gadd, bn);
+            case 8: return launch_grad_x_3x3s1_bn<GxW32H8>(gy, x, w, gx, d, s, gadd, bn);
+            default: return launch_grad_x_3x3s1_bn<GxW32H4>(gy, x, w, gx, d, s, gadd, bn);
+        }
         case 2: return launch_grad_x_3x3s1_bn<GxW16>(gy, x, w, gx, d, s, gadd, bn);
         case 3: return launch_grad_x_3x3s1_bn<GxW8>(gy, x, w, gx, d, s, gadd, bn);
         case 4: return launch_grad_x_3x3s2_bn<GxS2W32>(gy, x, w, gx, d, s, gadd, bn);

@@ -127,12 +127,14 @@ class _conv_bn_act(torch.autograd.Function):
         dy = dy.contiguous()
         link, ctx.out_link = ctx.out_link, None
         gx = gw = dgamma = dbeta = None
-        if (not ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and link.claims(dy) and link.coef is not None
-                and all(t.data_ptr() % 16 == 0 for t in (x, conv_out, dy))):
+        # (link is None on a second pass through a retained graph: the separate BatchNorm backward below)
+        if (link is not None and not ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and link.claims(dy)
+                and link.coef is not None and all(t.data_ptr() % 16 == 0 for t in (x, conv_out, dy))):
             gw = _adder.conv2d_weight_grad(dy, x, w, stride, padding, out_link=link)   # None: not with this kernel
             if gw is not None:
                 dgamma, dbeta = link.dgamma, link.dbeta
-        link.dz = None
+        if link is not None:
+            link.dz = None
         if gw is None:
             gy, _, dgamma, dbeta = bn_backward(dy, y, mask, conv_out, gamma, mean, rstd, ctx.relu, False)
             if ctx.needs_input_grad[0]:
@@ -151,11 +153,7 @@ class StemConv2d(nn.Conv2d):
     adder layers."""
 
     def forward(self, x):
-        plain = (x.is_cuda and x.dtype == torch.float32 and self.bias is None and self.groups == 1
-                 and self.dilation == (1, 1) and self.padding_mode == "zeros" and torch.is_grad_enabled()
-                 and self.stride[0] == self.stride[1] and self.padding[0] == self.padding[1]
-                 and isinstance(self.padding[0], int))
-        if not plain:
+        if not self._plain(x):
             return super().forward(x)
         return _conv2d_matrix_grad.apply(x, self.weight, self.stride[0], self.padding[0])[0]
 
@@ -183,10 +181,7 @@ class StemConv2d(nn.Conv2d):
     def forward_with_stats(self, x):
         """(output, stats) like ``adder2d.forward_with_stats``: the BatchNorm partial sums of the output from the
         kernel's epilogue, or None."""
-        if not (x.is_cuda and x.dtype == torch.float32 and self.bias is None and self.groups == 1
-                and self.dilation == (1, 1) and self.padding_mode == "zeros" and torch.is_grad_enabled()
-                and self.stride[0] == self.stride[1] and isinstance(self.padding[0], int)
-                and self.padding[0] == self.padding[1]):
+        if not self._plain(x):
             return super().forward(x), None
         y, stats = _conv2d_matrix_grad.apply(x, self.weight, self.stride[0], self.padding[0])
         return y, (stats if stats.numel() else None)

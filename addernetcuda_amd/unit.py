@@ -31,6 +31,17 @@ from ._lib import require_gpu_f32, bwd_bn_slots, conv_dims
 from .bn_act import BatchNormAct2d, bn_forward, bn_backward
 
 
+def _engine_will_run(node):
+    """Whether the autograd engine runs (or captures the input of) ``node`` in the backward pass that is under way;
+    True when that cannot be told."""
+    if node is None:
+        return False
+    try:
+        return bool(torch._C._will_engine_execute_node(node))
+    except Exception:   # not inside a backward pass, or a torch without this query
+        return True
+
+
 class _adder_bn_act(Function):
     @staticmethod
     def forward(ctx, X, W, gamma, beta, residual, running_mean, running_var, num_batches, momentum, eps, relu, stride,
@@ -98,6 +109,10 @@ class _adder_bn_act(Function):
             out_link.dz = None   # (the tensor is kept alive by autograd for as long as it is needed)
         if not (usable and need_x and in_link is not None and X.data_ptr() == in_link.out_ptr):
             in_link = None
+        if pair is not None and not ctx.with_shortcut and need_x and not _engine_will_run(ctx.next_functions[0][0]):
+            # needs_input_grad is fixed when the graph is built; in this pass nothing upstream of this layer was asked
+            # for (torch.autograd.grad(loss, [this layer's weight])): no input gradient, and nothing to hand over
+            need_x = False
         if pair is not None and not ctx.with_shortcut and need_x and X.is_contiguous():
             # this is the 1x1 layer of the pair: its input gradient is left to the 3x3 layer's node, which runs next
             pair.side_gy, pair.side_w = gy.contiguous(), W

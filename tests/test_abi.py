@@ -188,3 +188,30 @@ def test_staged_grad_w_and_batched_scaling_validate_without_a_gpu():
     assert lib.adder_grad_w_finish_workspace_bytes(1, stages, ctypes.byref(need)) == 0 and need.value >= 16 * 144 // 64 * 8
     assert lib.adder_grad_w_finish_f32(33, stages, fake, 1 << 20, None) == -2
     assert lib.adder_grad_w_finish_f32(1, stages, fake, 16, None) == -4
+
+
+def test_bn_linked_backward_checks_every_link_field_for_aliasing_without_a_gpu():
+    """adder_conv2d_bwd_bn_f32: each read-only field of adder_bn_links (the BatchNorm's weight and bias, the side
+    layer's gradient and weights as well) against each output, before any HIP call."""
+    from addernetcuda_amd._lib import lib, BnLinks, ADDER_ERR_ALIAS
+    P = ctypes.c_void_p
+    dims = (4, 16, 16, 16, 32, 3, 3, 2, 1)     # a strided 3x3 layer: the side fields apply
+    slots = ctypes.c_int()
+    assert lib.adder_conv2d_bwd_bn_slots(*dims, ctypes.byref(slots)) == 0 and slots.value > 0
+    need = ctypes.c_size_t()
+    assert lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)) == 0
+    MB = 1 << 20
+    a = {n: (i + 1) * 16 * MB for i, n in enumerate(
+        ("gy", "x", "w", "gx", "gw", "ws", "in_x", "mean", "rstd", "part", "gamma", "beta", "side_gy", "side_w"))}
+
+    def call(**over):
+        v = dict(a, **over)
+        links = BnLinks(None, None, None, v["in_x"], v["mean"], v["rstd"], v["part"], slots.value, 1, v["gamma"], v["beta"],
+                        v["side_gy"], v["side_w"])
+        return lib.adder_conv2d_bwd_bn_f32(P(v["gy"]), P(v["x"]), P(v["w"]), None, P(v["gx"]), P(v["gw"]), 0.1, P(v["ws"]),
+                                           need.value, *dims, ctypes.byref(links), None)
+
+    # (never called with all-valid arguments: the addresses are made up, and on a machine with a GPU that would launch)
+    for field in ("gamma", "beta", "side_gy", "side_w", "mean", "rstd", "in_x"):
+        for out in ("gx", "gw", "part", "ws"):
+            assert call(**{field: a[out] + 64}) == ADDER_ERR_ALIAS, (field, out)

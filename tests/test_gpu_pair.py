@@ -246,3 +246,42 @@ def test_uncollected_side_gradient_is_an_error(gpu):
     ys = adder_bn_act(side, bns, shortcut)
     with pytest.raises(RuntimeError, match="paired 1x1 layer"):
         torch.autograd.grad(ys.sum(), shortcut)
+
+
+def test_gradient_of_the_paired_layers_own_parameters_only(gpu):
+    """torch.autograd.grad with respect to the downsample layer's weight (and its BatchNorm) alone never runs the
+    3x3 layer's node: the 1x1 node must then neither hand its input gradient over nor raise, and what it returns
+    must equal the same parameters' gradients from a full backward pass."""
+    from addernetcuda_amd import adder, resnet20
+    from addernetcuda_amd.bn_act import BatchNormAct2d
+    import torch.nn as nn
+    torch.manual_seed(6)
+    ds = nn.Sequential(adder.adder2d(16, 32, kernel_size=1, stride=2, padding=0, bias=False), BatchNormAct2d(32, relu=False))
+    block = resnet20.BasicBlock(16, 32, stride=2, downsample=ds).to(gpu).train()
+    x = torch.randn(4, 16, 16, 16, device=gpu, requires_grad=True)
+    gy = torch.randn(4, 32, 8, 8, device=gpu)
+    params = [ds[0].adder, ds[1].weight, ds[1].bias]
+    y = block(x)
+    only = torch.autograd.grad(y, params, gy, retain_graph=True)
+    y2 = block(x)
+    y2.backward(gy)
+    for got, p in zip(only, params):
+        assert_close(got, p.grad, "gradient of the downsample branch's parameters", rtol=1e-4, atol=1e-4)
+
+
+def test_second_backward_through_a_retained_graph_of_the_whole_network(gpu):
+    """The stem's convolution + BatchNorm node (resnet20._conv_bn_act) hands over like the adder units do; a second
+    pass through a retained graph finds the hand-over used up and must take the plain path with the same result."""
+    from addernetcuda_amd.resnet20 import resnet20
+    torch.manual_seed(8)
+    model = resnet20(eta=0.1).to(gpu).train()
+    x = torch.randn(8, 3, 32, 32, device=gpu)
+    t = torch.randint(0, 10, (8,), device=gpu)
+    loss = torch.nn.functional.cross_entropy(model(x), t)
+    loss.backward(retain_graph=True)
+    first = {n: p.grad.clone() for n, p in model.named_parameters()}
+    model.zero_grad(set_to_none=True)
+    loss.backward()
+    for n, p in model.named_parameters():
+        scale = first[n].abs().max().item() + 1e-6
+        assert (p.grad - first[n]).abs().max().item() <= 1e-3 * scale, n
