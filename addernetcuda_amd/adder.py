@@ -71,8 +71,9 @@ class batched_eta_scaling:
     It only takes over layers whose weight is a leaf with ``grad is None`` when their backward runs (the usual
     ``zero_grad(set_to_none=True)`` loop); all others are finished on the spot as always.  One backward pass
     per block.  If the block is left by an exception, the gradients of the layers it had taken over are set to
-    None (they were never finished).  Not for code that looks at weight gradients from hooks during the backward pass, nor for
-    ``torch.autograd.grad``."""
+    None (they were never finished).  A weight with a gradient hook registered on it (``register_hook``,
+    ``register_post_accumulate_grad_hook``) is not taken over either, so the hook sees the finished gradient.  Not
+    for ``torch.autograd.grad``."""
 
     def __enter__(self):
         global _eta_batch
@@ -133,6 +134,12 @@ class batched_eta_scaling:
                     check(lib.adder_grad_norm_scale_batched_f32(count, ptrs, sizes, etas, 1e-12, ptr(ws), need.value,
                                                                 stream_ptr(dev)), "adder_grad_norm_scale_batched_f32")
         return False
+
+
+def _has_grad_hooks(W):
+    """A weight somebody watches during the backward pass (``register_hook``, ``register_post_accumulate_grad_hook``):
+    such a hook must see the finished gradient, so ``batched_eta_scaling`` leaves the layer to finish on the spot."""
+    return bool(getattr(W, "_backward_hooks", None)) or bool(getattr(W, "_post_accumulate_grad_hooks", None))
 
 
 def conv_forward(X, W, stride, padding, with_stats):
@@ -316,7 +323,7 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
         raise RuntimeError("batched_eta_scaling: this weight already has a pending gradient in the block "
                            "(one backward pass per block, no weight shared between layers)")
     staged = False
-    if (_eta_batch is not None and need_w and w_is_given and W.is_leaf and W.grad is None):
+    if (_eta_batch is not None and need_w and w_is_given and W.is_leaf and W.grad is None and not _has_grad_hooks(W)):
         with on_device(dev):
             ws, nbytes = conv2d_bwd_workspace(dims, dev)
             stage = GradWStage()
@@ -507,7 +514,7 @@ def conv2d_weight_grad(grad_out, X, W, stride, padding, out_link=None):
         if status == ADDER_ERR_UNSUPPORTED:
             return None
         check(status, "adder_conv2d_grad_w_staged_f32")
-        if (_eta_batch is not None and W.is_leaf and W.grad is None and W.is_contiguous()
+        if (_eta_batch is not None and W.is_leaf and W.grad is None and W.is_contiguous() and not _has_grad_hooks(W)
                 and not any(W is entry[0] for entry in _eta_batch)):
             _eta_batch.append((W, 0.0, stage, ws))
             return gw

@@ -300,6 +300,15 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
             for (int cc = 0; cc < ccnt; cc += 2) {
                 one_channel(cc, 0);
                 if (cc + 1 < ccnt) one_channel(cc + 1, 1);
+                // the two-instruction form folds its first-level sums every eight output channels (72 terms): with
+                // 144-term first levels its worst element sat at 0.71 of the parity tolerance for 1152 terms per
+                // output, with 72-term ones at 0.51
+                if (SAT && KS == 3 && ((cc + 2) & 7) == 0 && cc + 2 < ccnt) {
+#pragma unroll
+                    for (int m = 0; m < TM; ++m)
+#pragma unroll
+                        for (int t = 0; t < TN; ++t) { tot[m][t] += acc[m][t]; acc[m][t] = 0.f; }
+                }
             }
 
         }
@@ -516,12 +525,14 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
 }
 
 // The two-instruction form doubles a sum of products whose factors lie in [0, 1] and takes a second
-// sum off it, which about triples the rounding error of the three-instruction form (measured against
-// fp64: 0.2 of the parity tolerance |err| <= 1e-4 + 1e-5 |gx| at 144 terms per output, 0.4 at 576, 0.9
-// at 4608).  Layers with more terms per output than this keep the three-instruction form.  Single-tap
-// layers stop at 1024: their chunks are CC terms long, not 9 * CC, so the second level of the sum is long
-// and carries the full magnitude (512 -> 2048 @7x7 at batch 64 had one element in 1e5 at 1.2 of the tolerance).
-static constexpr int kSatMaxTerms = 2304, kSatMaxTerms1x1 = 1024;
+// sum off it, which about doubles the rounding error of the three-instruction form.  Measured against fp64
+// as the worst element's share of the parity tolerance |err| <= 1e-4 + 1e-5 |gx| over 8 seeds x {Kaiming,
+// N(0,1)} weights x input scale {1, 5}, first-level sums of at most 72 terms: 0.26 at 576 terms per output,
+// 0.51 at 1152, 0.62 at 2304 (256 output channels x 9 taps; 0.96 with 144-term first levels: too close), where
+// the three-instruction form sits at 0.45, and at 0.54 for 4608.  Layers with more than 1152 terms per output
+// therefore keep the three-instruction form.  Single-tap layers stop at 1024: their chunks are CC terms long, not 9 * CC, so the second level of the
+// sum is long and carries the full magnitude (0.46 at 1024 with the first level folded every fourth chunk).
+static constexpr int kSatMaxTerms = 1152, kSatMaxTerms1x1 = 1024;
 
 static const adder_bn_links kNoLinks{};
 

@@ -259,3 +259,35 @@ def test_batched_eta_scaling_leaves_the_same_gradients(gpu):
     with adder.batched_eta_scaling():
         layer(xin).sum().backward()
     assert torch.allclose(layer.adder.grad, 2 * first, rtol=1e-6, atol=0.0)
+
+
+# (N, Ci, H, W, Co, kh, kw, stride, pad): kernels that are not square.  The reference's operator assumes square
+# ones (adder.py:32 hands unfold the kernel's height only) and so does this build's Python layer; the C ABI takes
+# kh and kw separately, serves such layers with the generic kernels, and is held to the same oracle.
+NON_SQUARE = [(2, 5, 9, 11, 6, 3, 1, 1, 1), (2, 4, 8, 12, 7, 1, 3, 1, 1), (1, 3, 10, 9, 4, 3, 5, 2, 2),
+              (2, 6, 7, 7, 5, 1, 2, 1, 0), (1, 8, 12, 12, 8, 3, 1, 2, 1)]
+
+
+@pytest.mark.parametrize("case", NON_SQUARE, ids=str)
+def test_non_square_kernels_through_the_c_abi(case, gpu):
+    from addernetcuda_amd._lib import lib, ptr, stream_ptr, check
+    from oracle import c_oracle
+    N, Ci, H, W, Co, kh, kw, s, p = case
+    g = torch.Generator().manual_seed(77 + kh * 10 + kw)
+    x = torch.randn(N, Ci, H, W, generator=g)
+    w = torch.randn(Co, Ci, kh, kw, generator=g) * 0.5
+    Ho, Wo = (H - kh + 2 * p) // s + 1, (W - kw + 2 * p) // s + 1
+    gy = torch.randn(N, Co, Ho, Wo, generator=g)
+    dims = (N, Ci, H, W, Co, kh, kw, s, p)
+    xg, wg, gyg = x.to(gpu), w.to(gpu), gy.to(gpu)
+    y, gx, gw = torch.empty(N, Co, Ho, Wo, device=gpu), torch.empty_like(xg), torch.empty_like(wg)
+    need = ctypes.c_size_t()
+    check(lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)), "workspace")
+    ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=gpu)
+    st = stream_ptr(gpu)
+    check(lib.adder_conv2d_fwd_f32(ptr(xg), ptr(wg), ptr(y), *dims, st), "fwd")
+    check(lib.adder_conv2d_bwd_f32(ptr(gyg), ptr(xg), ptr(wg), ptr(gx), ptr(gw), 0.0, ptr(ws), need.value, *dims, st), "bwd")
+    torch.cuda.synchronize()
+    assert_close(y, c_oracle.conv2d_fwd(x, w, s, p), f"forward {case}")
+    assert_close(gx, c_oracle.conv2d_grad_x(gy, x, w, s, p), f"grad_X {case}")
+    assert_close(gw, c_oracle.conv2d_grad_w(gy, x, w, s, p), f"raw grad_W {case}")

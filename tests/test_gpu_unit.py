@@ -211,3 +211,72 @@ def test_resnet20_runs_three_batchnorm_backwards_of_its_own(gpu, monkeypatch):
     torch.cuda.synchronize()
     assert len(calls) == 3
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in net.parameters())
+
+
+def _unit_chain_grads(net, x, gout, forward=None):
+    xi = x.clone().requires_grad_(True)
+    out = (forward or _forward_units)(net, xi)
+    out.backward(gout)
+    return xi.grad, {n: p.grad.clone() for n, p in net.named_parameters()}
+
+
+def test_units_under_activation_checkpointing(gpu):
+    """torch.utils.checkpoint re-runs the forward inside the backward pass (new nodes, new links, new tensors):
+    the chain of units must give the gradients it gives without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+    hip, _ = _nets(gpu, 16, 2, 23)
+    twin = copy.deepcopy(hip)
+    x = torch.relu(torch.randn(4, 16, 32, 32, device=gpu))
+    gout = torch.randn(4, 32, 16, 16, device=gpu)
+    gx0, gp0 = _unit_chain_grads(twin, x, gout)
+    xi = x.clone().requires_grad_(True)
+    out = checkpoint(lambda t: _forward_units(hip, t), xi, use_reentrant=False)
+    out.backward(gout)
+    assert_close(xi.grad, gx0, "input gradient under checkpointing", rtol=1e-5, atol=1e-5)
+    for n, p in hip.named_parameters():
+        scale = max(1.0, float(gp0[n].abs().max()))
+        assert_close(p.grad / scale, gp0[n] / scale, n + " under checkpointing", rtol=1e-5, atol=1e-5)
+
+
+def test_autograd_grad_with_respect_to_the_chain_input(gpu):
+    """torch.autograd.grad(out, x): only the input gradient is asked for, no weight gradient -- the hand-over needs
+    the weight-gradient kernel (it is the one that forms a layer's output gradient), so every unit must take the
+    plain path and still deliver the same input gradient as a full backward pass."""
+    hip, _ = _nets(gpu, 16, 2, 29)
+    x = torch.relu(torch.randn(4, 16, 32, 32, device=gpu))
+    gout = torch.randn(4, 32, 16, 16, device=gpu)
+    gx0, _ = _unit_chain_grads(copy.deepcopy(hip), x, gout)
+    xi = x.clone().requires_grad_(True)
+    (gx,) = torch.autograd.grad(_forward_units(hip, xi), xi, gout)
+    assert_close(gx, gx0, "input gradient from autograd.grad", rtol=1e-4, atol=1e-4)
+    assert all(p.grad is None for p in hip.parameters())
+    # ... and with respect to one weight in the middle of the chain only
+    xi = x.clone().requires_grad_(True)
+    (gw,) = torch.autograd.grad(_forward_units(hip, xi), hip.b.adder, gout)
+    _, gp0 = _unit_chain_grads(copy.deepcopy(hip), x, gout)
+    scale = max(1.0, float(gp0["b.adder"].abs().max()))
+    assert_close(gw / scale, gp0["b.adder"] / scale, "one weight's gradient from autograd.grad", rtol=1e-4, atol=1e-4)
+
+
+def test_weight_hook_inside_batched_eta_scaling_sees_the_finished_gradient(gpu):
+    """A register_hook on an adder weight runs during the backward pass; inside batched_eta_scaling() that layer is
+    therefore not taken over (its gradient would be unfinished slabs at that moment) while the others still are."""
+    from addernetcuda_amd import adder as adder_mod
+    from addernetcuda_amd.adder import batched_eta_scaling
+    hip, _ = _nets(gpu, 16, 1, 31)
+    x = torch.relu(torch.randn(4, 16, 16, 16, device=gpu))
+    gout = torch.randn(4, 32, 16, 16, device=gpu)
+    _, gp0 = _unit_chain_grads(copy.deepcopy(hip), x, gout)
+    seen = {}
+    handle = hip.b.adder.register_hook(lambda g: seen.__setitem__("b", g.clone()))
+    xi = x.clone().requires_grad_(True)
+    out = _forward_units(hip, xi)
+    with batched_eta_scaling():
+        out.backward(gout)
+        pending = [id(entry[0]) for entry in adder_mod._eta_batch]
+    handle.remove()
+    assert id(hip.b.adder) not in pending and id(hip.a.adder) in pending
+    assert_close(seen["b"], gp0["b.adder"], "gradient seen by the hook", rtol=1e-5, atol=1e-6)
+    for n, p in hip.named_parameters():
+        scale = max(1.0, float(gp0[n].abs().max()))
+        assert_close(p.grad / scale, gp0[n] / scale, n, rtol=1e-5, atol=1e-6)
