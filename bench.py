@@ -69,7 +69,8 @@ LAYER_SETS = {"resnet20": (BATCH, RESNET20_LAYERS), "vgg_small": (128, VGG_SMALL
 OPS = {"fwd": (2, 2), "grad_x": (4, 2), "grad_w": (3, 1)}
 
 
-WARM_SECONDS = 0.04
+# seconds of the same call before every timing; ADDER_BENCH_WARM_S=0 for profiler runs that should hold few dispatches
+WARM_SECONDS = float(os.environ.get("ADDER_BENCH_WARM_S", "0.04"))
 
 
 def event_time(fn, warmup, iters):
@@ -112,8 +113,12 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
     st = stream_ptr(dev)
     E = Co * Ci * k * k * N * Ho * Wo
     nx, ny, nw = 4 * x.numel(), 4 * y.numel(), 4 * w.numel()
-    # algorithmic HBM bytes of each call: every tensor it reads or writes crosses HBM once
-    nbytes = {"fwd": nx + nw + ny, "grad_x": 2 * nx + ny + nw, "grad_w": nx + ny + 2 * nw}
+    # algorithmic HBM bytes of each call: every tensor it reads or writes crosses HBM once.  A 1x1 layer with a
+    # stride reads x at every stride-th row and column only: the rows it skips never leave HBM, the columns it skips
+    # share their 128-byte lines with the ones it reads, so x counts with 1 / stride of its bytes where it is read
+    # (grad_X still writes all of gx, the zeros included).
+    rx = nx // stride if k == 1 else nx
+    nbytes = {"fwd": rx + nw + ny, "grad_x": rx + nx + ny + nw, "grad_w": rx + ny + 2 * nw}
     keep = [x, w, y, gy, gx, gw, ws]
     ops = {
         "fwd": lambda: check(lib.adder_conv2d_fwd_f32(ptr(x), ptr(w), ptr(y), *dims, st), "fwd"),
@@ -163,7 +168,7 @@ def bench_layers(dev, warmup=5, iters=20, which="resnet20"):
                 "layer": f"{Ci}->{Co} k{k} s{s} p{p} @{H}x{W}", "count": cnt, "op": name, "us": round(t * 1e6, 2),
                 "tflops": round(flop * E / t / 1e12, 2),
                 "frac_fp32_peak": round(flop * E / t / 1e12 / PEAK_FP32_TFLOPS, 4),
-                "hbm_gbs": round(nbytes[name] / t / 1e9, 1),
+                "algorithmic_bytes": nbytes[name], "hbm_gbs": round(nbytes[name] / t / 1e9, 1),
                 "frac_hbm_peak": round(nbytes[name] / t / 1e9 / PEAK_HBM_GBS, 4),
             }
             if name in ("grad_w", "grad_w_bn") and k == 3:   # fp64 matrix-core kernel (+ finalize and scaling launches)
@@ -242,6 +247,50 @@ def dominant_kernel(dev, steps):
                 "sums per channel; xhat comes from the x the lanes hold) is the first pass of a BatchNorm backward that no longer "
                 "runs as a kernel of its own.",
     }
+
+
+def parity_gate(dev, images=4):
+    """Before anything is timed: forward, grad_X, raw and eta-scaled grad_W of the three config-2 layer shapes (a few
+    images each) through the C ABI against the float64 C oracle, at the bar rtol 1e-5 / atol 1e-4.  Reported per
+    output as the worst element's share of that tolerance, next to the same figure for the float32 pure-PyTorch
+    oracle (the reference's formulas) against the same float64 truth.  Raises if the HIP path misses the bar."""
+    from addernetcuda_amd._lib import lib, ptr, stream_ptr, conv_dims, check
+    from oracle import c_oracle, adder_oracle
+    rows = []
+    for cnt, Ci, H, W, Co, k, s, p in RESNET20_LAYERS:
+        if not (k == 3 and s == 1):
+            continue
+        g = torch.Generator().manual_seed(2000 + Ci)
+        x = torch.randn(images, Ci, H, W, generator=g)
+        w = torch.randn(Co, Ci, k, k, generator=g) * math.sqrt(2.0 / (Ci * k * k))
+        gy = torch.randn(images, Co, H, W, generator=g)
+        dims, Ho, Wo = conv_dims(x.shape, w.shape, s, p)
+        xg, wg, gyg = x.to(dev), w.to(dev), gy.to(dev)
+        y, gx, gw, gws = torch.empty_like(gyg), torch.empty_like(xg), torch.empty_like(wg), torch.empty_like(wg)
+        need = ctypes.c_size_t()
+        check(lib.adder_conv2d_bwd_workspace_bytes(*dims, ctypes.byref(need)), "workspace")
+        ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=dev)
+        st = stream_ptr(dev)
+        check(lib.adder_conv2d_fwd_f32(ptr(xg), ptr(wg), ptr(y), *dims, st), "fwd")
+        check(lib.adder_conv2d_bwd_f32(ptr(gyg), ptr(xg), ptr(wg), ptr(gx), ptr(gw), 0.0, ptr(ws), need.value, *dims, st), "bwd")
+        check(lib.adder_conv2d_bwd_f32(ptr(gyg), ptr(xg), ptr(wg), None, ptr(gws), ETA, ptr(ws), need.value, *dims, st), "bwd")
+        torch.cuda.synchronize()
+        truth = {"fwd": c_oracle.conv2d_fwd(x, w, s, p), "grad_x": c_oracle.conv2d_grad_x(gy, x, w, s, p),
+                 "grad_w": c_oracle.conv2d_grad_w(gy, x, w, s, p)}
+        truth["grad_w_eta_scaled"] = c_oracle.eta_scale(truth["grad_w"], ETA)
+        o_gx, o_gw, o_gws = adder_oracle.conv2d_backward(gy, x, w, s, p, eta=ETA)
+        torch32 = {"fwd": adder_oracle.conv2d_forward(x, w, s, p), "grad_x": o_gx, "grad_w": o_gw, "grad_w_eta_scaled": o_gws}
+        hip = {"fwd": y, "grad_x": gx, "grad_w": gw, "grad_w_eta_scaled": gws}
+        share = lambda got, want: float(((got.double().cpu() - want).abs() / (1e-4 + 1e-5 * want.abs())).max())
+        row = {"layer": f"{Ci}->{Co} k{k} s{s} p{p} @{H}x{W}", "images": images}
+        for name, want in truth.items():
+            row[name] = {"hip_share_of_tolerance": round(share(hip[name], want), 4),
+                         "torch_f32_oracle_share_of_tolerance": round(share(torch32[name], want), 4)}
+            if not row[name]["hip_share_of_tolerance"] <= 1.0:
+                raise SystemExit(f"bench.py: parity gate failed before timing: {row['layer']} {name} at "
+                                 f"{row[name]['hip_share_of_tolerance']} of rtol 1e-5 / atol 1e-4")
+        rows.append(row)
+    return rows
 
 
 def make_step(model, opt, x, y):
@@ -388,6 +437,60 @@ def other_configs(dev):
     return out
 
 
+def cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_layer_baseline(repeats=3):   # ~25 s of host work
+    """BASELINE config 2 on the host: the three 3x3 / stride 1 / pad 1 layer shapes (16, 32, 64 channels at 32, 16, 8
+    pixels, batch 256) through the chunked torch oracle -- unfold (adder.py:32-33), forward (test_cuda.py:18-22),
+    grad_W (test_cuda.py:35-41), grad_X (test_cuda.py:57-60), and grad_W with the scaling of adder.py:78 -- each
+    the median of `repeats` runs."""
+    from oracle import adder_oracle as o
+    rows = []
+    for cnt, Ci, H, W, Co, k, s, p in RESNET20_LAYERS:
+        if not (k == 3 and s == 1):
+            continue
+        g = torch.Generator().manual_seed(1000 + Ci + Co + k + s)
+        x = torch.randn(BATCH, Ci, H, W, generator=g)
+        w = torch.randn(Co, Ci, k, k, generator=g) * math.sqrt(2.0 / (Ci * k * k))
+        gy = torch.randn(BATCH, Co, H, W, generator=g)
+        E = Co * Ci * k * k * BATCH * H * W
+        W_col = w.reshape(Co, -1)
+        state = {}
+
+        def unfold():
+            state["X"], _, _ = o.im2col(x, k, s, p)
+            state["g"] = o.nchw_to_out_col(gy)
+        unfold()
+        ops = {
+            "unfold": (unfold, 0),
+            "fwd": (lambda: o.col_forward(state["X"], W_col), 2),
+            "grad_w": (lambda: state.__setitem__("gw", o.col_grad_w(state["X"], W_col, state["g"])), 3),
+            "grad_x": (lambda: o.col_grad_x(state["X"], W_col, state["g"]), 4),
+            "grad_w_eta_scaled": (lambda: o.eta_scale(o.col_grad_w(state["X"], W_col, state["g"]), ETA), 3),
+        }
+        for name, (fn, flop) in ops.items():
+            times = []
+            for _ in range(repeats):
+                t0 = time.perf_counter()
+                fn()
+                times.append(time.perf_counter() - t0)
+            med = statistics.median(times)
+            row = {"layer": f"{Ci}->{Co} k{k} s{s} p{p} @{H}x{W}", "batch": BATCH, "op": name, "ms": round(med * 1e3, 1)}
+            if flop:
+                row["gflops"] = round(flop * E / med / 1e9, 1)
+            rows.append(row)
+    return rows
+
+
 def cpu_baseline(repeats=15):   # ~10 s of host work
     """The CPU oracle's ResNet-20 training step at batch 8 (seeded), median of `repeats`, scaled to batch 256."""
     from addernetcuda_amd.resnet20 import resnet20
@@ -411,7 +514,11 @@ def cpu_baseline(repeats=15):   # ~10 s of host work
         "kind": "port",
         "sample": f"ResNet-20 AdderNet fwd+bwd+SGD at batch {bs} through the pure-PyTorch unfold oracle, median of "
                   f"{repeats} steps = {med * 1e3:.0f} ms, scaled x{BATCH // bs} to batch 256",
-        "host_cpus": os.cpu_count(),
+        "host_cpus": os.cpu_count(), "cpu_model": cpu_model_name(),
+        "layers": cpu_layer_baseline(),
+        "layers_note": "BASELINE config 2 on the host cores: the three stride-1 3x3 shapes at batch 256 through the "
+                       "chunked pure-PyTorch oracle (the formulas of adder_cuda/test_cuda.py:18-22,35-41,57-60 and "
+                       "adder.py:78 on the unfolded (K, L*N) matrix), median of 3 runs each, all intra-op threads",
     }
 
 
@@ -469,6 +576,7 @@ def main():
                           **layer_set_summary(rows)}))
         return
 
+    gate = None if args.no_cpu else parity_gate(dev)   # (needs the oracle, like the CPU leg)
     fused = not args.stock_modules
     ms, mode, graph_check = time_training(dev, args.model, fused, args.steps, args.warmup, use_graph=not args.no_graph,
                                           replays=4 if args.model == "resnet20" else 2)
@@ -503,6 +611,9 @@ def main():
     }
     if graph_check is not None:
         out["graph_check"] = graph_check
+    if gate is not None:
+        out["parity_gate"] = {"bar": "rtol 1e-5 / atol 1e-4 against the float64 C oracle, worst element as a share of it",
+                              "layers": gate}
     if not args.no_layers:
         rows = bench_layers(dev)
         out["layers"] = rows
