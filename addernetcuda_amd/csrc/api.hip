@@ -355,6 +355,8 @@ int adder_col_bwd_f32(const float *gy, const float *Xcol, const float *Wcol, flo
     if (int rc = col_alias(gy, Xcol, Wcol, gW, gX, K, NL, Co)) return rc;
     if (int rc = check_col_ws(ws, ws_bytes, K, NL, Co)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int small = launch_col_bwd_small(gy, Xcol, Wcol, gW, gX, K, NL, Co, s);   // few columns: one launch
+    if (small != ADDER_ERR_UNSUPPORTED) return small;
     const int fused = launch_col_bwd_fused(gy, Xcol, Wcol, gW, gX, K, NL, Co, ws, s);   // one pass over Xcol where it applies
     if (fused != ADDER_ERR_UNSUPPORTED) return fused;
     if (int rc = launch_col_grad_x(gy, Xcol, Wcol, gX, K, NL, Co, s)) return rc;

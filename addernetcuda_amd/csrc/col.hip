@@ -605,6 +605,140 @@ __global__ __launch_bounds__(256) void col_grad_w_kernel(const float *__restrict
     }
 }
 
+// ---------------------------------------------------------------------------
+// Both gradients of a matrix with few columns in ONE launch and without a workspace (the reference's own
+// comparison shape, adder_cuda/test_cuda.py:161-176: Co = 32, K = 288, NL = 1024).  With so few columns the slab
+// kernels above are a chain of launches that each last as long as a launch takes; here a workgroup owns KB rows of
+// X over ALL columns, so the weight gradient of its rows needs no partner: thread t holds columns t, t + 256, ... of
+// its rows in registers, walks the output channels once (gy straight from memory, coalesced; the weight as a scalar),
+// finishes its elements of gX on the spot and leaves, per output channel, its share of sum_c X[k,c] gy[co,c] and of
+// sum_c gy[co,c] to a wave reduction.  The per-thread shares are at most CPT terms long and the sums over the
+// columns at most 2048: fp32 throughout (the slab kernels use fp64 because they sum 262 144).
+//   gX[k,c] += sum_co hardtanh(W[co,k] - X[k,c]) gy[co,c]        (test_cuda.py:57-60; adder.cu:17,246)
+//   gW[co,k] += sum_c X[k,c] gy[co,c] - W[co,k] sum_c gy[co,c]   (test_cuda.py:35-41; adder.cu:247)
+// gW or gX may be null (ADDER_CONV_INPUT / ADDER_CONV_WEIGHT).
+// ---------------------------------------------------------------------------
+template <int KB, int CPT, int GB>
+__global__ __launch_bounds__(256) void col_bwd_small_kernel(const float *__restrict__ gy, const float *__restrict__ X,
+                                                            const float *__restrict__ Wm, float *__restrict__ gW,
+                                                            float *__restrict__ gX, int K, int NL, int Co) {
+    extern __shared__ __align__(16) float smem[];
+    float *wl = smem;                      // [Co][KB] weights of this workgroup's rows
+    float *red = smem + Co * KB;           // [4 waves][Co][KB + 1] wave sums
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int k0 = blockIdx.x * KB;
+    for (int e = threadIdx.x; e < Co * KB; e += 256) {
+        const int co = e / KB, kk = e - co * KB;
+        wl[e] = Wm[(size_t)co * K + min(k0 + kk, K - 1)];
+    }
+    float x[KB][CPT], acc[KB][CPT];
+#pragma unroll
+    for (int kk = 0; kk < KB; ++kk)
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            const int c = threadIdx.x + j * 256;
+            x[kk][j] = (k0 + kk < K && c < NL) ? X[(size_t)(k0 + kk) * NL + c] : 0.f;
+            acc[kk][j] = 0.f;
+        }
+    // gy of the own columns, GB output channels at a time with the next GB in flight: a channel's arithmetic is a
+    // few dozen instructions, far shorter than a trip to memory
+    float g[2][GB][CPT];
+    auto fetch = [&](int co0, float (&dst)[GB][CPT]) {
+#pragma unroll
+        for (int u = 0; u < GB; ++u)
+#pragma unroll
+            for (int j = 0; j < CPT; ++j) {
+                const int c = threadIdx.x + j * 256;
+                dst[u][j] = (co0 + u < Co && c < NL) ? gy[(size_t)(co0 + u) * NL + c] : 0.f;
+            }
+    };
+    fetch(0, g[0]);
+    __syncthreads();
+    auto batch = [&](int co0, const float (&gb)[GB][CPT]) {
+        // (channels past Co were fetched as zeros: their terms vanish and their sums are not stored)
+        float sxg[GB * KB], sg[GB];
+#pragma unroll
+        for (int u = 0; u < GB; ++u) {
+            const int co = min(co0 + u, Co - 1);
+            sg[u] = 0.f;
+#pragma unroll
+            for (int j = 0; j < CPT; ++j) sg[u] += gb[u][j];
+#pragma unroll
+            for (int kk = 0; kk < KB; ++kk) {
+                const float w = wl[co * KB + kk];
+                float pw = 0.f;
+#pragma unroll
+                for (int j = 0; j < CPT; ++j) {
+                    acc[kk][j] = fmaf(hardtanh(w - x[kk][j]), gb[u][j], acc[kk][j]);
+                    pw = fmaf(x[kk][j], gb[u][j], pw);
+                }
+                sxg[u * KB + kk] = pw;
+            }
+        }
+        if (gW) {
+            // all sums of the batch at once: a reduce-scatter over the lanes, lane l ends with sum number index(l)
+            const float a = wave_sum_scatter<GB * KB>(sxg, lane);
+            const float c = wave_sum_scatter<GB>(sg, lane);
+            if (lane < GB * KB) {
+                const int e = wave_sum_scatter_index<GB * KB>(lane), u = e / KB, kk = e - u * KB;
+                if (co0 + u < Co) red[(wave * Co + co0 + u) * (KB + 1) + kk] = a;
+            }
+            if (lane < GB) {
+                const int u = wave_sum_scatter_index<GB>(lane);
+                if (co0 + u < Co) red[(wave * Co + co0 + u) * (KB + 1) + KB] = c;
+            }
+        }
+    };
+    for (int co0 = 0; co0 < Co; co0 += 2 * GB) {
+        if (co0 + GB < Co) fetch(co0 + GB, g[1]);
+        batch(co0, g[0]);
+        if (co0 + 2 * GB < Co) fetch(co0 + 2 * GB, g[0]);
+        if (co0 + GB < Co) batch(co0 + GB, g[1]);
+    }
+    if (gX) {
+#pragma unroll
+        for (int kk = 0; kk < KB; ++kk)
+#pragma unroll
+            for (int j = 0; j < CPT; ++j) {
+                const int c = threadIdx.x + j * 256;
+                if (k0 + kk < K && c < NL) gX[(size_t)(k0 + kk) * NL + c] += acc[kk][j];
+            }
+    }
+    if (gW) {
+        __syncthreads();
+        const int stride = Co * (KB + 1);
+        for (int e = threadIdx.x; e < Co * KB; e += 256) {
+            const int co = e / KB, kk = e - co * KB;
+            if (k0 + kk >= K) continue;
+            const float *r = red + co * (KB + 1);
+            const float sxg = (r[kk] + r[stride + kk]) + (r[2 * stride + kk] + r[3 * stride + kk]);
+            const float sg = (r[KB] + r[stride + KB]) + (r[2 * stride + KB] + r[3 * stride + KB]);
+            gW[(size_t)co * K + k0 + kk] += sxg - wl[e] * sg;
+        }
+    }
+}
+
+// matrices the one-launch kernel above serves: few columns, a wave-sum table that fits the LDS
+static bool col_bwd_small_applies(int K, long NL, int Co) { return NL <= 2048 && Co <= 512; }
+
+// gW / gX: either may be null
+int launch_col_bwd_small(const float *gy, const float *X, const float *Wm, float *gW, float *gX, int K, long NL, int Co,
+                         hipStream_t s) {
+    if (!col_bwd_small_applies(K, NL, Co)) return ADDER_ERR_UNSUPPORTED;
+    const int cpt = (int)ceil_div_l(NL, 256);
+#define ADDER_COL_SMALL(KB, CPT, GB)                                                                                 \
+    hipLaunchKernelGGL((col_bwd_small_kernel<KB, CPT, GB>), dim3(ceil_div(K, KB)), dim3(256),                            \
+                       (Co * KB + 4 * Co * (KB + 1)) * 4, s, gy, X, Wm, gW, gX, K, (int)NL, Co)
+    // one row of X per workgroup while that fills the chip, two on taller matrices
+    const bool tall = K >= 1024;
+    if (cpt <= 1) { if (tall) ADDER_COL_SMALL(2, 1, 8); else ADDER_COL_SMALL(1, 1, 8); }
+    else if (cpt <= 2) { if (tall) ADDER_COL_SMALL(2, 2, 8); else ADDER_COL_SMALL(1, 2, 8); }
+    else if (cpt <= 4) { if (tall) ADDER_COL_SMALL(2, 4, 8); else ADDER_COL_SMALL(1, 4, 8); }
+    else { if (tall) ADDER_COL_SMALL(2, 8, 4); else ADDER_COL_SMALL(1, 8, 4); }
+#undef ADDER_COL_SMALL
+    return check_launch();
+}
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 static bool aligned8(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0; }
 
@@ -655,6 +789,7 @@ static bool col_bwd_fused_applies(int K, long NL, int Co) { return Co <= 16 && N
 static int col_bwd_fused_slots(long NL) { return (int)ceil_div_l(NL, 512); }
 
 size_t col_grad_w_workspace_bytes(int K, long NL, int Co) {
+    if (col_bwd_small_applies(K, NL, Co)) return 0;   // one launch, no slabs
     const ColGwPlan p = plan_col_grad_w(K, NL, Co);
     int slots = p.mfma ? p.slots : 0;
     if (col_bwd_fused_applies(K, NL, Co) && col_bwd_fused_slots(NL) > slots) slots = col_bwd_fused_slots(NL);
@@ -691,6 +826,7 @@ static void launch_col_gw(const float *gy, const float *X, double *part, double 
 
 int launch_col_grad_w(const float *gy, const float *X, const float *Wm, float *gW, int K, long NL, int Co,
                       void *ws, hipStream_t s) {
+    if (col_bwd_small_applies(K, NL, Co)) return launch_col_bwd_small(gy, X, Wm, gW, nullptr, K, NL, Co, s);
     const ColGwPlan p = plan_col_grad_w(K, NL, Co);
     if (p.mfma && ws && aligned16(X) && aligned16(gy) && (reinterpret_cast<uintptr_t>(ws) & 255) == 0) {
         double *part = reinterpret_cast<double *>(ws);
@@ -715,6 +851,7 @@ int launch_col_grad_w(const float *gy, const float *X, const float *Wm, float *g
 
 int launch_col_grad_x(const float *gy, const float *X, const float *Wm, float *gX, int K, long NL, int Co,
                       hipStream_t s) {
+    if (col_bwd_small_applies(K, NL, Co)) return launch_col_bwd_small(gy, X, Wm, nullptr, gX, K, NL, Co, s);
     if (Co <= 32) {
         // gy in registers, X streamed once; rows in blocks of KB whose weights fit a 32 KB LDS tile
         const int COB = Co <= 16 ? 16 : 32;

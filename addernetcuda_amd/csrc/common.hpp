@@ -309,6 +309,8 @@ int launch_col_grad_w(const float *gy, const float *X, const float *W, float *gW
                       int Co, void *ws, hipStream_t s);
 int launch_col_grad_x(const float *gy, const float *X, const float *W, float *gX, int K, long NL,
                       int Co, hipStream_t s);
+int launch_col_bwd_small(const float *gy, const float *X, const float *W, float *gW, float *gX, int K, long NL, int Co,
+                         hipStream_t s);
 int launch_col_bwd_fused(const float *gy, const float *X, const float *W, float *gW, float *gX, int K, long NL, int Co,
                          void *ws, hipStream_t s);
 

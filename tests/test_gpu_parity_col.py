@@ -12,7 +12,10 @@ CASES = [(32, 288, 1024), (16, 144, 512), (12, 36, 240), (7, 27, 101), (1, 1, 1)
          # many columns (two columns per lane, slabs from every workgroup) with a ragged last group; 17..32 and more
          # than 32 output channels (other kernels); tile tails on both sides of the weight-gradient product
          (16, 144, 65544), (9, 20, 70004), (24, 50, 66000), (48, 40, 2052), (64, 576, 1000), (20, 200, 4100),
-         (40, 150, 66562)]
+         (40, 150, 66562),
+         # few columns (one launch for both gradients, a workgroup per row or pair of rows of X over all columns):
+         # 1, 2, 4 and 8 columns per thread, a tall matrix with an odd row count, more channels than a batch of gy
+         (5, 7, 3), (17, 9, 1500), (40, 1031, 300), (64, 33, 2048), (130, 12, 700), (3, 2050, 513)]
 
 
 def _data(Co, K, NL, seed=0, scale=1.0):
