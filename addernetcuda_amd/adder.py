@@ -57,7 +57,9 @@ class adder(Function):
 
 
 # while a batched_eta_scaling() block is open: one entry per layer whose weight gradient is pending,
-# (weight, eta, stage, workspace) -- stage / workspace are None where only the scaling is pending
+# (weight, eta, stage, workspace) -- stage / workspace are None where only the scaling is pending.
+# A module global and not a thread-local: the block is entered on the caller's thread, while the backward nodes
+# that append to it run on the autograd engine's device thread.
 _eta_batch = None
 
 

@@ -12,6 +12,21 @@
  * pybind functions of adder_cuda/adder_cuda.cpp:88-93 and the host launchers
  * behind them (adder_cuda/adder.cu:274-465), plus the PyTorch glue the
  * reference runs around them (adder.py:22-41 im2col/col2im, adder.py:78 scaling).
+ *
+ * Groups, in the order they appear below.  [core] is the reference's boundary and what a port needs;
+ * every [optional] group has a [core] equivalent that gives the same results in more launches, and
+ * answers ADDER_ERR_UNSUPPORTED (nothing launched) where it does not apply.
+ *   [core]      status / version / adder_out_dim
+ *   [core]      fused NCHW path: adder_conv2d_fwd_f32, adder_conv2d_bwd_f32, adder_conv2d_bwd_workspace_bytes
+ *   [optional]  ... its variants: _fwd_stats_ (BatchNorm statistics in the epilogue), _fwd_pair_stats_ (a strided
+ *               1x1 layer beside a strided 3x3), adder_plain_conv2d_fwd_f32 (an ordinary convolution through the same
+ *               kernel), _bwd_add_ (a second gradient added), _bf16 (bfloat16 storage), _bwd_noalloc_ (no workspace)
+ *   [core]      column-matrix path: adder_col_fwd_f32 / _bwd_f32 / _gradw_f32 / _gradx_f32 (= ADDER_CONV,
+ *               ADDER_BACKWARD, ADDER_CONV_WEIGHT, ADDER_CONV_INPUT), adder_col_bwd_workspace_bytes
+ *   [core]      adder_grad_norm_scale_f32 (adder.py:78 on its own);  [optional] the batched form
+ *   [optional]  grad_W in two stages (all layers finished together after the backward pass)
+ *   [optional]  BatchNorm + residual + ReLU kernels (adder_bn_act_*)
+ *   [optional]  BatchNorm backward passes folded into the adder backward kernels (adder_bn_links, *_bn_*)
  */
 #ifndef ADDERNET_HIP_H
 #define ADDERNET_HIP_H
@@ -50,7 +65,8 @@ ADDER_API int adder_abi_version(void);
 ADDER_API int adder_out_dim(int h, int k, int pad, int stride);
 
 /* ------------------------------------------------------------------------
- * Fused NCHW path (what adder2d itself uses).
+ * [core] Fused NCHW path (what adder2d itself uses); the variants between here and the column-matrix path
+ * are [optional].
  *   x  (N, Ci, H, W)        w  (Co, Ci, kh, kw)        y, gy (N, Co, Ho, Wo)
  * Zero padding; padded taps count as x = 0 (they add -|w| to y and -w*gy to
  * grad_w) exactly as F.unfold makes them do in adder.py:32.
@@ -160,7 +176,7 @@ ADDER_API int adder_conv2d_bwd_noalloc_f32(const float *gy, const float *x, cons
                          int stride, int pad, void *stream);
 
 /* ------------------------------------------------------------------------
- * Column-matrix path: the literal signatures of the reference extension.
+ * [core] Column-matrix path: the literal signatures of the reference extension.
  *   Xcol (K, NL)   Wcol (Co, K)   out, gy (Co, NL)   gW (Co, K)   gX (K, NL)
  * The reference ACCUMULATES into gW / gX (atomicAdd into caller-zeroed
  * buffers, adder.cu:125,186,266-267; adder.py:66-67); so do these.
@@ -190,7 +206,7 @@ ADDER_API int adder_col_gradx_f32(const float *gy, const float *Xcol, const floa
                         float *gX, int K, long NL, int Co, void *stream);
 
 /* ------------------------------------------------------------------------
- * Adaptive learning-rate scaling, in place (adder.py:78):
+ * [core] Adaptive learning-rate scaling, in place (adder.py:78):
  *   g <- g / max(||g||_2, eps) * sqrt(n) * eta
  * ws must hold adder_norm_scale_workspace_bytes(n) bytes.
  * ---------------------------------------------------------------------- */
@@ -209,7 +225,7 @@ ADDER_API int adder_grad_norm_scale_batched_f32(int count, float *const *g, cons
                               float eps, void *ws, size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
- * grad_W in two stages, for callers that finish the weight gradients of all their layers together after
+ * [optional] grad_W in two stages, for callers that finish the weight gradients of all their layers together after
  * the backward pass (two launches in all instead of two per layer; adder.py:62-80 has no counterpart, it
  * finishes every layer on the spot).
  *   adder_conv2d_grad_w_staged_f32: the position reduction of grad_W into partial slabs inside ws (same size
@@ -241,7 +257,7 @@ ADDER_API int adder_grad_w_finish_f32(int count, const adder_grad_w_stage *stage
                          void *stream);
 
 /* ------------------------------------------------------------------------
- * The element-wise neighbours of every adder layer: training-mode BatchNorm2d fused with the
+ * [optional] The element-wise neighbours of every adder layer: training-mode BatchNorm2d fused with the
  * residual add and ReLU that follow it.  The reference runs these as separate PyTorch ops
  * (resnet20.py:28-39: bn -> relu, bn -> += residual -> relu); here each direction is one
  * statistics pass and one apply pass.  x, y, residual, dy, dx, dresidual are (N, C, H*W).
@@ -278,7 +294,7 @@ ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsign
                                    int N, int C, int HW, void *ws, size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
- * The BatchNorm backward passes folded into the adder layers' backward kernels.  No counterpart in the
+ * [optional] The BatchNorm backward passes folded into the adder layers' backward kernels.  No counterpart in the
  * reference, where bn -> relu and the adder layer are separate autograd nodes (resnet20.py:28-39) and the
  * BatchNorm backward is two passes of its own over every activation gradient.  In a chain
  *     ... -> adder A -> BatchNorm P -> (+ residual) -> ReLU -> adder B -> BatchNorm Q -> ...
