@@ -102,6 +102,8 @@ STATS_CASES = [
     (2, 16, 32, 32, 32, 1, 2, 0), (3, 32, 16, 16, 64, 1, 2, 0), (2, 8, 8, 8, 4, 1, 1, 0), (3, 12, 7, 7, 20, 1, 1, 0),
     (2, 6, 9, 9, 10, 1, 2, 0), (3, 64, 14, 14, 72, 1, 1, 0), (2, 64, 28, 28, 72, 1, 2, 0),   # 1x1 kernels, element-wise and tiled
     (3, 84, 16, 16, 48, 1, 1, 0), (5, 68, 8, 8, 20, 1, 1, 0), (2, 76, 20, 20, 24, 1, 2, 0),   # ... units of four input channels
+    (2, 8, 24, 40, 12, 3, 1, 1), (3, 8, 20, 24, 8, 3, 1, 1), (2, 16, 56, 56, 8, 3, 1, 1),    # wide maps, 8- and 4-row tiles
+    (2, 64, 56, 56, 72, 1, 2, 0), (3, 72, 14, 14, 130, 1, 2, 0),                             # strided 1x1, 64-channel blocks
 ]
 
 

@@ -20,6 +20,9 @@ pytestmark = pytest.mark.gpu
 CASES = [(8, 16, 32, 32, 16, 1), (6, 16, 32, 32, 32, 2), (8, 32, 16, 16, 32, 1), (8, 32, 16, 16, 64, 2),
          (8, 64, 8, 8, 64, 1), (3, 20, 16, 16, 24, 1), (5, 12, 32, 32, 40, 1), (3, 6, 24, 40, 9, 2),
          (2, 5, 12, 20, 3, 1), (4, 8, 8, 8, 260, 1),   # the last one: the three-instruction grad_X form (2340 terms)
+         # wide maps whose height is not a multiple of 16: tiles of 8 rows (24, 56) and of 4 rows x two images (20, 28;
+         # three images: the last tile holds one)
+         (2, 8, 24, 40, 8, 1), (3, 8, 20, 24, 12, 1), (2, 16, 56, 56, 8, 1), (3, 8, 28, 28, 8, 1),
          # 1x1 layers: planes of 196 and 784 positions, planes of 64 (few and many workgroups), 128-channel blocks
          (4, 64, 14, 14, 256, 1, 1), (2, 256, 28, 28, 64, 1, 1), (8, 64, 8, 8, 64, 1, 1), (40, 72, 8, 8, 64, 1, 1),
          (3, 128, 8, 8, 128, 1, 1), (2, 128, 14, 14, 136, 1, 1), (2, 64, 6, 6, 1100, 1, 1)]

@@ -32,6 +32,10 @@ TILED = [
     (2, 9, 10, 18, 8, 3, 1, 1),     # odd channel count and W = 18
     (2, 8, 28, 28, 16, 3, 2, 1),    # strided, Wo = 14
     (2, 16, 14, 14, 16, 3, 2, 1),   # strided, W = 14 -> Wo = 7
+    (2, 8, 24, 40, 12, 3, 1, 1),    # wide map, 24 rows: tiles of 8 rows in four-wave workgroups
+    (3, 8, 20, 24, 8, 3, 1, 1),     # wide map, 20 rows: tiles of 4 rows of two images, odd image count
+    (2, 16, 56, 56, 8, 3, 1, 1),    # ResNet-50's 56x56 maps (7 x 8 rows)
+    (3, 8, 28, 28, 8, 3, 1, 1),     # ... and 28x28 (7 x 4 rows)
     (2, 16, 32, 32, 32, 1, 2, 0),   # ResNet-20 1x1 stride-2 downsample
     (2, 32, 16, 16, 64, 1, 2, 0),   # second downsample
     (2, 8, 8, 8, 16, 1, 1, 0),      # 1x1 stride 1
