@@ -81,7 +81,10 @@ class BnLinks(ctypes.Structure):
                 ("in_x", ctypes.c_void_p),
                 ("in_mean", ctypes.c_void_p), ("in_rstd", ctypes.c_void_p), ("in_part", ctypes.c_void_p),
                 ("in_slots", ctypes.c_int), ("in_relu", ctypes.c_int), ("in_gamma", ctypes.c_void_p),
-                ("in_beta", ctypes.c_void_p), ("side_gy", ctypes.c_void_p), ("side_w", ctypes.c_void_p)]
+                ("in_beta", ctypes.c_void_p), ("side_gy", ctypes.c_void_p), ("side_w", ctypes.c_void_p),
+                ("out_part", ctypes.c_void_p), ("out_slots", ctypes.c_int), ("out_gamma", ctypes.c_void_p),
+                ("out_mean", ctypes.c_void_p), ("out_rstd", ctypes.c_void_p), ("out_dgamma", ctypes.c_void_p),
+                ("out_dbeta", ctypes.c_void_p)]
 
 
 def check(status, what):

@@ -231,11 +231,11 @@ class BnLink:
     Made in the forward of the BatchNorm's node, which records the BatchNorm's input, statistics and weight; the
     layer that consumes the BatchNorm's output keeps a reference.  In the backward pass the consumer runs first:
     its input-gradient kernel leaves ``dz`` (the gradient of the BatchNorm's output before the ReLU) as its result
-    and the partial sums of the BatchNorm's backward, a small kernel turns those into ``coef`` / ``dgamma`` /
-    ``dbeta``, and the node of the BatchNorm, when it is handed exactly that ``dz`` tensor, skips its own two
-    passes."""
+    and the partial sums of the BatchNorm's backward (``sums``, (C, slots, 2) float64).  The node of the BatchNorm,
+    when it is handed exactly that ``dz`` tensor, skips its own two passes: the weight-gradient kernel of the layer
+    in front of the BatchNorm adds the sums, forms its output gradient from them and fills ``dgamma`` / ``dbeta``."""
     __slots__ = ("bn_x", "mean", "rstd", "gamma", "beta", "beta_version", "relu", "out_ptr", "out_shape", "out_version", "dz",
-                 "dz_version", "coef", "dgamma", "dbeta")
+                 "dz_version", "sums", "dgamma", "dbeta")
 
     def __init__(self, bn_x, mean, rstd, gamma, relu, beta=None):
         """``beta``: the BatchNorm's bias, given only when nothing was added to the BatchNorm's output (no residual):
@@ -243,7 +243,7 @@ class BnLink:
         self.bn_x, self.mean, self.rstd, self.gamma, self.beta, self.relu = bn_x, mean, rstd, gamma, beta, relu
         self.beta_version = None if beta is None else (beta._version, gamma._version)
         self.out_ptr = self.out_shape = self.out_version = None
-        self.dz = self.dz_version = self.coef = self.dgamma = self.dbeta = None
+        self.dz = self.dz_version = self.sums = self.dgamma = self.dbeta = None
 
     def attach(self, out):
         """Tie the link to the tensor that left the BatchNorm's node; consumers find it as ``out._adder_bn_link``."""
@@ -262,8 +262,15 @@ class BnLink:
     def claims(self, dy):
         """Whether ``dy`` is the very tensor the consumer's kernel wrote (not a sum autograd formed from it)."""
         dz = self.dz
-        return (dz is not None and dy.data_ptr() == dz.data_ptr() and dy.shape == dz.shape
+        return (dz is not None and self.sums is not None and dy.data_ptr() == dz.data_ptr() and dy.shape == dz.shape
                 and dy._version == self.dz_version and dy.is_contiguous())
+
+    def fill_out_half(self, links, gy_formed):
+        """The out_* half of ``links`` (a BnLinks) for the layer in front of this BatchNorm."""
+        links.out_x, links.out_gy = ptr(self.bn_x), ptr(gy_formed)
+        links.out_part, links.out_slots = ptr(self.sums), self.sums.size(1)
+        links.out_gamma, links.out_mean, links.out_rstd = ptr(self.gamma), ptr(self.mean), ptr(self.rstd)
+        links.out_dgamma, links.out_dbeta = ptr(self.dgamma), ptr(self.dbeta)
 
 
 def _aligned16(*tensors):
@@ -285,10 +292,11 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
     """The backward launches shared by the autograd nodes: (grad_X, grad_W), either None where not needed.
 
     ``grad_short``: a second gradient of X (a residual shortcut), added to grad_X by the kernel where it can.
-    ``out_link``: a BnLink whose ``coef`` is ready -- ``grad_out`` is then dz of the BatchNorm behind the layer
-    (the caller has checked ``bwd_bn_slots(dims)``, the alignment of the tensors and ``need_w``).
-    ``in_link``: the BnLink of the BatchNorm whose output X is -- grad_X leaves as dz, and the link receives dz,
-    coef, dgamma and dbeta (same checks by the caller, and ``need_x``).
+    ``out_link``: a BnLink that ``claims`` grad_out -- ``grad_out`` is then dz of the BatchNorm behind the layer, and
+    the weight-gradient kernel fills the link's dgamma / dbeta (the caller has checked ``bwd_bn_slots(dims)``, the
+    alignment of the tensors and ``need_w``).
+    ``in_link``: the BnLink of the BatchNorm whose output X is -- grad_X leaves as dz, and the link receives dz, the
+    sums and empty dgamma / dbeta (same checks by the caller, and ``need_x``).
     ``side``: (side_gy, side_w) of the strided 1x1 layer that reads X beside this (strided 3x3) layer and has left its
     input gradient to this call: added inside the input-gradient kernel where that takes ``in_link``, else computed
     by the 1x1 layer's own kernel and added like ``grad_short``."""
@@ -311,7 +319,7 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
         links = BnLinks()
         if out_link is not None:
             gy_formed = torch.empty_like(grad_out)
-            links.out_x, links.out_coef, links.out_gy = ptr(out_link.bn_x), ptr(out_link.coef), ptr(gy_formed)
+            out_link.fill_out_half(links, gy_formed)
         if in_link is not None:
             slots = bwd_bn_slots(dims)
             part = torch.empty((X.size(1), slots, 2), device=dev, dtype=torch.float64)
@@ -349,7 +357,7 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
         gw = None
         if out_link is not None:   # the staged kernel has formed the gradient of the layer's output
             grad_out = gy_formed
-            links.out_x = links.out_coef = links.out_gy = None
+            links.out_x = links.out_part = links.out_gy = None
     if need_x or gw is not None:
         with on_device(dev):
             ws, nbytes = conv2d_bwd_workspace(dims, dev) if gw is not None else (None, 0)
@@ -371,14 +379,9 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
                     if need_x and grad_short is not None:
                         gx += grad_short
             if in_link is not None:
-                C = X.size(1)
-                in_link.coef = torch.empty((C, 4), device=dev, dtype=torch.float32)
-                in_link.dgamma = torch.empty(C, device=dev, dtype=torch.float32)
-                in_link.dbeta = torch.empty(C, device=dev, dtype=torch.float32)
-                count = float(X.numel() // C)
-                check(lib.adder_bn_bwd_coef_f32(ptr(part), slots, ptr(in_link.gamma), ptr(in_link.mean), ptr(in_link.rstd),
-                                                count, ptr(in_link.coef), ptr(in_link.dgamma), ptr(in_link.dbeta), C,
-                                                stream_ptr(dev)), "adder_bn_bwd_coef_f32")
+                in_link.sums = part
+                in_link.dgamma = torch.empty(X.size(1), device=dev, dtype=torch.float32)
+                in_link.dbeta = torch.empty(X.size(1), device=dev, dtype=torch.float32)
                 in_link.dz, in_link.dz_version = gx, gx._version
     return gx, gw_out
 
@@ -492,9 +495,9 @@ def conv2d_weight_grad(grad_out, X, W, stride, padding, out_link=None):
     ``sum x * gy`` half of the adder layer's weight gradient, from the same fp64 matrix-core kernel (the slab
     finalize leaves the ``- w * sum gy`` term out).  Inside a ``batched_eta_scaling()`` block it is finished
     together with the adder layers' gradients.  Returns None where the geometry has no such kernel.
-    ``out_link``: a BnLink whose ``coef`` is ready -- ``grad_out`` is then dz of the BatchNorm behind the
-    convolution, and the kernel forms the convolution's output gradient from it (None is returned, and nothing
-    launched, where the kernel cannot)."""
+    ``out_link``: a BnLink that ``claims`` grad_out -- ``grad_out`` is then dz of the BatchNorm behind the
+    convolution, and the kernel forms the convolution's output gradient from it and fills the link's dgamma / dbeta
+    (None is returned, and nothing launched, where the kernel cannot)."""
     grad_out, X = grad_out.contiguous(), X.contiguous()
     require_gpu_f32(grad_out, "grad_output")
     require_gpu_f32(X, "X")
@@ -506,7 +509,7 @@ def conv2d_weight_grad(grad_out, X, W, stride, padding, out_link=None):
         stage = GradWStage()
         if out_link is not None:
             links = BnLinks()
-            links.out_x, links.out_coef = ptr(out_link.bn_x), ptr(out_link.coef)
+            out_link.fill_out_half(links, None)
             status = lib.adder_conv2d_grad_w_staged_bn_f32(ptr(grad_out), ptr(X), None, ptr(gw), 0.0, ptr(ws), nbytes,
                                                            *dims, ctypes.byref(links), ctypes.byref(stage),
                                                            stream_ptr(dev))

@@ -64,6 +64,35 @@ static bool overlaps(const void *a, size_t na, const void *b, size_t nb) {
     return pa < pb + nb && pb < pa + na;
 }
 
+struct Span { const void *p; size_t bytes; };
+
+// no output may overlap an input or another output
+template <int NO, int NI>
+static bool any_alias(const Span (&outs)[NO], const Span (&ins)[NI]) {
+    for (int o = 0; o < NO; ++o) {
+        for (int i = 0; i < NI; ++i)
+            if (overlaps(outs[o].p, outs[o].bytes, ins[i].p, ins[i].bytes)) return true;
+        for (int q = o + 1; q < NO; ++q)
+            if (overlaps(outs[o].p, outs[o].bytes, outs[q].p, outs[q].bytes)) return true;
+    }
+    return false;
+}
+
+// The out_* half of adder_bn_links: out_x with exactly one of out_coef and out_part (+ what belongs to it).
+static int bn_out_half(const adder_bn_links &bn, const ConvDims &d, BnSums &sums) {
+    sums = kNoBnSums;
+    if (!bn.out_x) return (bn.out_coef || bn.out_part || bn.out_gy) ? ADDER_ERR_NULL_POINTER : ADDER_OK;
+    if ((bn.out_coef == nullptr) == (bn.out_part == nullptr)) return ADDER_ERR_NULL_POINTER;
+    if (bn.out_part) {
+        if (!bn.out_gamma || !bn.out_mean || !bn.out_rstd || !bn.out_dgamma || !bn.out_dbeta)
+            return ADDER_ERR_NULL_POINTER;
+        if (bn.out_slots < 1) return ADDER_ERR_BAD_SHAPE;
+        sums = BnSums{bn.out_part, bn.out_slots, (double)d.N * d.Ho * d.Wo, bn.out_gamma, bn.out_mean, bn.out_rstd,
+                      bn.out_dgamma, bn.out_dbeta};
+    }
+    return ADDER_OK;
+}
+
 }  // namespace adder
 
 using namespace adder;
@@ -86,7 +115,7 @@ const char *adder_strerror(int status) {
 
 const char *adder_last_hip_error(void) { return g_last_hip_error.c_str(); }
 
-int adder_abi_version(void) { return 5; }
+int adder_abi_version(void) { return 6; }
 
 int adder_out_dim(int h, int k, int pad, int stride) {
     if (h <= 0 || k <= 0 || pad < 0 || stride <= 0 || h + 2 * pad < k) return 0;
@@ -389,25 +418,23 @@ int adder_conv2d_grad_w_staged_bn_f32(const float *gy, const float *x, const flo
                                       size_t ws_bytes, int N, int Ci, int H, int W, int Co, int kh, int kw, int stride,
                                       int pad, const adder_bn_links *links, adder_grad_w_stage *stage, void *stream) {
     if (!gy || !x || !gw || !stage) return ADDER_ERR_NULL_POINTER;
-    const float *bn_y = links ? links->out_x : nullptr, *bn_coef = links ? links->out_coef : nullptr;
-    float *gy_out = links ? links->out_gy : nullptr;
-    if ((bn_y == nullptr) != (bn_coef == nullptr) || (gy_out && !bn_y)) return ADDER_ERR_NULL_POINTER;
     if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
     ConvDims d;
     if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    const adder_bn_links bn = links ? *links : adder_bn_links{};
+    BnSums sums;
+    if (int rc = bn_out_half(bn, d, sums)) return rc;
     const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
-                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo;
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo, nco = sizeof(float) * (size_t)Co;
     const size_t need = grad_w_workspace_bytes(d);
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
-    if (overlaps(ws, need, x, nx) || overlaps(ws, need, w, nw) || overlaps(ws, need, gy, ny) ||
-        overlaps(ws, need, gw, nw) || overlaps(gw, nw, x, nx) || overlaps(gw, nw, w, nw) || overlaps(gw, nw, gy, ny) ||
-        overlaps(ws, need, bn_y, ny) || overlaps(gw, nw, bn_y, ny) || overlaps(ws, need, bn_coef, 16 * (size_t)Co) ||
-        overlaps(gw, nw, bn_coef, 16 * (size_t)Co) || overlaps(gy_out, ny, gy, ny) || overlaps(gy_out, ny, x, nx) ||
-        overlaps(gy_out, ny, w, nw) || overlaps(gy_out, ny, bn_y, ny) || overlaps(gy_out, ny, bn_coef, 16 * (size_t)Co) ||
-        overlaps(gy_out, ny, gw, nw) || overlaps(gy_out, ny, ws, need))
-        return ADDER_ERR_ALIAS;
-    return launch_grad_w_staged(gy, x, w, gw, eta, ws, ws_bytes, d, stage, static_cast<hipStream_t>(stream), bn_y,
-                                bn_coef, gy_out);
+    const Span outs[] = {{ws, need}, {gw, nw}, {bn.out_gy, ny}, {bn.out_dgamma, nco}, {bn.out_dbeta, nco}};
+    const Span ins[] = {{x, nx}, {w, nw}, {gy, ny}, {bn.out_x, ny}, {bn.out_coef, 4 * nco},
+                        {bn.out_part, sizeof(double) * 2 * (size_t)Co * (size_t)(bn.out_slots > 0 ? bn.out_slots : 0)},
+                        {bn.out_gamma, nco}, {bn.out_mean, nco}, {bn.out_rstd, nco}};
+    if (any_alias(outs, ins)) return ADDER_ERR_ALIAS;
+    return launch_grad_w_staged(gy, x, w, gw, eta, ws, ws_bytes, d, stage, static_cast<hipStream_t>(stream), bn.out_x,
+                                bn.out_coef, bn.out_gy, sums);
 }
 
 int adder_conv2d_bwd_bn_slots(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad, int *slots) {
@@ -426,47 +453,42 @@ int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, con
     if (!gx && !gw) return ADDER_ERR_NULL_POINTER;
     if (!(eta >= 0.f)) return ADDER_ERR_BAD_SHAPE;
     const adder_bn_links bn = *links;
-    if ((bn.out_x == nullptr) != (bn.out_coef == nullptr) || (bn.out_gy && !bn.out_x)) return ADDER_ERR_NULL_POINTER;
+    ConvDims d;
+    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
+    BnSums sums;
+    if (int rc = bn_out_half(bn, d, sums)) return rc;
     if (bn.out_x && gx && !bn.out_gy) return ADDER_ERR_NULL_POINTER;   // grad_X reads the gradient grad_W leaves there
     if (bn.in_part && (!bn.in_x || !bn.in_mean || !bn.in_rstd || !gx)) return ADDER_ERR_NULL_POINTER;
     if ((bn.in_gamma == nullptr) != (bn.in_beta == nullptr)) return ADDER_ERR_NULL_POINTER;
     if ((bn.side_gy == nullptr) != (bn.side_w == nullptr)) return ADDER_ERR_NULL_POINTER;
     if (bn.side_gy && (!bn.in_part || kh != 3 || kw != 3 || stride != 2 || pad != 1 || (H & 1) || (W & 1)))
         return ADDER_ERR_UNSUPPORTED;
-    ConvDims d;
-    if (int rc = make_dims(N, Ci, H, W, Co, kh, kw, stride, pad, d)) return rc;
     const int slots = grad_w_bn_supported(d, nullptr, nullptr, nullptr, nullptr) ? grad_x_bn_slots(d) : 0;
     if (slots == 0 || (bn.out_x && !gw)) return ADDER_ERR_UNSUPPORTED;   // (the grad_W kernel is the one that forms gy)
     if (bn.in_part && bn.in_slots != slots) return ADDER_ERR_BAD_SHAPE;
     const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
                  ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo, np = sizeof(double) * 2 * (size_t)Ci * slots,
-                 nc = 16 * (size_t)Co;
-    const void *ins[] = {gy, x, w, gx_add, bn.out_x, bn.out_coef, bn.in_x, bn.in_mean, bn.in_rstd,
-                         bn.in_gamma, bn.in_beta, bn.side_gy, bn.side_w};
-    const size_t in_bytes[] = {ny, nx, nw, nx, ny, nc, nx, 4 * (size_t)Ci, 4 * (size_t)Ci,
-                               4 * (size_t)Ci, 4 * (size_t)Ci, ny, sizeof(float) * (size_t)Co * Ci};
-    constexpr int kIns = sizeof(ins) / sizeof(ins[0]);
-    static_assert(kIns == sizeof(in_bytes) / sizeof(in_bytes[0]), "one size per input");
+                 nci = sizeof(float) * (size_t)Ci, nco = sizeof(float) * (size_t)Co;
     const size_t need = gw ? grad_w_workspace_bytes(d) : 0;
     if (gw && (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255))) return ADDER_ERR_WORKSPACE;
-    for (int i = 0; i < kIns; ++i)
-        if (overlaps(gx, nx, ins[i], in_bytes[i]) || overlaps(gw, nw, ins[i], in_bytes[i]) ||
-            overlaps(bn.in_part, np, ins[i], in_bytes[i]) || overlaps(bn.out_gy, ny, ins[i], in_bytes[i]) ||
-            (gw && overlaps(ws, need, ins[i], in_bytes[i])))
-            return ADDER_ERR_ALIAS;
-    if (overlaps(gx, nx, gw, nw) || overlaps(gx, nx, bn.in_part, np) || overlaps(gw, nw, bn.in_part, np) ||
-        overlaps(bn.out_gy, ny, gx, nx) || overlaps(bn.out_gy, ny, gw, nw) || overlaps(bn.out_gy, ny, bn.in_part, np) ||
-        (gw && (overlaps(ws, need, gx, nx) || overlaps(ws, need, gw, nw) || overlaps(ws, need, bn.in_part, np) ||
-                overlaps(ws, need, bn.out_gy, ny))))
-        return ADDER_ERR_ALIAS;
+    const Span outs[] = {{gx, nx}, {gw, nw}, {bn.in_part, np}, {bn.out_gy, ny}, {gw ? ws : nullptr, need},
+                         {bn.out_dgamma, nco}, {bn.out_dbeta, nco}};
+    const Span ins[] = {{gy, ny}, {x, nx}, {w, nw}, {gx_add, nx}, {bn.out_x, ny}, {bn.out_coef, 4 * nco},
+                        {bn.out_part, sizeof(double) * 2 * (size_t)Co * (size_t)(bn.out_slots > 0 ? bn.out_slots : 0)},
+                        {bn.out_gamma, nco}, {bn.out_mean, nco}, {bn.out_rstd, nco},
+                        {bn.in_x, nx}, {bn.in_mean, nci}, {bn.in_rstd, nci}, {bn.in_gamma, nci}, {bn.in_beta, nci},
+                        {bn.side_gy, ny}, {bn.side_w, sizeof(float) * (size_t)Co * Ci}};
+    if (any_alias(outs, ins)) return ADDER_ERR_ALIAS;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (bn.out_x && !grad_w_bn_supported(d, gy, x, bn.out_x, bn.out_coef)) return ADDER_ERR_UNSUPPORTED;
+    if (bn.out_x && !grad_w_bn_supported(d, gy, x, bn.out_x, bn.out_coef ? (const void *)bn.out_coef : (const void *)bn.out_part))
+        return ADDER_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(bn.out_gy) | reinterpret_cast<uintptr_t>(gx) | reinterpret_cast<uintptr_t>(gx_add) |
          reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(bn.in_x)) & 15)
         return ADDER_ERR_UNSUPPORTED;   // before the first launch: the grad_X kernel would refuse these
     // grad_W first: with the out_* half it is the kernel that turns dz into the gradient of y, which grad_X reads
     if (gw)
-        if (int rc = launch_grad_w(gy, x, w, gw, eta, ws, ws_bytes, d, s, bn.out_x, bn.out_coef, bn.out_gy)) return rc;
+        if (int rc = launch_grad_w(gy, x, w, gw, eta, ws, ws_bytes, d, s, bn.out_x, bn.out_coef, bn.out_gy, sums))
+            return rc;
     if (gx)
         if (int rc = launch_grad_x_bn(bn.out_x ? bn.out_gy : gy, x, w, gx, d, s, gx_add, bn)) return rc;
     return ADDER_OK;

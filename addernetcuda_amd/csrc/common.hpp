@@ -240,9 +240,21 @@ int launch_mulconv_fwd(const float *x, const float *w, float *y, double *stats, 
 int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d,
                   hipStream_t s, const float *gadd = nullptr);
 size_t grad_w_workspace_bytes(const ConvDims &d);
+// The sums of the backward of the BatchNorm behind a layer, as the consumer's input-gradient kernel left them
+// ((C, slots, 2) doubles: sum dz, sum dz * xhat), with what turns them into the four coefficients per channel.
+// A weight-gradient kernel that is given these instead of ready coefficients adds the slots itself (every
+// workgroup its own channels, all in the same order) and writes dgamma / dbeta on the way.  part == null: not used.
+struct BnSums {
+    const double *part;
+    int slots;
+    double count;            // N * Ho * Wo: values per channel of the BatchNorm
+    const float *gamma, *mean, *rstd;
+    float *dgamma, *dbeta;
+};
+static constexpr BnSums kNoBnSums{nullptr, 0, 0.0, nullptr, nullptr, nullptr, nullptr, nullptr};
 int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta,
                   void *ws, size_t ws_bytes, const ConvDims &d, hipStream_t s, const float *bn_y = nullptr,
-                  const float *bn_coef = nullptr, float *gy_out = nullptr);
+                  const float *bn_coef = nullptr, float *gy_out = nullptr, const BnSums &sums = kNoBnSums);
 // the BatchNorm backward passes of a layer's neighbours inside the layer's backward kernels (adder_bn_links)
 int grad_x_bn_slots(const ConvDims &d);
 int launch_grad_x_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d, hipStream_t s,
@@ -257,7 +269,8 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d);
 int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
                        const GradWMfmaPlan &p, hipStream_t s);
 int launch_grad_w_mfma_bn(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
-                          const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s);
+                          const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s,
+                          const BnSums &sums = kNoBnSums);
 
 // 1x1 / pad 0 / stride 1-2 kernels (conv1x1.hip)
 bool conv1x1_supported(const ConvDims &d, const void *a, const void *b);
@@ -286,7 +299,8 @@ static constexpr int kNormBatchMax = ADDER_NORM_BATCH_MAX;
 static constexpr int kGwFinishMax = ADDER_GRAD_W_FINISH_MAX;
 int launch_grad_w_staged(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
                          size_t ws_bytes, const ConvDims &d, adder_grad_w_stage *stage, hipStream_t s,
-                         const float *bn_y = nullptr, const float *bn_coef = nullptr, float *gy_out = nullptr);
+                         const float *bn_y = nullptr, const float *bn_coef = nullptr, float *gy_out = nullptr,
+                         const BnSums &sums = kNoBnSums);
 size_t grad_w_finish_workspace_bytes(int count, const adder_grad_w_stage *st);
 int launch_grad_w_finish(int count, const adder_grad_w_stage *st, void *ws, hipStream_t s);
 size_t norm_scale_batched_workspace_bytes(int count);

@@ -374,15 +374,16 @@ size_t grad_w_workspace_bytes(const ConvDims &d) {
     return (bytes + 255) & ~(size_t)255;
 }
 
-// bn_y, bn_coef (both or neither): gy is the gradient dz of the output of the BatchNorm behind the layer and the
-// kernel forms the layer's own output gradient from it, leaving it in gy_out (nullable) on the way (matrix-core
-// 3x3 kernels only: ADDER_ERR_UNSUPPORTED, nothing launched, elsewhere)
+// bn_y with either bn_coef or sums.part: gy is the gradient dz of the output of the BatchNorm behind the layer and
+// the kernel forms the layer's own output gradient from it, leaving it in gy_out (nullable) on the way (matrix-core
+// kernels only: ADDER_ERR_UNSUPPORTED, nothing launched, elsewhere)
 int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
                   size_t ws_bytes, const ConvDims &d, hipStream_t s, const float *bn_y, const float *bn_coef,
-                  float *gy_out) {
+                  float *gy_out, const BnSums &sums) {
     if (ws_bytes < grad_w_workspace_bytes(d)) return ADDER_ERR_WORKSPACE;
     GradWPlan p = plan_grad_w(d);
-    if (bn_y && !grad_w_bn_supported(d, gy, x, bn_y, bn_coef)) return ADDER_ERR_UNSUPPORTED;
+    if (bn_y && !grad_w_bn_supported(d, gy, x, bn_y, bn_coef ? (const void *)bn_coef : (const void *)sums.part))
+        return ADDER_ERR_UNSUPPORTED;
     // float4 loads need 16-byte aligned bases; tensors whose rows are read element by element do not
     // (1x1 layers on the matrix cores walk whole planes as rows: their row length is H*W)
     const bool rows_1x1 = p.variant == 2 && d.kh == 1;
@@ -402,7 +403,7 @@ int launch_grad_w(const float *gy, const float *x, const float *w, float *gw, fl
         if (p.variant == 2) {
             double *part = reinterpret_cast<double *>(ss + kNormBlocksMax);
             double *sgpart = part + (size_t)p.slots * d.Co * K;
-            rc = bn_y ? launch_grad_w_mfma_bn(gy, x, part, sgpart, d, p.mfma, bn_y, bn_coef, gy_out, s)
+            rc = bn_y ? launch_grad_w_mfma_bn(gy, x, part, sgpart, d, p.mfma, bn_y, bn_coef, gy_out, s, sums)
                       : launch_grad_w_mfma(gy, x, part, sgpart, d, p.mfma, s);
             if (rc) return rc;
             hipLaunchKernelGGL(grad_w_finalize_kernel<double>, dim3(nb), dim3(kFinOut * kFinLanes), 0, s, part,
@@ -474,10 +475,11 @@ int launch_grad_w_bf16(const bf16_t *gy, const bf16_t *x, const float *w, float 
 // ---- staged weight gradient: partial slabs now, finalize + scaling for many layers later --------------
 int launch_grad_w_staged(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
                          size_t ws_bytes, const ConvDims &d, adder_grad_w_stage *stage, hipStream_t s,
-                         const float *bn_y, const float *bn_coef, float *gy_out) {
+                         const float *bn_y, const float *bn_coef, float *gy_out, const BnSums &sums) {
     if (ws_bytes < grad_w_workspace_bytes(d)) return ADDER_ERR_WORKSPACE;
     GradWPlan p = plan_grad_w(d);
-    if (bn_y && !grad_w_bn_supported(d, gy, x, bn_y, bn_coef)) return ADDER_ERR_UNSUPPORTED;
+    if (bn_y && !grad_w_bn_supported(d, gy, x, bn_y, bn_coef ? (const void *)bn_coef : (const void *)sums.part))
+        return ADDER_ERR_UNSUPPORTED;
     const bool rows_1x1 = p.variant == 2 && d.kh == 1;
     const bool need_x16 = p.variant == 2 && !(rows_1x1 && d.stride > 1) && (rows_1x1 ? d.H * d.W : d.W) % 4 == 0;
     const bool need_g16 = p.variant == 2 && (rows_1x1 ? d.Ho * d.Wo : d.Wo) % 4 == 0;
@@ -490,7 +492,7 @@ int launch_grad_w_staged(const float *gy, const float *x, const float *w, float 
     if (p.variant == 2) {
         double *part = reinterpret_cast<double *>(ss + kNormBlocksMax);
         double *sgpart = part + (size_t)p.slots * d.Co * K;
-        rc = bn_y ? launch_grad_w_mfma_bn(gy, x, part, sgpart, d, p.mfma, bn_y, bn_coef, gy_out, s)
+        rc = bn_y ? launch_grad_w_mfma_bn(gy, x, part, sgpart, d, p.mfma, bn_y, bn_coef, gy_out, s, sums)
                   : launch_grad_w_mfma(gy, x, part, sgpart, d, p.mfma, s);
         stage->part = part;
         stage->sgpart = sgpart;

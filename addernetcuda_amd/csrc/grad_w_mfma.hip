@@ -134,6 +134,53 @@ __device__ __forceinline__ void gy_commit_m_bn(const GyStageM<G> &sg, const GySt
     }
 }
 
+// The four coefficients of gy_commit_m_bn for the workgroup's COB channels, from the sums the consumer's
+// input-gradient kernel left (BnSums): 32 lanes add the slots of one channel, always in the same order, so every
+// workgroup that needs a channel arrives at the same bits.  `write`: also store dgamma / dbeta of these channels
+// (one workgroup per channel block does).  Stands in for a launch of its own between the two kernels.
+template <class G>
+__device__ __forceinline__ void bn_coef_from_sums(const BnSums &b, int co0, int Co, float4 *coef, bool write) {
+    constexpr int GROUPS = G::NTHREADS / 32;
+    constexpr int CHUNK = G::KS == 3 ? 16 : 8;   // (the 1x1 kernels have few registers to spare)
+    const int sub = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    for (int cb = 0; cb < G::COB; cb += GROUPS) {
+        const int c = cb + grp;
+        if (G::COB % GROUPS == 0 || c < G::COB) {
+            const int co = min(co0 + c, Co - 1);
+            const float rs = b.rstd[co], gm = b.gamma[co], mu = b.mean[co];
+            const double2 *p = reinterpret_cast<const double2 *>(b.part) + (size_t)co * b.slots;
+            double s1 = 0.0, s2 = 0.0;
+            for (int s0 = sub; s0 < b.slots; s0 += 32 * CHUNK) {   // CHUNK loads in flight, then added in slot order
+                double2 v[CHUNK];
+#pragma unroll
+                for (int j = 0; j < CHUNK; ++j) {
+                    const int s = s0 + 32 * j;
+                    v[j] = s < b.slots ? p[s] : make_double2(0.0, 0.0);
+                }
+#pragma unroll
+                for (int j = 0; j < CHUNK; ++j) {
+                    s1 += v[j].x;
+                    s2 += v[j].y;
+                }
+            }
+#pragma unroll
+            for (int m = 16; m >= 1; m >>= 1) {   // (stays inside the 32-lane half)
+                s1 += __shfl_xor(s1, m, 64);
+                s2 += __shfl_xor(s2, m, 64);
+            }
+            if (sub == 0) {
+                const float m1 = (float)(s1 / b.count), m2 = (float)(s2 / b.count);
+                const float k = gm * rs;
+                coef[c] = make_float4(k, -k * rs * m2, mu, k * m1);
+                if (write && co0 + c < Co) {
+                    b.dbeta[co] = (float)s1;
+                    b.dgamma[co] = (float)s2;
+                }
+            }
+        }
+    }
+}
+
 // SUB (single tap only): x is a sampled tensor (see Subsample), read element by element at the sampled
 // positions; gy is dense.  VEC then only says how gy is read.
 // T: storage type of gy and x (float, or bf16_t for the reduced-storage mode); staged as fp32, multiplied in fp64.
@@ -148,7 +195,7 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
                                                                   int tilesW, int ntiles, const Subsample sub,
                                                                   const float *__restrict__ bn_y,
                                                                   const float *__restrict__ bn_coef,
-                                                                  float *__restrict__ gy_out) {
+                                                                  float *__restrict__ gy_out, const BnSums sums) {
     static_assert(!FUSE || (VEC && !SUB && sizeof(T) == 4), "the BatchNorm link belongs to the float kernels");
     using XP = typename G::XP;
     constexpr int S = G::S, MT = G::MT, NT = G::NT;
@@ -183,12 +230,6 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
     GyStageM<G> gs, ys;   // (ys: FUSE only)
     const float4 *coef = reinterpret_cast<const float4 *>(smem + G::LDS_FLOATS);
     float *const gy_dst = blockIdx.z == 0 ? gy_out : nullptr;   // every gy tile is staged once per k block
-    if constexpr (FUSE) {
-        for (int e = threadIdx.x; e < G::COB; e += G::NTHREADS)
-            reinterpret_cast<float4 *>(smem + G::LDS_FLOATS)[e] =
-                reinterpret_cast<const float4 *>(bn_coef)[min(co_blk + e, Co - 1)];
-        __syncthreads();
-    }
     int tile = blockIdx.x;
     int n0 = 0, h0 = 0, w0 = 0;
     auto decode = [&](int t) {
@@ -201,6 +242,18 @@ __global__ __launch_bounds__(G::NTHREADS) void grad_w_mfma_kernel(const T *__res
         tile_fetch<XP, VEC && !SUB, SUB, T>(xs, x, ci_blk, Ci, n0, N, h0 * S - G::PAD, w0 * S, H, W, sub);
         gy_fetch_m<G, VEC, T>(gs, gy, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         if constexpr (FUSE) gy_fetch_m<G, true, float>(ys, bn_y, co_blk, Co, n0, N, h0, w0, Ho, Wo);
+    }
+    if constexpr (FUSE) {   // the block's coefficients, while the first tile's loads are under way
+        float4 *cdst = reinterpret_cast<float4 *>(smem + G::LDS_FLOATS);
+        if (sums.part) {
+            bn_coef_from_sums<G>(sums, co_blk, Co, cdst, blockIdx.x == 0 && blockIdx.z == 0);
+        } else {
+            for (int e = threadIdx.x; e < G::COB; e += G::NTHREADS)
+                cdst[e] = reinterpret_cast<const float4 *>(bn_coef)[min(co_blk + e, Co - 1)];
+        }
+        __syncthreads();
+    }
+    if (tile < ntiles) {
         tile_commit<XP>(xs, smem);
         if constexpr (FUSE) gy_commit_m_bn<G>(gs, ys, smem + XP::BUF, coef, gy_dst, co_blk, Co, n0, N, h0, w0, Ho, Wo);
         else gy_commit_m<G>(gs, smem + XP::BUF);
@@ -395,12 +448,13 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
 template <class G, bool VEC, bool SUB = false, class T = float, bool FUSE = false>
 static int launch_one_v(const T *gy, const T *x, double *part, double *sgpart, const ConvDims &d,
                       const GradWMfmaPlan &p, hipStream_t s, const Subsample sub = Subsample{1, 0, 0, 0},
-                      const float *bn_y = nullptr, const float *bn_coef = nullptr, float *gy_out = nullptr) {
+                      const float *bn_y = nullptr, const float *bn_coef = nullptr, float *gy_out = nullptr,
+                      const BnSums &sums = kNoBnSums) {
     constexpr int LDS_BYTES = G::LDS_BYTES + (FUSE ? G::COB * 16 : 0);   // + the BatchNorm coefficients of the block
     if (int rc = allow_dynamic_lds<&grad_w_mfma_kernel<G, VEC, SUB, T, FUSE>>(LDS_BYTES)) return rc;
     hipLaunchKernelGGL((grad_w_mfma_kernel<G, VEC, SUB, T, FUSE>), dim3(p.slots, p.gy, p.gz), dim3(G::NTHREADS), LDS_BYTES, s,
                        gy, x, part, sgpart, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, p.tilesH, p.tilesW, p.ntiles, sub, bn_y,
-                       bn_coef, gy_out);
+                       bn_coef, gy_out, sums);
     return check_launch();
 }
 
@@ -429,30 +483,26 @@ int launch_grad_w_mfma_bf16(const bf16_t *gy, const bf16_t *x, double *part, dou
 // left in gy_out (nullable) on the way (see gy_commit_m_bn); ADDER_ERR_UNSUPPORTED for other variants and for rows
 // (planes, for 1x1 layers) that are not whole float4 groups.
 int launch_grad_w_mfma_bn(const float *gy, const float *x, double *part, double *sgpart, const ConvDims &d,
-                          const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s) {
+                          const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s,
+                          const BnSums &sums) {
     const Subsample none{1, 0, 0, 0};
     if (p.variant >= 1 && p.variant <= 5 && (d.W % 4 != 0 || d.Wo % 4 != 0)) return ADDER_ERR_UNSUPPORTED;
     switch (p.variant) {
-        case 1: return launch_one_v<GmW32, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
-                                                                           gy_out);
-        case 2: return launch_one_v<GmW16, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
-                                                                           gy_out);
-        case 3: return launch_one_v<GmW8, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
-                                                                           gy_out);
-        case 4: return launch_one_v<GmW16S2, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
-                                                                           gy_out);
-        case 5: return launch_one_v<GmW8S2, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
-                                                                           gy_out);
+        case 1: return launch_one_v<GmW32, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
+        case 2: return launch_one_v<GmW16, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
+        case 3: return launch_one_v<GmW8, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
+        case 4: return launch_one_v<GmW16S2, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
+        case 5: return launch_one_v<GmW8S2, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
         default: break;
     }
     // 1x1 stride-1 layers: whole planes as rows
     const ConvDims f = mfma_one_row(d);
     if (d.stride != 1 || f.W % 4 != 0) return ADDER_ERR_UNSUPPORTED;
     switch (p.variant) {
-        case 6: return launch_one_v<Gm1x1, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
-        case 7: return launch_one_v<Gm1x1s, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
-        case 10: return launch_one_v<Gm1x1b, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
-        case 12: return launch_one_v<Gm1x1c, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out);
+        case 6: return launch_one_v<Gm1x1, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out, sums);
+        case 7: return launch_one_v<Gm1x1s, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out, sums);
+        case 10: return launch_one_v<Gm1x1b, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out, sums);
+        case 12: return launch_one_v<Gm1x1c, true, false, float, true>(gy, x, part, sgpart, f, p, s, none, bn_y, bn_coef, gy_out, sums);
         default: return ADDER_ERR_UNSUPPORTED;
     }
 }

@@ -129,7 +129,7 @@ class _conv_bn_act(torch.autograd.Function):
         gx = gw = dgamma = dbeta = None
         # (link is None on a second pass through a retained graph: the separate BatchNorm backward below)
         if (link is not None and not ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and link.claims(dy)
-                and link.coef is not None and all(t.data_ptr() % 16 == 0 for t in (x, conv_out, dy))):
+                and all(t.data_ptr() % 16 == 0 for t in (x, conv_out, dy))):
             gw = _adder.conv2d_weight_grad(dy, x, w, stride, padding, out_link=link)   # None: not with this kernel
             if gw is not None:
                 dgamma, dbeta = link.dgamma, link.dbeta

@@ -10,11 +10,11 @@ disappear into the adder kernels on either side of the BatchNorm.
 
 * V's input-gradient kernel has x = U's output and its own result in registers: it writes
   dz = (grad_X + shortcut gradient) * [x > 0], which is the gradient of P's output before the ReLU and of the
-  shortcut, together with P's per-channel sums of dz and dz * xhat; a one-workgroup-per-channel kernel turns the
-  sums into dgamma, dbeta and four coefficients per channel (``BnLink``).
+  shortcut, together with P's per-channel partial sums of dz and dz * xhat (``BnLink``).
 * U's backward is handed that very tensor by autograd, recognises it (``BnLink.claims``), and A's weight-gradient
-  kernel forms A's output gradient from (dz, A's output, coefficients) while staging it, leaving it in memory for
-  A's input-gradient kernel.
+  kernel adds the partial sums (which gives dgamma, dbeta and four coefficients per channel) and forms A's output
+  gradient from (dz, A's output, coefficients) while staging it, leaving it in memory for A's input-gradient
+  kernel.
 
 Whenever the hand-over does not apply (autograd summed several gradients into a new tensor, the consumer is not
 an adder layer with such kernels, the weights are frozen, a tensor is not 16-byte aligned) the node runs the
@@ -99,7 +99,7 @@ class _adder_bn_act(Function):
         usable = _adder.bn_links_usable(ctx.dims, X, W, conv_out, dy, grad_short)
         out_link, in_link = ctx.out_link, ctx.in_link
         ctx.out_link = ctx.in_link = None
-        if usable and need_w and out_link is not None and out_link.claims(dy) and out_link.coef is not None:
+        if usable and need_w and out_link is not None and out_link.claims(dy):
             # dy is dz, written by the consumer's kernel together with this BatchNorm's sums
             gy, dres, dgamma, dbeta = dy, (dy if ctx.has_res else None), out_link.dgamma, out_link.dbeta
         else:

@@ -304,14 +304,20 @@ ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsign
  * first pass of P's backward).  And A's grad_W kernel can form its gy = dP_input from (dz, A's output y, four
  * numbers per channel) while it stages gy into LDS (the second pass):
  *     gy = k * dz + c2 * (y - mean) - km1,   k = gamma * rstd, c2 = -k * rstd * mean(dz * xhat), km1 = k * mean(dz),
- * and leave the result in memory for A's grad_X kernel, which runs after it.  P's backward is then one tiny
- * launch (adder_bn_bwd_coef_f32) instead of two passes over the activation gradient.
+ * and leave the result in memory for A's grad_X kernel, which runs after it.  P's backward is then no pass over
+ * the activation gradient at all: the four numbers come from the sums either in a tiny launch of their own
+ * (adder_bn_bwd_coef_f32) or in the first microsecond of A's grad_W kernel (out_part).
  *
  *   adder_bn_links: what a layer's backward is told about its two neighbours; either half may be absent (NULL).
- *     out_x, out_coef, out_gy   the BatchNorm BEHIND the layer: out_x = the layer's output y (N, Co, Ho, Wo),
- *                      out_coef = 4 floats per output channel {k, c2, mean, km1} from adder_bn_bwd_coef_f32;
- *                      the `gy` argument is then dz, not the gradient of y; out_gy (N, Co, Ho, Wo) receives the
- *                      gradient of y from the grad_W kernel.
+ *     out_x, out_coef | out_part.., out_gy   the BatchNorm BEHIND the layer: out_x = the layer's output y
+ *                      (N, Co, Ho, Wo); the `gy` argument is then dz, not the gradient of y; out_gy (N, Co, Ho, Wo)
+ *                      receives the gradient of y from the grad_W kernel.  The coefficients: exactly one of
+ *                      out_coef = 4 floats per output channel {k, c2, mean, km1} from adder_bn_bwd_coef_f32, or
+ *                      out_part = the sums as the consumer's call left them in its in_part (Co, out_slots, 2),
+ *                      16-byte aligned, with out_gamma / out_mean / out_rstd (Co): every workgroup of the grad_W
+ *                      kernel then adds the slots of its channels itself (the same fixed order as
+ *                      adder_bn_bwd_coef_f32, so the same values) and out_dgamma / out_dbeta (Co) are written by
+ *                      that kernel -- one launch fewer per layer.
  *     in_x, in_mean, in_rstd, in_part, in_slots, in_relu   the BatchNorm IN FRONT of the layer, whose output
  *                      (after the residual add and, if in_relu, the ReLU) is the layer's x: in_x = that
  *                      BatchNorm's input (N, Ci, H, W), its saved mean / rstd (Ci); in_part receives
@@ -351,6 +357,14 @@ typedef struct adder_bn_links {
        grad_X inside the kernel (before the mask and the sums), as if it had been passed as gx_add. */
     const float *side_gy;
     const float *side_w;
+    /* the alternative to out_coef (see above); all of them or none */
+    const double *out_part;
+    int out_slots;
+    const float *out_gamma;
+    const float *out_mean;
+    const float *out_rstd;
+    float *out_dgamma;
+    float *out_dbeta;
 } adder_bn_links;
 ADDER_API int adder_conv2d_bwd_bn_slots(int N, int Ci, int H, int W, int Co, int kh, int kw, int stride, int pad,
                                         int *slots);

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_status_strings_and_version():
     from addernetcuda_amd._lib import lib
-    assert lib.adder_abi_version() == 5
+    assert lib.adder_abi_version() == 6
     assert lib.adder_strerror(0) == b"ok"
     seen = {lib.adder_strerror(c) for c in range(-7, 1)}
     assert len(seen) == 8 and b"unknown status" not in seen

@@ -1,5 +1,5 @@
 """The BatchNorm backward passes folded into the adder backward kernels (adder_conv2d_bwd_bn_f32,
-adder_conv2d_grad_w_staged_bn_f32, adder_bn_bwd_coef_f32), through the C ABI, against the oracle's adder
+adder_conv2d_grad_w_staged_bn_f32, adder_bn_bwd_coef_f32 or the sums added by the grad_W kernel), through the C ABI, against the oracle's adder
 backward and the textbook BatchNorm backward evaluated in float64.
 
 Chain under test:  xp -> BatchNorm P -> (+ residual) -> ReLU -> x -> adder layer B -> y -> BatchNorm Q -> ...
@@ -163,6 +163,48 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, fro
     torch.cuda.synchronize()
     assert torch.equal(gx2, gxg)
 
+    # the same with Q's sums handed to the grad_W kernel itself (out_part) instead of ready coefficients: one slot
+    # gives the very same bits; many slots (unrolled part of the slot loop and its tail) the same values
+    for S in (1, 1100):
+        if S == 1:
+            part_s = part_qg
+        else:
+            g = torch.Generator().manual_seed(S)
+            pieces = torch.randn(Co, S, 2, generator=g, dtype=torch.float64)
+            pieces[:, -1] += part_q.view(Co, 2) - pieces.sum(1)
+            part_s = d(pieces)
+        dg3, db3 = torch.full((Co,), float("nan"), device=gpu), torch.full((Co,), float("nan"), device=gpu)
+        gy_out3, gw3, gx3 = torch.full_like(dzqg, float("nan")), torch.empty_like(wg), torch.empty_like(xg)
+        part3 = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float64, device=gpu)
+        links3 = BnLinks(ptr(y32g), None, ptr(gy_out3), ptr(xpg), ptr(mean_pg), ptr(rstd_pg), ptr(part3), slots, 1,
+                         ptr(gamma_pg), ptr(beta_pg), None, None, ptr(part_s), S, ptr(gamma_qg), ptr(mean_qg),
+                         ptr(rstd_qg), ptr(dg3), ptr(db3))
+        check(lib.adder_conv2d_bwd_bn_f32(ptr(dzqg), ptr(xg), ptr(wg), ptr(addg), ptr(gx3), ptr(gw3), 0.2, ptr(ws),
+                                          nbytes, *dims, ctypes.byref(links3), st), "adder_conv2d_bwd_bn_f32")
+        stage3 = GradWStage()
+        gw4, gy_out4 = torch.empty_like(wg), torch.empty_like(dzqg)
+        dg4, db4 = torch.empty(Co, device=gpu), torch.empty(Co, device=gpu)
+        links4 = BnLinks(ptr(y32g), None, ptr(gy_out4), None, None, None, None, 0, 0, None, None, None, None,
+                         ptr(part_s), S, ptr(gamma_qg), ptr(mean_qg), ptr(rstd_qg), ptr(dg4), ptr(db4))
+        check(lib.adder_conv2d_grad_w_staged_bn_f32(ptr(dzqg), ptr(xg), ptr(wg), ptr(gw4), 0.2, ptr(ws), nbytes, *dims,
+                                                    ctypes.byref(links4), ctypes.byref(stage3), st),
+              "adder_conv2d_grad_w_staged_bn_f32")
+        arr3 = (GradWStage * 1)(stage3)
+        check(lib.adder_grad_w_finish_f32(1, arr3, ptr(fws), need.value, st), "adder_grad_w_finish_f32")
+        torch.cuda.synchronize()
+        assert torch.equal(gw4, gw3) and torch.equal(gy_out4, gy_out3)
+        assert torch.equal(dg4, dg3) and torch.equal(db4, db3)
+        if S == 1:
+            assert torch.equal(dg3, dgq) and torch.equal(db3, dbq)
+            assert torch.equal(gy_out3, gy_out) and torch.equal(gw3, gwg) and torch.equal(gx3, gxg)
+            assert torch.equal(part3, part)
+        else:
+            assert_close(dg3, dgamma_q, "dgamma of Q from the grad_W kernel", rtol=1e-5, atol=1e-3)
+            assert_close(db3, dbeta_q, "dbeta of Q from the grad_W kernel", rtol=1e-5, atol=1e-3)
+            assert_close(gy_out3, gy, "gradient of y (sums added in the kernel)", rtol=1e-5, atol=1e-5)
+            assert_close(gx3, dz, "dz (sums added in the kernel)", rtol=2e-5, atol=2e-4)
+            assert_close(gw3, gw_scaled, "grad_W (sums added in the kernel)", rtol=2e-5, atol=2e-4)
+
 
 @pytest.mark.parametrize("case", [(8, 16, 32, 32, 16, 1), (8, 32, 16, 16, 64, 2), (3, 20, 16, 16, 24, 1),
                                   (4, 64, 14, 14, 96, 1, 1)], ids=str)
@@ -225,7 +267,17 @@ def test_refusals(gpu):
     rc = lib.adder_conv2d_bwd_bn_f32(ptr(t), ptr(t), ptr(t), None, ptr(t), None, 0.0, None, 0, *dims3, ctypes.byref(links),
                                      stream_ptr(gpu))
     assert rc == -1
-    links = BnLinks(ptr(t), None, None, None, None, None, None, 0, 0)     # out_x without out_coef
+    links = BnLinks(ptr(t), None, None, None, None, None, None, 0, 0)     # out_x without out_coef or out_part
+    rc = lib.adder_conv2d_bwd_bn_f32(ptr(t), ptr(t), ptr(t), None, ptr(t), None, 0.0, None, 0, *dims3, ctypes.byref(links),
+                                     stream_ptr(gpu))
+    assert rc == -1
+    links = BnLinks(ptr(t), ptr(t), None, None, None, None, None, 0, 0, None, None, None, None, ptr(part), 1, ptr(t), ptr(t),
+                    ptr(t), ptr(t), ptr(t))                               # both of them
+    rc = lib.adder_conv2d_bwd_bn_f32(ptr(t), ptr(t), ptr(t), None, ptr(t), None, 0.0, None, 0, *dims3, ctypes.byref(links),
+                                     stream_ptr(gpu))
+    assert rc == -1
+    links = BnLinks(ptr(t), None, None, None, None, None, None, 0, 0, None, None, None, None, ptr(part), 1, ptr(t), ptr(t),
+                    ptr(t), None, ptr(t))                                 # out_part without a place for dgamma
     rc = lib.adder_conv2d_bwd_bn_f32(ptr(t), ptr(t), ptr(t), None, ptr(t), None, 0.0, None, 0, *dims3, ctypes.byref(links),
                                      stream_ptr(gpu))
     assert rc == -1
