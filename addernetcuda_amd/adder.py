@@ -231,7 +231,7 @@ class BnLink:
     Made in the forward of the BatchNorm's node, which records the BatchNorm's input, statistics and weight; the
     layer that consumes the BatchNorm's output keeps a reference.  In the backward pass the consumer runs first:
     its input-gradient kernel leaves ``dz`` (the gradient of the BatchNorm's output before the ReLU) as its result
-    and the partial sums of the BatchNorm's backward (``sums``, (C, slots, 2) float64).  The node of the BatchNorm,
+    and the partial sums of the BatchNorm's backward (``sums``, (C, slots, 2) float32).  The node of the BatchNorm,
     when it is handed exactly that ``dz`` tensor, skips its own two passes: the weight-gradient kernel of the layer
     in front of the BatchNorm adds the sums, forms its output gradient from them and fills ``dgamma`` / ``dbeta``."""
     __slots__ = ("bn_x", "mean", "rstd", "gamma", "beta", "beta_version", "relu", "out_ptr", "out_shape", "out_version", "dz",
@@ -322,7 +322,7 @@ def conv_backward(X, W, grad_out, grad_short, dims, eta, need_x, need_w, w_is_gi
             out_link.fill_out_half(links, gy_formed)
         if in_link is not None:
             slots = bwd_bn_slots(dims)
-            part = torch.empty((X.size(1), slots, 2), device=dev, dtype=torch.float64)
+            part = torch.empty((X.size(1), slots, 2), device=dev, dtype=torch.float32)
             links.in_x, links.in_mean, links.in_rstd = ptr(in_link.bn_x), ptr(in_link.mean), ptr(in_link.rstd)
             links.in_part, links.in_slots, links.in_relu = ptr(part), slots, int(in_link.relu)
             if in_link.beta is not None and in_link.beta_version == (in_link.beta._version, in_link.gamma._version):

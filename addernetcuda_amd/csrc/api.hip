@@ -430,7 +430,7 @@ int adder_conv2d_grad_w_staged_bn_f32(const float *gy, const float *x, const flo
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255)) return ADDER_ERR_WORKSPACE;
     const Span outs[] = {{ws, need}, {gw, nw}, {bn.out_gy, ny}, {bn.out_dgamma, nco}, {bn.out_dbeta, nco}};
     const Span ins[] = {{x, nx}, {w, nw}, {gy, ny}, {bn.out_x, ny}, {bn.out_coef, 4 * nco},
-                        {bn.out_part, sizeof(double) * 2 * (size_t)Co * (size_t)(bn.out_slots > 0 ? bn.out_slots : 0)},
+                        {bn.out_part, sizeof(float) * 2 * (size_t)Co * (size_t)(bn.out_slots > 0 ? bn.out_slots : 0)},
                         {bn.out_gamma, nco}, {bn.out_mean, nco}, {bn.out_rstd, nco}};
     if (any_alias(outs, ins)) return ADDER_ERR_ALIAS;
     return launch_grad_w_staged(gy, x, w, gw, eta, ws, ws_bytes, d, stage, static_cast<hipStream_t>(stream), bn.out_x,
@@ -467,14 +467,14 @@ int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, con
     if (slots == 0 || (bn.out_x && !gw)) return ADDER_ERR_UNSUPPORTED;   // (the grad_W kernel is the one that forms gy)
     if (bn.in_part && bn.in_slots != slots) return ADDER_ERR_BAD_SHAPE;
     const size_t nx = sizeof(float) * (size_t)N * Ci * H * W, nw = sizeof(float) * (size_t)Co * d.K(),
-                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo, np = sizeof(double) * 2 * (size_t)Ci * slots,
+                 ny = sizeof(float) * (size_t)N * Co * d.Ho * d.Wo, np = sizeof(float) * 2 * (size_t)Ci * slots,
                  nci = sizeof(float) * (size_t)Ci, nco = sizeof(float) * (size_t)Co;
     const size_t need = gw ? grad_w_workspace_bytes(d) : 0;
     if (gw && (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255))) return ADDER_ERR_WORKSPACE;
     const Span outs[] = {{gx, nx}, {gw, nw}, {bn.in_part, np}, {bn.out_gy, ny}, {gw ? ws : nullptr, need},
                          {bn.out_dgamma, nco}, {bn.out_dbeta, nco}};
     const Span ins[] = {{gy, ny}, {x, nx}, {w, nw}, {gx_add, nx}, {bn.out_x, ny}, {bn.out_coef, 4 * nco},
-                        {bn.out_part, sizeof(double) * 2 * (size_t)Co * (size_t)(bn.out_slots > 0 ? bn.out_slots : 0)},
+                        {bn.out_part, sizeof(float) * 2 * (size_t)Co * (size_t)(bn.out_slots > 0 ? bn.out_slots : 0)},
                         {bn.out_gamma, nco}, {bn.out_mean, nco}, {bn.out_rstd, nco},
                         {bn.in_x, nx}, {bn.in_mean, nci}, {bn.in_rstd, nci}, {bn.in_gamma, nci}, {bn.in_beta, nci},
                         {bn.side_gy, ny}, {bn.side_w, sizeof(float) * (size_t)Co * Ci}};
@@ -494,7 +494,7 @@ int adder_conv2d_bwd_bn_f32(const float *gy, const float *x, const float *w, con
     return ADDER_OK;
 }
 
-int adder_bn_bwd_coef_f32(const double *part, int slots, const float *gamma, const float *save_mean,
+int adder_bn_bwd_coef_f32(const float *part, int slots, const float *gamma, const float *save_mean,
                           const float *save_rstd, double count, float *coef, float *dgamma, float *dbeta, int C,
                           void *stream) {
     if (!part || !gamma || !save_mean || !save_rstd || !coef || !dgamma || !dbeta) return ADDER_ERR_NULL_POINTER;

@@ -102,12 +102,13 @@ __global__ __launch_bounds__(kBnThreads) void bn_partial_kernel(const float *__r
 
 // Every workgroup of the second pass adds the S partials of its channel itself (same order in every
 // workgroup, so all of them see the same statistics) instead of waiting for a finalize launch.
-__device__ __forceinline__ void bn_reduce_partials(const double *__restrict__ part, int c, int S, double &s1,
+template <class T>
+__device__ __forceinline__ void bn_reduce_partials(const T *__restrict__ part, int c, int S, double &s1,
                                                    double &s2) {
     double a = 0.0, b = 0.0;
     for (int s = threadIdx.x; s < S; s += kBnThreads) {
-        a += part[((size_t)c * S + s) * 2];
-        b += part[((size_t)c * S + s) * 2 + 1];
+        a += (double)part[((size_t)c * S + s) * 2];
+        b += (double)part[((size_t)c * S + s) * 2 + 1];
     }
     __shared__ double ra[kBnThreads / 64], rb[kBnThreads / 64];
     a = wave_sum(a);
@@ -237,7 +238,7 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_apply_kernel(const float *_
 // kernel left (fixed order: the result does not depend on which workgroup finished first) and writes dbeta, dgamma
 // and the four numbers per channel from which the producer's backward kernels form their output gradient,
 //   dx = k * dz + c2 * (x - mean) - km1,   k = gamma * rstd, c2 = -k * rstd * mean(dz * xhat), km1 = k * mean(dz).
-__global__ __launch_bounds__(kBnThreads) void bn_bwd_coef_kernel(const double *__restrict__ part, int S, double count,
+__global__ __launch_bounds__(kBnThreads) void bn_bwd_coef_kernel(const float *__restrict__ part, int S, double count,
                                                                  const float *__restrict__ gamma,
                                                                  const float *__restrict__ mean,
                                                                  const float *__restrict__ rstd,
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_coef_kernel(const double *_
     }
 }
 
-int launch_bn_bwd_coef(const double *part, int slots, const float *gamma, const float *mean, const float *rstd,
+int launch_bn_bwd_coef(const float *part, int slots, const float *gamma, const float *mean, const float *rstd,
                        double count, float *coef, float *dgamma, float *dbeta, int C, hipStream_t s) {
     hipLaunchKernelGGL(bn_bwd_coef_kernel, dim3(C), dim3(kBnThreads), 0, s, part, slots, count, gamma, mean, rstd, coef,
                        dgamma, dbeta);

@@ -241,11 +241,11 @@ int launch_grad_x(const float *gy, const float *x, const float *w, float *gx, co
                   hipStream_t s, const float *gadd = nullptr);
 size_t grad_w_workspace_bytes(const ConvDims &d);
 // The sums of the backward of the BatchNorm behind a layer, as the consumer's input-gradient kernel left them
-// ((C, slots, 2) doubles: sum dz, sum dz * xhat), with what turns them into the four coefficients per channel.
+// ((C, slots, 2) floats -- a wave's fp32 totals: sum dz, sum dz * xhat), with what turns them into the four coefficients per channel.
 // A weight-gradient kernel that is given these instead of ready coefficients adds the slots itself (every
 // workgroup its own channels, all in the same order) and writes dgamma / dbeta on the way.  part == null: not used.
 struct BnSums {
-    const double *part;
+    const float *part;
     int slots;
     double count;            // N * Ho * Wo: values per channel of the BatchNorm
     const float *gamma, *mean, *rstd;
@@ -260,7 +260,7 @@ int grad_x_bn_slots(const ConvDims &d);
 int launch_grad_x_bn(const float *gy, const float *x, const float *w, float *gx, const ConvDims &d, hipStream_t s,
                      const float *gadd, const adder_bn_links &bn);
 bool grad_w_bn_supported(const ConvDims &d, const void *gy, const void *x, const void *bn_y, const void *bn_coef);
-int launch_bn_bwd_coef(const double *part, int slots, const float *gamma, const float *mean, const float *rstd,
+int launch_bn_bwd_coef(const float *part, int slots, const float *gamma, const float *mean, const float *rstd,
                        double count, float *coef, float *dgamma, float *dbeta, int C, hipStream_t s);
 
 // matrix-core weight gradient of the 3x3 / pad-1 layers (grad_w_mfma.hip); variant 0 = not applicable

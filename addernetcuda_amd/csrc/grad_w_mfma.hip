@@ -141,26 +141,24 @@ __device__ __forceinline__ void gy_commit_m_bn(const GyStageM<G> &sg, const GySt
 template <class G>
 __device__ __forceinline__ void bn_coef_from_sums(const BnSums &b, int co0, int Co, float4 *coef, bool write) {
     constexpr int GROUPS = G::NTHREADS / 32;
-    constexpr int CHUNK = G::KS == 3 ? 16 : 8;   // (the 1x1 kernels have few registers to spare)
+    constexpr int CHUNK = 16;
     const int sub = threadIdx.x & 31, grp = threadIdx.x >> 5;
     for (int cb = 0; cb < G::COB; cb += GROUPS) {
         const int c = cb + grp;
         if (G::COB % GROUPS == 0 || c < G::COB) {
             const int co = min(co0 + c, Co - 1);
             const float rs = b.rstd[co], gm = b.gamma[co], mu = b.mean[co];
-            const double2 *p = reinterpret_cast<const double2 *>(b.part) + (size_t)co * b.slots;
+            const float2 *p = reinterpret_cast<const float2 *>(b.part) + (size_t)co * b.slots;
             double s1 = 0.0, s2 = 0.0;
             for (int s0 = sub; s0 < b.slots; s0 += 32 * CHUNK) {   // CHUNK loads in flight, then added in slot order
-                double2 v[CHUNK];
+                float2 v[CHUNK];
+#pragma unroll
+                for (int j = 0; j < CHUNK; ++j) v[j] = p[min(s0 + 32 * j, b.slots - 1)];   // (unconditional: no waits between them)
 #pragma unroll
                 for (int j = 0; j < CHUNK; ++j) {
-                    const int s = s0 + 32 * j;
-                    v[j] = s < b.slots ? p[s] : make_double2(0.0, 0.0);
-                }
-#pragma unroll
-                for (int j = 0; j < CHUNK; ++j) {
-                    s1 += v[j].x;
-                    s2 += v[j].y;
+                    const bool in = s0 + 32 * j < b.slots;
+                    s1 += in ? (double)v[j].x : 0.0;
+                    s2 += in ? (double)v[j].y : 0.0;
                 }
             }
 #pragma unroll

@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const T *__restrict
 // T: storage type of gy, x, gx and gadd (float, or bf16_t for the reduced-storage mode).
 // FUSE: the statistics pass of the backward of the BatchNorm in front of the layer is done here (the in_* fields
 // of adder_bn_links): the result is masked with x > 0 (bn.in_relu) and its per-channel sums are left in
-// bn.in_part, (Ci, gridDim.x * POSW, 2) doubles.  Float storage, rows of whole float4 groups, no sampling.
+// bn.in_part, (Ci, gridDim.x * POSW, 2) floats.  Float storage, rows of whole float4 groups, no sampling.
 template <class C, bool VEC = true, bool SAT = true, bool SUB = false, class T = float, bool FUSE = false>
 __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *__restrict__ gy,
                                                                    const T *__restrict__ x,
@@ -456,7 +456,7 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
         // trip to memory per channel.
         if (lane < 2 * TM) {
             const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
-            if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = (double)total;
+            if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = total;
         }
         if (pos_ok && wi0 < W) {
 #pragma unroll
@@ -889,7 +889,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
         const float total = wave_sum_scatter<2 * TM>(sums, lane);
         if (lane < 2 * TM) {
             const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
-            if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = (double)total;
+            if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = total;
         }
         if (lane_ok && n < N && wi0 < W) {
 #pragma unroll

@@ -313,15 +313,16 @@ ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsign
  *                      (N, Co, Ho, Wo); the `gy` argument is then dz, not the gradient of y; out_gy (N, Co, Ho, Wo)
  *                      receives the gradient of y from the grad_W kernel.  The coefficients: exactly one of
  *                      out_coef = 4 floats per output channel {k, c2, mean, km1} from adder_bn_bwd_coef_f32, or
- *                      out_part = the sums as the consumer's call left them in its in_part (Co, out_slots, 2),
- *                      16-byte aligned, with out_gamma / out_mean / out_rstd (Co): every workgroup of the grad_W
- *                      kernel then adds the slots of its channels itself (the same fixed order as
- *                      adder_bn_bwd_coef_f32, so the same values) and out_dgamma / out_dbeta (Co) are written by
- *                      that kernel -- one launch fewer per layer.
+ *                      out_part = the sums as the consumer's call left them in its in_part (Co, out_slots, 2)
+ *                      floats, 16-byte aligned, with out_gamma / out_mean / out_rstd (Co): every workgroup of the grad_W
+ *                      kernel then adds the slots of its channels itself, in fp64 and in a fixed order (all of
+ *                      them arrive at the same values), and out_dgamma / out_dbeta (Co) are written by that kernel
+ *                      -- one launch fewer per layer.
  *     in_x, in_mean, in_rstd, in_part, in_slots, in_relu   the BatchNorm IN FRONT of the layer, whose output
  *                      (after the residual add and, if in_relu, the ReLU) is the layer's x: in_x = that
  *                      BatchNorm's input (N, Ci, H, W), its saved mean / rstd (Ci); in_part receives
- *                      (Ci, in_slots, 2) doubles, in_slots = adder_conv2d_bwd_bn_slots; gx receives dz.
+ *                      (Ci, in_slots, 2) floats (per-wave fp32 totals), in_slots = adder_conv2d_bwd_bn_slots; gx
+ *                      receives dz.
  *   adder_conv2d_bwd_bn_slots: partial-sum slots per channel for in_part; 0 = this layer has no such kernels
  *     (they exist for 3x3 / pad 1 / stride 1 or 2 layers whose rows are whole groups of four floats, and for 1x1 /
  *     stride 1 layers with at least 64 input and output channels whose planes are whole groups of four floats).
@@ -332,7 +333,7 @@ ADDER_API int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsign
  *     16-byte aligned.
  *   adder_conv2d_grad_w_staged_bn_f32: adder_conv2d_grad_w_staged_f32 with the out_* half of the links
  *     (out_gy nullable).
- *   adder_bn_bwd_coef_f32: sums the slots of `part` (C, slots, 2) in a fixed order and writes coef (C, 4),
+ *   adder_bn_bwd_coef_f32: sums the slots of `part` (C, slots, 2) floats in fp64, in a fixed order, and writes coef (C, 4),
  *     dgamma and dbeta (C); count = N * H * W of the BatchNorm.
  * ---------------------------------------------------------------------- */
 typedef struct adder_bn_links {
@@ -342,7 +343,7 @@ typedef struct adder_bn_links {
     const float *in_x;
     const float *in_mean;
     const float *in_rstd;
-    double *in_part;
+    float *in_part;
     int in_slots;
     int in_relu;
     /* optional, both or neither, and only for a BatchNorm whose output reached the layer through nothing but the
@@ -358,7 +359,7 @@ typedef struct adder_bn_links {
     const float *side_gy;
     const float *side_w;
     /* the alternative to out_coef (see above); all of them or none */
-    const double *out_part;
+    const float *out_part;
     int out_slots;
     const float *out_gamma;
     const float *out_mean;
@@ -377,7 +378,7 @@ ADDER_API int adder_conv2d_grad_w_staged_bn_f32(const float *gy, const float *x,
                          void *ws, size_t ws_bytes,
                          int N, int Ci, int H, int W, int Co, int kh, int kw,
                          int stride, int pad, const adder_bn_links *links, adder_grad_w_stage *stage, void *stream);
-ADDER_API int adder_bn_bwd_coef_f32(const double *part, int slots, const float *gamma, const float *save_mean,
+ADDER_API int adder_bn_bwd_coef_f32(const float *part, int slots, const float *gamma, const float *save_mean,
                                     const float *save_rstd, double count, float *coef, float *dgamma, float *dbeta,
                                     int C, void *stream);
 

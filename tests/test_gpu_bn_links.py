@@ -110,6 +110,7 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, fro
     # Q's coefficients from one slot of partial sums (what B's consumer would have left)
     xhat_q = (y32.double() - b(mean_q32.double())) * b(rstd_q32.double())
     part_q = torch.stack([dzq.double().sum((0, 2, 3)), (dzq.double() * xhat_q).sum((0, 2, 3))], 1).view(Co, 1, 2)
+    part_q = part_q.float()                                         # (the slots hold float32 totals)
     part_qg = d(part_q)
     coef = torch.empty(Co, 4, device=gpu)
     dgq, dbq = torch.empty(Co, device=gpu), torch.empty(Co, device=gpu)
@@ -118,7 +119,7 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, fro
     assert_close(dgq, dgamma_q, "dgamma of Q", rtol=1e-5, atol=1e-3)
     assert_close(dbq, dbeta_q, "dbeta of Q", rtol=1e-5, atol=1e-3)
 
-    part = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float64, device=gpu)
+    part = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float32, device=gpu)
     gy_out = torch.full_like(dzqg, float("nan"))
     gamma_pg, beta_pg = (d(gamma_p), d(beta_p)) if from_x else (None, None)
     links = BnLinks(ptr(y32g), ptr(coef), ptr(gy_out), ptr(xpg), ptr(mean_pg), ptr(rstd_pg), ptr(part), slots, 1,
@@ -132,7 +133,7 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, fro
     # grad_X inherits the rounding of gy = k * dz + ... (a float32 value of size ~1), which the plain backward gets exact
     assert_close(gxg, dz, "dz", rtol=2e-5, atol=2e-4)
     assert_close(gwg, gw_scaled, "grad_W (scaled)", rtol=2e-5, atol=2e-4)
-    got_part = part.sum(1)
+    got_part = part.double().sum(1)
     assert torch.isfinite(part).all()
     scale = max(1.0, float(want_part.abs().max()))
     assert_close(got_part / scale, want_part / scale, "sums of dz, dz * xhat", rtol=1e-5, atol=1e-5)
@@ -171,11 +172,11 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, fro
         else:
             g = torch.Generator().manual_seed(S)
             pieces = torch.randn(Co, S, 2, generator=g, dtype=torch.float64)
-            pieces[:, -1] += part_q.view(Co, 2) - pieces.sum(1)
-            part_s = d(pieces)
+            pieces[:, -1] += part_q.view(Co, 2).double() - pieces.sum(1)
+            part_s = d(pieces.float())
         dg3, db3 = torch.full((Co,), float("nan"), device=gpu), torch.full((Co,), float("nan"), device=gpu)
         gy_out3, gw3, gx3 = torch.full_like(dzqg, float("nan")), torch.empty_like(wg), torch.empty_like(xg)
-        part3 = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float64, device=gpu)
+        part3 = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float32, device=gpu)
         links3 = BnLinks(ptr(y32g), None, ptr(gy_out3), ptr(xpg), ptr(mean_pg), ptr(rstd_pg), ptr(part3), slots, 1,
                          ptr(gamma_pg), ptr(beta_pg), None, None, ptr(part_s), S, ptr(gamma_qg), ptr(mean_qg),
                          ptr(rstd_qg), ptr(dg3), ptr(db3))
@@ -225,7 +226,7 @@ def test_each_half_of_the_links_alone(case, gpu):
           "adder_conv2d_bwd_f32")
     # in-links only: same gy; the result is the plain one masked, the weight gradient is unchanged
     mean, rstd = d(torch.randn(Ci) - 90), d(torch.rand(Ci) * 0.05 + 0.02)
-    part = torch.empty((Ci, slots, 2), dtype=torch.float64, device=gpu)
+    part = torch.empty((Ci, slots, 2), dtype=torch.float32, device=gpu)
     links = BnLinks(None, None, None, ptr(xpg), ptr(mean), ptr(rstd), ptr(part), slots, 1)
     gx1, gw1 = torch.empty_like(xg), torch.empty_like(wg)
     check(lib.adder_conv2d_bwd_bn_f32(ptr(gyg), ptr(xg), ptr(wg), None, ptr(gx1), ptr(gw1), 0.2, ptr(ws), nbytes, *dims,
@@ -236,7 +237,7 @@ def test_each_half_of_the_links_alone(case, gpu):
     xhat = (xpg.double() - mean.double()[None, :, None, None]) * rstd.double()[None, :, None, None]
     want = torch.stack([gx1.double().sum((0, 2, 3)), (gx1.double() * xhat).sum((0, 2, 3))], 1)
     scale = max(1.0, float(want.abs().max()))
-    assert_close(part.sum(1) / scale, want / scale, "partial sums", rtol=1e-5, atol=1e-5)
+    assert_close(part.double().sum(1) / scale, want / scale, "partial sums", rtol=1e-5, atol=1e-5)
     # without the ReLU gate the result is the plain one
     links.in_relu = 0
     check(lib.adder_conv2d_bwd_bn_f32(ptr(gyg), ptr(xg), ptr(wg), None, ptr(gx1), None, 0.0, None, 0, *dims,
@@ -262,7 +263,7 @@ def test_refusals(gpu):
     assert rc == -7
     dims3, _, _ = conv_dims((2, 16, 8, 8), (16, 16, 3, 3), 1, 1)
     slots3 = bwd_bn_slots(dims3)
-    part = torch.empty(16 * slots3 * 2, dtype=torch.float64, device=gpu)
+    part = torch.empty(16 * slots3 * 2, dtype=torch.float32, device=gpu)
     links = BnLinks(None, None, None, ptr(t), ptr(t), ptr(t), ptr(part), slots3, 1, ptr(t), None)   # weight, no bias
     rc = lib.adder_conv2d_bwd_bn_f32(ptr(t), ptr(t), ptr(t), None, ptr(t), None, 0.0, None, 0, *dims3, ctypes.byref(links),
                                      stream_ptr(gpu))

@@ -122,7 +122,7 @@ def test_full_batch_links(layer, from_x, gpu):
     st = stream_ptr(gpu)
     ws, nbytes = conv2d_bwd_workspace(dims, gpu)
 
-    part = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float64, device=gpu)
+    part = torch.full((Ci, slots, 2), float("nan"), dtype=torch.float32, device=gpu)
     gy_out = torch.empty_like(dz)
     links = BnLinks(ptr(y), ptr(coef), ptr(gy_out), ptr(bn_in), ptr(mean), ptr(rstd), ptr(part), slots, 1,
                     ptr(gamma) if from_x else None, ptr(beta) if from_x else None)
@@ -145,4 +145,4 @@ def test_full_batch_links(layer, from_x, gpu):
     want = torch.stack([gx.double().sum((0, 2, 3)), (gx.double() * xhat).sum((0, 2, 3))], 1)
     assert torch.isfinite(part).all()
     scale = max(1.0, float(want.abs().max()))
-    assert_close(part.sum(1) / scale, want / scale, f"sums of dz, dz * xhat {layer}", rtol=1e-5, atol=1e-5)
+    assert_close(part.double().sum(1) / scale, want / scale, f"sums of dz, dz * xhat {layer}", rtol=1e-5, atol=1e-5)

@@ -91,7 +91,7 @@ def test_side_input_gradient_inside_the_strided_kernel(case, with_add, gpu):
     assert slots > 0
     st = stream_ptr(gpu)
     gxd, gxa, gxb = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
-    pa = torch.empty(Ci, slots, 2, dtype=torch.float64, device=gpu)
+    pa = torch.empty(Ci, slots, 2, dtype=torch.float32, device=gpu)
     pb = torch.full_like(pa, float("nan"))
     la = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(pa), slots, 1)
     lb = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(pb), slots, 1, None, None, ptr(gyd), ptr(ws))
@@ -103,8 +103,8 @@ def test_side_input_gradient_inside_the_strided_kernel(case, with_add, gpu):
                                       ctypes.byref(lb), st), "side")
     torch.cuda.synchronize()
     assert_close(gxb, gxa, f"dz {case}", rtol=1e-5, atol=1e-4)
-    scale = max(1.0, float(pa.sum(1).abs().max()))
-    assert_close(pb.sum(1) / scale, pa.sum(1) / scale, f"sums {case}", rtol=1e-6, atol=1e-6)
+    scale = max(1.0, float(pa.double().sum(1).abs().max()))
+    assert_close(pb.double().sum(1) / scale, pa.double().sum(1) / scale, f"sums {case}", rtol=1e-6, atol=1e-6)
     # refusals: one of the two pointers, no in-links, a stride-1 layer
     lc = BnLinks(None, None, None, ptr(bn_in), ptr(mean), ptr(rstd), ptr(pb), slots, 1, None, None, ptr(gyd), None)
     assert lib.adder_conv2d_bwd_bn_f32(ptr(gy), ptr(x), ptr(w), None, ptr(gxb), None, 0.0, None, 0, *dims,
