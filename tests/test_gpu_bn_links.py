@@ -165,8 +165,9 @@ def test_fused_backward_matches_the_unfused_chain_in_float64(case, with_add, fro
     assert torch.equal(gx2, gxg)
 
     # the same with Q's sums handed to the grad_W kernel itself (out_part) instead of ready coefficients: one slot
-    # gives the very same bits; many slots (unrolled part of the slot loop and its tail) the same values
-    for S in (1, 1100):
+    # gives the very same bits; many slots the same values (an even count is read two slots at a time: less than one
+    # load per lane, several rounds of loads with a tail; an odd count slot by slot)
+    for S in (1, 6, 1100, 333):
         if S == 1:
             part_s = part_qg
         else:
