@@ -60,6 +60,9 @@ _SIGNATURES = {
     "adder_conv2d_bwd_bn_f32": (_i, [_p, _p, _p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p, _p]),
     "adder_conv2d_grad_w_staged_bn_f32": (_i, [_p, _p, _p, _p, _f, _p, _sz] + [_i] * 9 + [_p, _p, _p]),
     "adder_bn_bwd_coef_f32": (_i, [_p, _i, _p, _p, _p, ctypes.c_double, _p, _p, _p, _i, _p]),
+    "adder_head_supported": (_i, [_i, _i, _i, _i]),
+    "adder_head_fwd_f32": (_i, [_p] * 12 + [_f, _f, _i, _i, _i, _i, _p]),
+    "adder_head_bwd_f32": (_i, [_p] * 12 + [_i, _i, _i, _i, _p]),
 }
 for _name, (_res, _args) in _SIGNATURES.items():
     _fn = getattr(lib, _name)

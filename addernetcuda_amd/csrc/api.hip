@@ -622,4 +622,48 @@ int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsigned int *re
                              N, C, HW, ws, static_cast<hipStream_t>(stream));
 }
 
+int adder_head_supported(int N, int C, int HW, int classes) {
+    return (N > 0 && C > 0 && HW > 0 && classes > 0 && head_supported(N, C, HW, classes)) ? 1 : 0;
+}
+
+int adder_head_fwd_f32(const float *x, const float *w, const float *gamma, const float *beta, float *pooled, float *z,
+                       float *y, float *save_mean, float *save_rstd, float *running_mean, float *running_var,
+                       long long *num_batches_tracked, float momentum, float eps, int N, int C, int HW, int classes,
+                       void *stream) {
+    if (!x || !w || !gamma || !beta || !pooled || !z || !y || !save_mean || !save_rstd) return ADDER_ERR_NULL_POINTER;
+    if ((running_mean == nullptr) != (running_var == nullptr)) return ADDER_ERR_NULL_POINTER;
+    if (N <= 0 || C <= 0 || HW <= 0 || classes <= 0 || !(eps >= 0.f)) return ADDER_ERR_BAD_SHAPE;
+    if ((long)N * C * HW > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    if (!head_supported(N, C, HW, classes)) return ADDER_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(pooled)) & 15) return ADDER_ERR_UNSUPPORTED;
+    const size_t nx = sizeof(float) * (size_t)N * C * HW, nw = sizeof(float) * (size_t)classes * C,
+                 np = sizeof(float) * (size_t)N * C, nz = sizeof(float) * (size_t)N * classes,
+                 nj = sizeof(float) * (size_t)classes;
+    const Span outs[] = {{pooled, np}, {z, nz}, {y, nz}, {save_mean, nj}, {save_rstd, nj}, {running_mean, nj},
+                         {running_var, nj}, {num_batches_tracked, sizeof(long long)}};
+    const Span ins[] = {{x, nx}, {w, nw}, {gamma, nj}, {beta, nj}};
+    if (any_alias(outs, ins)) return ADDER_ERR_ALIAS;
+    return launch_head_fwd(x, w, gamma, beta, pooled, z, y, save_mean, save_rstd, running_mean, running_var,
+                           num_batches_tracked, momentum, eps, N, C, HW, classes, static_cast<hipStream_t>(stream));
+}
+
+int adder_head_bwd_f32(const float *dy, const float *z, const float *pooled, const float *w, const float *gamma,
+                       const float *save_mean, const float *save_rstd, float *dz, float *dx, float *dw, float *dgamma,
+                       float *dbeta, int N, int C, int HW, int classes, void *stream) {
+    if (!dy || !z || !pooled || !w || !gamma || !save_mean || !save_rstd || !dz || !dw || !dgamma || !dbeta)
+        return ADDER_ERR_NULL_POINTER;
+    if (N <= 0 || C <= 0 || HW <= 0 || classes <= 0) return ADDER_ERR_BAD_SHAPE;
+    if ((long)N * C * HW > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    if (!head_supported(N, C, HW, classes)) return ADDER_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(dx) | reinterpret_cast<uintptr_t>(pooled)) & 15) return ADDER_ERR_UNSUPPORTED;
+    const size_t nx = sizeof(float) * (size_t)N * C * HW, nw = sizeof(float) * (size_t)classes * C,
+                 np = sizeof(float) * (size_t)N * C, nz = sizeof(float) * (size_t)N * classes,
+                 nj = sizeof(float) * (size_t)classes;
+    const Span outs[] = {{dz, nz}, {dx, nx}, {dw, nw}, {dgamma, nj}, {dbeta, nj}};
+    const Span ins[] = {{dy, nz}, {z, nz}, {pooled, np}, {w, nw}, {gamma, nj}, {save_mean, nj}, {save_rstd, nj}};
+    if (any_alias(outs, ins)) return ADDER_ERR_ALIAS;
+    return launch_head_bwd(dy, z, pooled, w, gamma, save_mean, save_rstd, dz, dx, dw, dgamma, dbeta, N, C, HW, classes,
+                           static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

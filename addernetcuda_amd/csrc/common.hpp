@@ -293,6 +293,15 @@ int launch_bn_act_bwd(const float *dy, const float *y, const unsigned *mask, con
                       const float *mean, const float *rstd, float *dx, float *dres, float *dgamma, float *dbeta,
                       int relu, int N, int C, int HW, void *ws, hipStream_t s);
 
+// average pool over the whole map -> matrix product -> BatchNorm of the ResNet classifier head (head.hip)
+bool head_supported(int N, int C, int HW, int J);
+int launch_head_fwd(const float *x, const float *w, const float *gamma, const float *beta, float *pooled, float *z,
+                    float *y, float *mean, float *rstd, float *running_mean, float *running_var, long long *num_batches,
+                    float momentum, float eps, int N, int C, int HW, int J, hipStream_t s);
+int launch_head_bwd(const float *dy, const float *z, const float *pooled, const float *w, const float *gamma,
+                    const float *mean, const float *rstd, float *dz, float *dx, float *dw, float *dgamma, float *dbeta,
+                    int N, int C, int HW, int J, hipStream_t s);
+
 size_t norm_scale_workspace_bytes(long n);
 int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);
 static constexpr int kNormBatchMax = ADDER_NORM_BATCH_MAX;

@@ -27,6 +27,7 @@
  *   [optional]  grad_W in two stages (all layers finished together after the backward pass)
  *   [optional]  BatchNorm + residual + ReLU kernels (adder_bn_act_*)
  *   [optional]  BatchNorm backward passes folded into the adder backward kernels (adder_bn_links, *_bn_*)
+ *   [optional]  the classifier head of the ResNets: average pool, matrix product, BatchNorm (adder_head_*)
  */
 #ifndef ADDERNET_HIP_H
 #define ADDERNET_HIP_H
@@ -381,6 +382,32 @@ ADDER_API int adder_conv2d_grad_w_staged_bn_f32(const float *gy, const float *x,
 ADDER_API int adder_bn_bwd_coef_f32(const float *part, int slots, const float *gamma, const float *save_mean,
                                     const float *save_rstd, double count, float *coef, float *dgamma, float *dbeta,
                                     int C, void *stream);
+
+/* ------------------------------------------------------------------------
+ * [optional] The classifier head behind the last adder block (resnet20.py:55-57, 89-93 of the reference:
+ * AvgPool2d over the whole map, a 1x1 convolution without bias, BatchNorm2d in training mode), two launches
+ * forward and two backward where the framework's own operators take eight of 5-10 us each on N x classes values.
+ *   x (N, C, HW) -> pooled (N, C) = plane means -> z (N, classes) = pooled * w^T, w (classes, C)
+ *     -> y (N, classes) = gamma * (z - mean) * rstd + beta, batch statistics per class (biased variance; the running
+ *     statistics, nullable, receive the unbiased one, as torch.nn.BatchNorm2d does).
+ *   adder_head_supported: 1 where the kernels apply -- N >= 2, a plane of 4, 8, ... 256 positions, C a divisor of
+ *     256 with N * C a multiple of four, at most 32 classes, and a batch whose pooled matrix fits the LDS (with
+ *     P = 16 or 32 padded classes: N * (C + P) + max(3 * classes * (N | 1), 512 * P) floats within 144 KiB) -- else
+ *     0, and the calls return ADDER_ERR_UNSUPPORTED.  x, dx and pooled 16-byte aligned.
+ *   adder_head_fwd_f32: pooled, z, save_mean, save_rstd are kept for the backward.
+ *   adder_head_bwd_f32: dy (N, classes) -> dgamma, dbeta, dz (N, classes: the gradient of z, scratch for the caller),
+ *     dw (classes, C) = dz^T * pooled, dx (N, C, HW; nullable) = (dz * w) / HW on every position.
+ * Every sum has a fixed order: results do not change from run to run.
+ * ---------------------------------------------------------------------- */
+ADDER_API int adder_head_supported(int N, int C, int HW, int classes);
+ADDER_API int adder_head_fwd_f32(const float *x, const float *w, const float *gamma, const float *beta,
+                                 float *pooled, float *z, float *y, float *save_mean, float *save_rstd,
+                                 float *running_mean, float *running_var, long long *num_batches_tracked,
+                                 float momentum, float eps, int N, int C, int HW, int classes, void *stream);
+ADDER_API int adder_head_bwd_f32(const float *dy, const float *z, const float *pooled, const float *w,
+                                 const float *gamma, const float *save_mean, const float *save_rstd,
+                                 float *dz, float *dx, float *dw, float *dgamma, float *dbeta,
+                                 int N, int C, int HW, int classes, void *stream);
 
 #ifdef __cplusplus
 }
