@@ -16,7 +16,7 @@ namespace adder {
 
 static constexpr int kHeadThreads = 256;
 static constexpr int kHeadMaxClasses = 32;    // two per wave of the one-workgroup kernels
-static constexpr int kHeadMaxChannels = 256;  // = the workgroup: a thread per channel in the backward
+static constexpr int kHeadMaxChannels = 256;  // channels divide the 256-thread workgroups of the per-image kernels
 
 // G lanes (a power of two <= 64, aligned) share a plane: their sum in the first of them
 template <int G>
