@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libaddernet_hip.so")
-SOURCES = ["api.hip", "fwd.hip", "grad_x.hip", "grad_w.hip", "grad_w_mfma.hip", "conv1x1.hip", "col.hip", "bn_act.hip", "head.hip"]
+SOURCES = ["api.hip", "fwd.hip", "grad_x.hip", "grad_w.hip", "grad_w_mfma.hip", "conv1x1.hip", "col.hip", "bn_act.hip", "head.hip", "sgd.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

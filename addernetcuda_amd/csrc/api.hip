@@ -622,6 +622,36 @@ int adder_bn_act_bwd_f32(const float *dy, const float *y, const unsigned int *re
                              N, C, HW, ws, static_cast<hipStream_t>(stream));
 }
 
+int adder_sgd_momentum_step_f32(int count, float *const *params, const float *const *grads, float *const *momentum_bufs,
+                                const long *n, const float *lr_device, float lr, float momentum, float weight_decay,
+                                void *stream) {
+    if (!params || !grads || !momentum_bufs || !n) return ADDER_ERR_NULL_POINTER;
+    if (count <= 0 || count > ADDER_SGD_BATCH_MAX) return ADDER_ERR_BAD_SHAPE;
+    if (!(momentum >= 0.f) || !(weight_decay >= 0.f) || !(lr_device || lr >= 0.f)) return ADDER_ERR_BAD_SHAPE;
+    long blocks = 0;
+    for (int t = 0; t < count; ++t) {
+        if (!params[t] || !grads[t] || !momentum_bufs[t]) return ADDER_ERR_NULL_POINTER;
+        if (n[t] <= 0) return ADDER_ERR_BAD_SHAPE;
+        if (n[t] > kMaxElems) return ADDER_ERR_TOO_LARGE;
+        blocks += (n[t] + 1023) / 1024;
+    }
+    if (blocks > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    for (int t = 0; t < count; ++t) {
+        const size_t bytes = sizeof(float) * (size_t)n[t];
+        if (overlaps(params[t], bytes, grads[t], bytes) || overlaps(params[t], bytes, momentum_bufs[t], bytes) ||
+            overlaps(momentum_bufs[t], bytes, grads[t], bytes))
+            return ADDER_ERR_ALIAS;
+        for (int u = t + 1; u < count; ++u) {
+            const size_t other = sizeof(float) * (size_t)n[u];
+            if (overlaps(params[t], bytes, params[u], other) || overlaps(momentum_bufs[t], bytes, momentum_bufs[u], other) ||
+                overlaps(params[t], bytes, momentum_bufs[u], other) || overlaps(momentum_bufs[t], bytes, params[u], other))
+                return ADDER_ERR_ALIAS;
+        }
+    }
+    return launch_sgd_momentum(count, params, grads, momentum_bufs, n, lr_device, lr, momentum, weight_decay,
+                               static_cast<hipStream_t>(stream));
+}
+
 int adder_head_supported(int N, int C, int HW, int classes) {
     return (N > 0 && C > 0 && HW > 0 && classes > 0 && head_supported(N, C, HW, classes)) ? 1 : 0;
 }

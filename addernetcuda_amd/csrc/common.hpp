@@ -305,6 +305,9 @@ int launch_head_bwd(const float *dy, const float *z, const float *pooled, const 
 size_t norm_scale_workspace_bytes(long n);
 int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);
 static constexpr int kNormBatchMax = ADDER_NORM_BATCH_MAX;
+static constexpr int kSgdBatchMax = ADDER_SGD_BATCH_MAX;
+int launch_sgd_momentum(int count, float *const *p, const float *const *g, float *const *buf, const long *n,
+                        const float *lr_ptr, float lr, float momentum, float weight_decay, hipStream_t s);
 static constexpr int kGwFinishMax = ADDER_GRAD_W_FINISH_MAX;
 int launch_grad_w_staged(const float *gy, const float *x, const float *w, float *gw, float eta, void *ws,
                          size_t ws_bytes, const ConvDims &d, adder_grad_w_stage *stage, hipStream_t s,

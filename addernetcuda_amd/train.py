@@ -190,7 +190,8 @@ def run(args):
         net.load_state_dict(torch.load(args.resume, map_location=dev, weights_only=True))
     # the learning rate lives on the device so that the captured step sees each epoch's value
     lr_now = torch.tensor(float(args.lr), device=dev)
-    opt = torch.optim.SGD(net.parameters(), lr=lr_now, momentum=0.9, weight_decay=5e-4, fused=True)
+    from addernetcuda_amd.optim import SGD   # torch.optim.SGD's rule and state, all parameters in one launch
+    opt = SGD(net.parameters(), lr=lr_now, momentum=0.9, weight_decay=5e-4)
     if args.eval_only:   # the reference's test.py: load a checkpoint, one pass over the test split
         test_loss, acc = evaluate(net, *data["test"], args.test_batch_size, args.bf16_activations)
         print(f"test loss {test_loss:.4f}  accuracy {acc:.4f}", flush=True)

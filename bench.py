@@ -321,8 +321,13 @@ def build_training(dev, seed=0, which="resnet20", fused=True):
         from addernetcuda_amd import models
         model = getattr(models, which)(num_classes=classes, eta=ETA, fused=fused)
     model = model.to(dev)
-    # fused=True: the same update as the default implementation, in one kernel per parameter group
-    opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4, fused=True)
+    # torch.optim.SGD's update rule and state (main.py:67) with all parameters in one launch; with the reference's
+    # stock modules (fused=False) the framework's own fused update
+    if fused:
+        from addernetcuda_amd.optim import SGD
+        opt = SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4)
+    else:
+        opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=5e-4, fused=True)
     g = torch.Generator(device=dev).manual_seed(seed + 1)
     x = torch.randn(batch, 3, size, size, device=dev, generator=g)
     y = torch.randint(0, classes, (batch,), device=dev, generator=g)

@@ -28,6 +28,7 @@
  *   [optional]  BatchNorm + residual + ReLU kernels (adder_bn_act_*)
  *   [optional]  BatchNorm backward passes folded into the adder backward kernels (adder_bn_links, *_bn_*)
  *   [optional]  the classifier head of the ResNets: average pool, matrix product, BatchNorm (adder_head_*)
+ *   [optional]  the momentum-SGD update of all parameters in one launch (adder_sgd_momentum_step_f32)
  */
 #ifndef ADDERNET_HIP_H
 #define ADDERNET_HIP_H
@@ -408,6 +409,21 @@ ADDER_API int adder_head_bwd_f32(const float *dy, const float *z, const float *p
                                  const float *gamma, const float *save_mean, const float *save_rstd,
                                  float *dz, float *dx, float *dw, float *dgamma, float *dbeta,
                                  int N, int C, int HW, int classes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * [optional] The parameter update of the training script (main.py:67 of the reference: torch.optim.SGD with
+ * momentum and weight decay, no dampening, no Nesterov) for `count` <= ADDER_SGD_BATCH_MAX tensors in one launch:
+ *     g' = grads[t] + weight_decay * params[t];  momentum_bufs[t] = momentum * momentum_bufs[t] + g';
+ *     params[t] -= lr * momentum_bufs[t]
+ * (a zero-filled buffer gives the framework's first step, buf = g').  params, grads, momentum_bufs and n are host
+ * arrays of `count` device pointers / element counts.  lr_device (nullable): the learning rate as one float in
+ * device memory, read by the kernel -- for callers that capture the step in a HIP graph and change the rate
+ * between replays; `lr` is used when it is NULL.
+ * ---------------------------------------------------------------------- */
+#define ADDER_SGD_BATCH_MAX 96
+ADDER_API int adder_sgd_momentum_step_f32(int count, float *const *params, const float *const *grads,
+                                          float *const *momentum_bufs, const long *n, const float *lr_device,
+                                          float lr, float momentum, float weight_decay, void *stream);
 
 #ifdef __cplusplus
 }
