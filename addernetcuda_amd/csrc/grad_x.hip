@@ -26,6 +26,12 @@
 
 namespace adder {
 
+// Partial-sum slots a workgroup of the BatchNorm-linked kernels leaves per channel: one per position wave -- except
+// that two position waves add theirs through LDS first (the consumer of the sums, the weight-gradient kernel of the
+// layer in front, reads all slots of its channels in every one of its workgroups: half the slots, half that prologue).
+template <class C>
+constexpr int bn_slots_per_wg() { return C::POSW == 2 ? 1 : C::POSW; }
+
 // ---------------------------------------------------------------------------
 // Generic kernel: any kernel size / stride / padding.
 // ---------------------------------------------------------------------------
@@ -98,7 +104,7 @@ __global__ __launch_bounds__(256) void grad_x_generic_kernel(const T *__restrict
 // T: storage type of gy, x, gx and gadd (float, or bf16_t for the reduced-storage mode).
 // FUSE: the statistics pass of the backward of the BatchNorm in front of the layer is done here (the in_* fields
 // of adder_bn_links): the result is masked with x > 0 (bn.in_relu) and its per-channel sums are left in
-// bn.in_part, (Ci, gridDim.x * POSW, 2) floats.  Float storage, rows of whole float4 groups, no sampling.
+// bn.in_part, (Ci, gridDim.x * bn_slots_per_wg, 2) floats.  Float storage, rows of whole float4 groups, no sampling.
 template <class C, bool VEC = true, bool SAT = true, bool SUB = false, class T = float, bool FUSE = false>
 __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *__restrict__ gy,
                                                                    const T *__restrict__ x,
@@ -410,7 +416,9 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
         // With one round of workgroups on the chip nothing overlaps this epilogue, so it is kept short: one mask bit
         // per position decides what counts (inside the tensor, an own channel, the ReLU passed); per term one
         // select, one add, one subtract and one multiply-add; the scale of xhat is applied to the wave's sum.
-        const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+        constexpr bool MERGE = C::POSW == 2;   // see bn_slots_per_wg
+        const int slots = gridDim.x * bn_slots_per_wg<C>(), slot = MERGE ? (int)blockIdx.x : (int)blockIdx.x * C::POSW + pw;
+        __shared__ float pw_sums[MERGE ? C::COW * 2 * TM : 1];
         unsigned keep = 0;
 #pragma unroll
         for (int t = 0; t < TN; ++t) keep |= (pos_ok && wi0 + t < W ? 1u : 0u) << t;
@@ -454,10 +462,11 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
         // Only stores from here on, and nothing that would have to be waited for between them: loads and stores
         // share one counter, in order, so a wait for any later load is a wait for every store before it -- a round
         // trip to memory per channel.
-        if (lane < 2 * TM) {
+        if (!MERGE && lane < 2 * TM) {
             const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
             if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = total;
         }
+        if (MERGE && pw == 1 && lane < 2 * TM) pw_sums[cw * 2 * TM + lane] = total;
         if (pos_ok && wi0 < W) {
 #pragma unroll
             for (int m = 0; m < TM; ++m) {
@@ -465,6 +474,14 @@ __global__ __launch_bounds__(C::NTHREADS, 4) void grad_x_3x3s1_kernel(const T *_
                 float *dst = reinterpret_cast<float *>(gx) + pofs + m * (H * W);
                 if constexpr (TN == 4) stf4(dst, make_float4(tot[m][0], tot[m][1], tot[m][2], tot[m][3]));
                 else stf2(dst, make_float2(tot[m][0], tot[m][1]));
+            }
+        }
+        if constexpr (MERGE) {   // the second position wave's sums, added behind the stores of dz
+            __syncthreads();
+            if (pw == 0 && lane < 2 * TM) {
+                const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
+                if (ci >= ci_first)
+                    bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = total + pw_sums[cw * 2 * TM + lane];
             }
         }
         return;
@@ -544,7 +561,7 @@ static int launch_grad_x_3x3s1_v(const T *gy, const T *x, const float *w, T *gx,
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::COW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    if (FUSE && (!bn.in_part || bn.in_slots != gxd * C::POSW)) return ADDER_ERR_BAD_SHAPE;
+    if (FUSE && (!bn.in_part || bn.in_slots != gxd * bn_slots_per_wg<C>())) return ADDER_ERR_BAD_SHAPE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     if (int rc = allow_dynamic_lds<&grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T, FUSE>>(LDS_BYTES)) return rc;
     hipLaunchKernelGGL((grad_x_3x3s1_kernel<C, VEC, SAT, SUB, T, FUSE>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS),
@@ -853,7 +870,9 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
     if constexpr (FUSE) {
         // dz = (gx + gadd) * [x > 0] and its per-channel sums, as in the stride-1 kernel (one mask bit per position,
         // every load before the first store)
-        const int slots = gridDim.x * C::POSW, slot = blockIdx.x * C::POSW + pw;
+        constexpr bool MERGE = C::POSW == 2;   // see bn_slots_per_wg
+        const int slots = gridDim.x * bn_slots_per_wg<C>(), slot = MERGE ? (int)blockIdx.x : (int)blockIdx.x * C::POSW + pw;
+        __shared__ float pw_sums[MERGE ? C::CIW * 2 * TM : 1];
         unsigned keep = 0;
 #pragma unroll
         for (int rp = 0; rp < 2; ++rp)
@@ -887,10 +906,11 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
             sums[2 * m + 1] = a2 * rs;
         }
         const float total = wave_sum_scatter<2 * TM>(sums, lane);
-        if (lane < 2 * TM) {
+        if (!MERGE && lane < 2 * TM) {
             const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
             if (ci >= ci_first) bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = total;
         }
+        if (MERGE && pw == 1 && lane < 2 * TM) pw_sums[cw * 2 * TM + lane] = total;
         if (lane_ok && n < N && wi0 < W) {
 #pragma unroll
             for (int m = 0; m < TM; ++m) {
@@ -899,6 +919,14 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
                 for (int rp = 0; rp < 2; ++rp)
                     if (hi0 + rp < H)
                         stf2(reinterpret_cast<float *>(gx) + pofs[rp] + m * (H * W), make_float2(tot[m][rp][0], tot[m][rp][1]));
+            }
+        }
+        if constexpr (MERGE) {   // the second position wave's sums, added behind the stores of dz
+            __syncthreads();
+            if (pw == 0 && lane < 2 * TM) {
+                const int j = wave_sum_scatter_index<2 * TM>(lane), ci = ci_base + (j >> 1);
+                if (ci >= ci_first)
+                    bn.in_part[((size_t)ci * slots + slot) * 2 + (j & 1)] = total + pw_sums[cw * 2 * TM + lane];
             }
         }
         return;
@@ -956,7 +984,7 @@ static int launch_grad_x_3x3s2_v(const T *gy, const T *x, const float *w, T *gx,
     const long gxd = (long)ceil_div(d.N, C::NIMG) * tilesH * tilesW;
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
-    if (FUSE && (!bn.in_part || bn.in_slots != gxd * C::POSW)) return ADDER_ERR_BAD_SHAPE;
+    if (FUSE && (!bn.in_part || bn.in_slots != gxd * bn_slots_per_wg<C>())) return ADDER_ERR_BAD_SHAPE;
     constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
     hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T, FUSE, PAIR>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS),
@@ -1101,7 +1129,7 @@ static int grad_x_bn_variant(const ConvDims &d) {
 
 template <class C>
 static int bn_slots_of(const ConvDims &d) {
-    return ceil_div(d.N, C::NIMG) * ceil_div(d.H, C::TH) * ceil_div(d.W, C::TW) * C::POSW;
+    return ceil_div(d.N, C::NIMG) * ceil_div(d.H, C::TH) * ceil_div(d.W, C::TW) * bn_slots_per_wg<C>();
 }
 
 // partial-sum slots per input channel that launch_grad_x_bn writes into bn.in_part; 0: no such kernel for the layer
