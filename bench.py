@@ -135,7 +135,7 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
     if slots > 0:
         bn_in = torch.randn(N, Ci, H, W, device=dev, generator=g) * 20 - 90
         mean, rstd = bn_in.mean((0, 2, 3)), 1.0 / bn_in.std((0, 2, 3))
-        part = torch.empty(Ci, slots, 2, dtype=torch.float64, device=dev)
+        part = torch.empty(Ci, slots, 2, dtype=torch.float32, device=dev)
         coef = torch.randn(Co, 4, device=dev, generator=g) * 0.01
         yo = torch.randn(N, Co, Ho, Wo, device=dev, generator=g) * 20 - 90
         gyo = torch.empty_like(gy)
@@ -151,7 +151,7 @@ def layer_ops(N, Ci, H, W, Co, k, stride, pad, dev):
                                                                       ptr(ws), need.value, *dims, ctypes.byref(lw), st),
                                          "grad_w_bn")
         # + the partial sums, + the BatchNorm's input where the kernel reads it (stride 2)
-        nbytes["grad_x_bn"] = nbytes["grad_x"] + 16 * Ci * slots + (nx if stride != 1 else 0)
+        nbytes["grad_x_bn"] = nbytes["grad_x"] + 8 * Ci * slots + (nx if stride != 1 else 0)
         nbytes["grad_w_bn"] = nbytes["grad_w"] + 2 * ny                 # + the layer's output, + the formed gradient
     return E, ops, keep, nbytes
 
