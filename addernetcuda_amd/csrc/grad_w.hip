@@ -361,7 +361,7 @@ bool grad_w_bn_supported(const ConvDims &d, const void *gy, const void *x, const
     const uintptr_t align = reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(x) |
                             reinterpret_cast<uintptr_t>(bn_y) | reinterpret_cast<uintptr_t>(bn_coef);
     const int v = p.mfma.variant;
-    const bool k3 = v >= 1 && v <= 5 && d.W % 4 == 0 && d.Wo % 4 == 0;
+    const bool k3 = ((v >= 1 && v <= 5) || v == 14) && d.W % 4 == 0 && d.Wo % 4 == 0;
     const bool k1 = (v == 6 || v == 7 || v == 10 || v == 12) && d.stride == 1 && (d.H * d.W) % 4 == 0;
     return p.variant == 2 && (k3 || k1) && (align & 15) == 0;
 }

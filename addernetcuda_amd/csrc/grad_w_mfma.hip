@@ -33,7 +33,10 @@ struct GwMfmaCfg {
     static constexpr int KS = KS_, KK = KS_ * KS_, PAD = KS_ / 2;   // 3x3 taps with pad 1, or a single tap
     static constexpr int COB = 16 * MT * MW;          // output channels per workgroup
     static constexpr int KB = 16 * NT * NW;           // k columns per workgroup
-    static constexpr int CIB = KB / KK;               // = input channels per workgroup
+    static constexpr int CIB = ceil_div(KB, KK);      // input channels per workgroup (staged)
+    // false: the k block ends inside an input channel -- usable only where one block holds all of K (a layer with
+    // very few input channels; the columns past K read a channel that does not exist, i.e. staged zeros)
+    static constexpr bool WHOLE = KB % KK == 0;
     static constexpr int NWAVES = MW * NW * PW;
     static constexpr int NTHREADS = 64 * NWAVES;
     // LPAD puts the interior columns on a 16-byte boundary (3 + one halo column, or no halo at all)
@@ -49,7 +52,6 @@ struct GwMfmaCfg {
     static constexpr int RED = 2 * (NWAVES / 2) * (REGS + MT) * 64;  // fp64 fold area, in floats
     static constexpr int LDS_FLOATS = (2 * BUF > RED) ? 2 * BUF : RED;
     static constexpr int LDS_BYTES = LDS_FLOATS * 4;
-    static_assert(KB % KK == 0, "a workgroup's k block must cover whole input channels");
     static_assert(TW % 4 == 0 && STEPS % PW == 0, "positions must split evenly over the position waves");
     static_assert((PW & (PW - 1)) == 0, "the fold is a binary tree over the position waves");
     static_assert(NTHREADS <= 1024 && LDS_BYTES <= 160 * 1024, "workgroup limits");
@@ -377,6 +379,10 @@ using GmW16   = GwMfmaCfg<1, 16, 16, 1, 1, 3, 1, 3, 4>;  // outputs 16 wide: one
 using GmW8    = GwMfmaCfg<1, 8, 8, 4, 1, 3, 1, 3, 4>;    // outputs 8 wide:  four images
 using GmW16S2 = GwMfmaCfg<2, 8, 16, 1, 1, 3, 1, 3, 4>;   // stride 2, outputs 16 wide: half an image
 using GmW8S2  = GwMfmaCfg<2, 8, 8, 2, 1, 3, 1, 3, 4>;    // stride 2, outputs 8 wide: two images
+// At most three input channels (the 3 -> 16 stem that precedes the adder layers: K = 27): two accumulator tiles cover
+// all of K, eight position waves.  Through the 144-column block above, four fifths of the matrix instructions of
+// such a layer multiply staged zeros: 28 us for 0.23 GFLOP.
+using GmW32K32 = GwMfmaCfg<1, 8, 32, 1, 1, 2, 1, 1, 8>;
 // 1x1, stride 1: a plain (Co x positions) x (positions x Ci) product; (H, W) planes walked as one row.
 // 64 output channels x 64 input channels per workgroup (two k waves with eight accumulator tiles each, times four
 // position waves), 128 positions per staged tile; every wave does eight steps of 8 MFMAs on 4 + 2 LDS reads per tile.
@@ -430,9 +436,10 @@ GradWMfmaPlan plan_grad_w_mfma(const ConvDims &d) {
     }
     const bool ok = d.kh == 3 && d.kw == 3 && d.pad == 1;
     if (!ok) return p;
-    if (d.stride == 1) p.variant = d.Wo > 16 ? 1 : (d.Wo > 8 ? 2 : 3);
+    if (d.stride == 1) p.variant = d.Wo > 16 ? (d.Ci * 9 <= GmW32K32::KB ? 14 : 1) : (d.Wo > 8 ? 2 : 3);
     else if (d.stride == 2) p.variant = d.Wo > 8 ? 4 : 5;
     switch (p.variant) {
+        case 14: plan_one<GmW32K32>(d, p); break;
         case 1: plan_one<GmW32>(d, p); break;
         case 2: plan_one<GmW16>(d, p); break;
         case 3: plan_one<GmW8>(d, p); break;
@@ -473,6 +480,7 @@ int launch_grad_w_mfma_bf16(const bf16_t *gy, const bf16_t *x, double *part, dou
         case 3: return launch_one<GmW8, bf16_t>(gy, x, part, sgpart, d, p, s);
         case 4: return launch_one<GmW16S2, bf16_t>(gy, x, part, sgpart, d, p, s);
         case 5: return launch_one<GmW8S2, bf16_t>(gy, x, part, sgpart, d, p, s);
+        case 14: return launch_one<GmW32K32, bf16_t>(gy, x, part, sgpart, d, p, s);
         default: return ADDER_ERR_UNSUPPORTED;
     }
 }
@@ -484,8 +492,11 @@ int launch_grad_w_mfma_bn(const float *gy, const float *x, double *part, double 
                           const GradWMfmaPlan &p, const float *bn_y, const float *bn_coef, float *gy_out, hipStream_t s,
                           const BnSums &sums) {
     const Subsample none{1, 0, 0, 0};
-    if (p.variant >= 1 && p.variant <= 5 && (d.W % 4 != 0 || d.Wo % 4 != 0)) return ADDER_ERR_UNSUPPORTED;
+    if (((p.variant >= 1 && p.variant <= 5) || p.variant == 14) && (d.W % 4 != 0 || d.Wo % 4 != 0))
+        return ADDER_ERR_UNSUPPORTED;
     switch (p.variant) {
+        case 14: return launch_one_v<GmW32K32, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef,
+                                                                            gy_out, sums);
         case 1: return launch_one_v<GmW32, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
         case 2: return launch_one_v<GmW16, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
         case 3: return launch_one_v<GmW8, true, false, float, true>(gy, x, part, sgpart, d, p, s, none, bn_y, bn_coef, gy_out, sums);
@@ -513,6 +524,7 @@ int launch_grad_w_mfma(const float *gy, const float *x, double *part, double *sg
         case 3: return launch_one<GmW8>(gy, x, part, sgpart, d, p, s);
         case 4: return launch_one<GmW16S2>(gy, x, part, sgpart, d, p, s);
         case 5: return launch_one<GmW8S2>(gy, x, part, sgpart, d, p, s);
+        case 14: return launch_one<GmW32K32>(gy, x, part, sgpart, d, p, s);
         case 6: return launch_one<Gm1x1>(gy, x, part, sgpart, mfma_one_row(d), p, s);
         case 7: return launch_one<Gm1x1s>(gy, x, part, sgpart, mfma_one_row(d), p, s);
         case 10: return launch_one<Gm1x1b>(gy, x, part, sgpart, mfma_one_row(d), p, s);

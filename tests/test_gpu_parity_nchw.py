@@ -36,6 +36,9 @@ TILED = [
     (3, 8, 20, 24, 8, 3, 1, 1),     # wide map, 20 rows: tiles of 4 rows of two images, odd image count
     (2, 16, 56, 56, 8, 3, 1, 1),    # ResNet-50's 56x56 maps (7 x 8 rows)
     (3, 8, 28, 28, 8, 3, 1, 1),     # ... and 28x28 (7 x 4 rows)
+    (5, 3, 32, 32, 16, 3, 1, 1),    # three input channels on a wide map (a stem's shape): the weight gradient's 32-column block
+    (3, 2, 24, 36, 20, 3, 1, 1),    # ... two channels, channel tail on Co
+    (2, 1, 32, 30, 8, 3, 1, 1),     # ... one channel, rows that are not whole float4 groups
     (2, 16, 32, 32, 32, 1, 2, 0),   # ResNet-20 1x1 stride-2 downsample
     (2, 32, 16, 16, 64, 1, 2, 0),   # second downsample
     (2, 8, 8, 8, 16, 1, 1, 0),      # 1x1 stride 1
