@@ -622,7 +622,8 @@ struct GradX3x3S2Cfg {
 // downsample branch of a residual block) is added in here: bn.side_gy is that layer's output gradient (shaped like
 // gy), bn.side_w its weights (Co, Ci).  Its one tap is the centre tap of the 3x3 window, so its gradient lands on
 // the even positions -- element (0, 0) of every lane's 2 x 2 block -- and takes the gy value of the block's own
-// output position, one float per lane and output channel, read from memory one channel ahead.
+// output position.  side_gy is staged in LDS chunk by chunk beside gy (a load from memory per lane and output
+// channel, asked for one channel ahead, has a few hundred cycles to arrive and needs a microsecond: +10 us).
 template <class C, bool VEC = true, bool SAT = true, class T = float, bool FUSE = false, bool PAIR = false>
 __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__restrict__ gy,
                                                                    const T *__restrict__ x,
@@ -687,30 +688,34 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
     const int lane_off = img * C::CC * C::PLANE + brow * C::PITCH + bcol * (TNW / 2);
     const int nchunks = ceil_div(Co, C::CC);
     const int hb = h0 / 2, wb = w0 / 2;
-    // PAIR: the side layer's gy at the lane's own output position (clamped into the tensor: what lands outside is
-    // not stored), its weights for the lane's TM channels, and the sum of its gy for the correction at the end
+    // PAIR: the side layer's gy chunks, staged like gy behind the channel-sum plane (the lane needs the value at its
+    // own output position: no halo involved), its weights for the lane's TM channels, and the sum of its gy for the
+    // correction at the end
     uniform_f32_ptr wsc = as_uniform(bn.side_w) + ci_base;
-    const float *gdp = nullptr;
+    float *side_lds = gplane + GN;
     float gd_next = 0.f, gd_sum = 0.f;
-    if constexpr (PAIR) {
-        gdp = bn.side_gy + ((size_t)nc * Co * Ho + min(hi0 / 2, Ho - 1)) * Wo + min(wi0 / 2, Wo - 1);
-        gd_next = gdp[0];
-    }
 
-    TileStage<typename C::Patch> st;
+    TileStage<typename C::Patch> st, st_side;
     tile_fetch<typename C::Patch, VEC, false, T>(st, gy, 0, Co, n0, N, hb, wb, Ho, Wo);
+    if constexpr (PAIR) tile_fetch<typename C::Patch, VEC, false, T>(st_side, bn.side_gy, 0, Co, n0, N, hb, wb, Ho, Wo);
     {   // this workgroup's input channels: one run of weights per output channel
         const int ci_blk = min((int)blockIdx.y * C::CIW * TM, Ci - TM);
         l2_warm(w + ci_blk * 9, Co, K, min(C::CIW * TM, Ci - ci_blk) * 9);
     }
     tile_commit<typename C::Patch>(st, smem);
+    if constexpr (PAIR) tile_commit<typename C::Patch>(st_side, side_lds);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const int co0 = c * C::CC;
-        if (c + 1 < nchunks) tile_fetch<typename C::Patch, VEC, false, T>(st, gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
+        if (c + 1 < nchunks) {
+            tile_fetch<typename C::Patch, VEC, false, T>(st, gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
+            if constexpr (PAIR)
+                tile_fetch<typename C::Patch, VEC, false, T>(st_side, bn.side_gy, co0 + C::CC, Co, n0, N, hb, wb, Ho, Wo);
+        }
 
         const float *lbase = smem + (c & 1) * C::BUF + lane_off;
+        const float *sbase = side_lds + (c & 1) * C::BUF + lane_off;   // (PAIR)
         const int ccnt = min(C::CC, Co - co0);
         // same software pipeline as the stride-1 kernel: units of HM input channels, next unit's
         // weights and next channel's gy strips requested right after a unit's first instruction
@@ -728,6 +733,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
         if constexpr (PAIR) {
 #pragma unroll
             for (int m = 0; m < TM; ++m) wsv[0][m] = wsc[co0 * Ci + m];
+            gd_next = sbase[0];
         }
 
         auto one_channel = [&](const int cc, const int cur) {
@@ -763,7 +769,7 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
                         if constexpr (PAIR) {
                             if (h == 0) {   // the next output channel's side operands (the last one asks for itself again)
                                 const int cn = min(co0 + cc + 1, Co - 1);
-                                gd_next = gdp[(size_t)cn * Ho * Wo];
+                                gd_next = sbase[(more ? cc + 1 : cc) * C::PLANE];
 #pragma unroll
                                 for (int m2 = 0; m2 < TM; ++m2) wsv[cur ^ 1][m2] = wsc[cn * Ci + m2];
                             }
@@ -810,7 +816,10 @@ __global__ __launch_bounds__(C::NTHREADS) void grad_x_3x3s2_kernel(const T *__re
             }
         }
 
-        if (c + 1 < nchunks) tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
+        if (c + 1 < nchunks) {
+            tile_commit<typename C::Patch>(st, smem + ((c + 1) & 1) * C::BUF);
+            if constexpr (PAIR) tile_commit<typename C::Patch>(st_side, side_lds + ((c + 1) & 1) * C::BUF);
+        }
         __syncthreads();
     }
 
@@ -985,7 +994,8 @@ static int launch_grad_x_3x3s2_v(const T *gy, const T *x, const float *w, T *gx,
     const int gyd = ceil_div(d.Ci, C::TM * C::CIW);
     if (gxd > 0x7fffffffL) return ADDER_ERR_TOO_LARGE;
     if (FUSE && (!bn.in_part || bn.in_slots != gxd * bn_slots_per_wg<C>())) return ADDER_ERR_BAD_SHAPE;
-    constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4;   // two gy chunk buffers + the channel-sum plane
+    // two gy chunk buffers + the channel-sum plane (+ two chunk buffers of the side layer's gy)
+    constexpr int LDS_BYTES = C::LDS_BYTES + C::NIMG * C::PLANE * 4 + (PAIR ? C::LDS_BYTES : 0);
     static_assert(LDS_BYTES <= 48 * 1024, "raise the dynamic LDS limit for this tile");
     hipLaunchKernelGGL((grad_x_3x3s2_kernel<C, VEC, SAT, T, FUSE, PAIR>), dim3((unsigned)gxd, gyd), dim3(C::NTHREADS),
                        LDS_BYTES, s, gy, x, w, gx, d.N, d.Ci, d.H, d.W, d.Co, d.Ho, d.Wo, tilesH, tilesW, gadd, bn);
