@@ -137,6 +137,25 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const float *__res
                                                               long long *__restrict__ num_batches, int relu, int N,
                                                               int C, int HW4) {
     const int c = blockIdx.y;
+    // The loads of the first PRE rounds are issued before the partial sums are added: they do not depend on the
+    // statistics, and a workgroup that first waits for its 16 KB of partial sums and only then asks for its data
+    // spends 1-2 us of a 5-11 us kernel with nothing in flight.
+    constexpr int PRE = 4;
+    const int total = N * HW4, i0 = blockIdx.x * kBnThreads + threadIdx.x, stride = gridDim.x * kBnThreads;
+    Pack<V> pv[PRE], pr[PRE];
+    size_t poff[PRE];
+#pragma unroll
+    for (int k = 0; k < PRE; ++k) {
+        const int i = min(i0 + k * stride, total - 1), n = i / HW4, q = i - n * HW4;
+        poff[k] = ((size_t)n * C + c) * HW4 + q;
+        pv[k] = ld<V>(x, poff[k]);
+#pragma unroll
+        for (int e = 0; e < V; ++e) pr[k].v[e] = 0.f;
+    }
+    if (res) {
+#pragma unroll
+        for (int k = 0; k < PRE; ++k) pr[k] = ld<V>(res, poff[k]);
+    }
     double s1, s2;
     bn_reduce_partials(part, c, S, s1, s2);
     const double mud = s1 / count;
@@ -154,16 +173,11 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const float *__res
         if (c == 0 && num_batches) *num_batches += 1;
     }
     const float sc = gamma[c] * rs, sh = beta[c];
-    const int total = N * HW4;
-    for (int i = blockIdx.x * kBnThreads + threadIdx.x; i < total; i += gridDim.x * kBnThreads) {
-        const int n = i / HW4, q = i - n * HW4;
-        const size_t off = ((size_t)n * C + c) * HW4 + q;
-        const Pack<V> v = ld<V>(x, off);
+    auto emit = [&](const size_t off, const Pack<V> &v, const Pack<V> &r) {
         Pack<V> o;
 #pragma unroll
         for (int e = 0; e < V; ++e) o.v[e] = fmaf(v.v[e] - mu, sc, sh);   // subtract first: |x| >> |x - mean| here
         if (res) {
-            const Pack<V> r = ld<V>(res, off);
 #pragma unroll
             for (int e = 0; e < V; ++e) o.v[e] += r.v[e];
         }
@@ -176,7 +190,7 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const float *__res
             }
             if (V == 4 && mask) {
                 // planes are whole multiples of 8 float4 groups, so the eight lanes of an aligned group hold
-                // the eight consecutive groups of one mask word and are all inside the loop together
+                // the eight consecutive groups of one mask word and are all inside a round together
                 unsigned w = bits << (4 * (unsigned)(off & 7));
                 w |= __shfl_xor(w, 1, 64);
                 w |= __shfl_xor(w, 2, 64);
@@ -185,6 +199,17 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const float *__res
             }
         }
         st<V>(y, off, o);
+    };
+#pragma unroll
+    for (int k = 0; k < PRE; ++k)
+        if (i0 + k * stride < total) emit(poff[k], pv[k], pr[k]);
+    for (int i = i0 + PRE * stride; i < total; i += stride) {
+        const int n = i / HW4, q = i - n * HW4;
+        const size_t off = ((size_t)n * C + c) * HW4 + q;
+        const Pack<V> v = ld<V>(x, off);
+        Pack<V> r = pr[0];   // (any value: not used without a residual)
+        if (res) r = ld<V>(res, off);
+        emit(off, v, r);
     }
 }
 
