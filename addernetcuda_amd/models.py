@@ -37,6 +37,7 @@ import torch.nn.functional as F
 from . import adder as _adder
 from .bn_act import BatchNormAct2d
 from .unit import adder_bn_act
+from .resnet20 import StemConv2d   # nn.Conv2d with the same parameters; forward and weight gradient through the tiled kernels
 
 
 def _bn(channels, relu, fused):
@@ -146,7 +147,7 @@ class VGGSmall(nn.Module):
                 layers.append(nn.MaxPool2d(kernel_size=2, stride=2))
                 continue
             if channels == 3 and not first_adder:
-                conv = nn.Conv2d(3, v, kernel_size=3, padding=1, bias=False)
+                conv = (StemConv2d if fused else nn.Conv2d)(3, v, kernel_size=3, padding=1, bias=False)
             else:
                 conv = make(channels, v, kernel_size=3, stride=1, padding=1, bias=False, **adder_kw)
             layers += [conv, _bn(v, True, fused)]
@@ -314,7 +315,7 @@ class DenseNet(nn.Module):
         self.growth_rate = growth_rate
         kw = dict(adder2d_cls=adder2d_cls, fused=fused, **adder_kw)
         planes = 2 * growth_rate
-        self.conv1 = nn.Conv2d(3, planes, kernel_size=3, padding=1, bias=False)
+        self.conv1 = (StemConv2d if fused else nn.Conv2d)(3, planes, kernel_size=3, padding=1, bias=False)
         for i, blocks in enumerate(num_block, start=1):
             stage = []
             for _ in range(blocks):

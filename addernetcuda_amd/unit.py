@@ -147,6 +147,9 @@ def adder_bn_act(conv, bn, x, residual=None, with_shortcut=False, side_conv=None
                                     and residual.shape[0] == x.shape[0] and residual.dtype == torch.float32
                                     and residual.device == x.device)))
     if not ok:
+        if (not with_shortcut and residual is None and hasattr(conv, "forward_bn_act") and bn.training and x.is_cuda
+                and torch.is_grad_enabled()):
+            return conv.forward_bn_act(x, bn)   # an ordinary convolution with the same kernels (the stem of a network)
         if with_shortcut:
             if hasattr(conv, "forward_with_stats") and bn.training and x.is_cuda:
                 out, stats, shortcut = conv.forward_with_stats(x, with_shortcut=True)
