@@ -63,6 +63,8 @@ _SIGNATURES = {
     "adder_head_supported": (_i, [_i, _i, _i, _i]),
     "adder_head_fwd_f32": (_i, [_p] * 12 + [_f, _f, _i, _i, _i, _i, _p]),
     "adder_head_bwd_f32": (_i, [_p] * 12 + [_i, _i, _i, _i, _p]),
+    "adder_cross_entropy_fwd_f32": (_i, [_p, _p, _p, _p, _i, _i, _p]),
+    "adder_cross_entropy_bwd_f32": (_i, [_p, _p, _p, _p, _p, _i, _i, _p]),
     "adder_sgd_momentum_step_f32": (_i, [_i, _p, _p, _p, _p, _p, _f, _f, _f, _p]),
 }
 for _name, (_res, _args) in _SIGNATURES.items():

@@ -652,6 +652,30 @@ int adder_sgd_momentum_step_f32(int count, float *const *params, const float *co
                                static_cast<hipStream_t>(stream));
 }
 
+int adder_cross_entropy_fwd_f32(const float *logits, const long long *target, float *loss, float *lse, int N,
+                                int classes, void *stream) {
+    if (!logits || !target || !loss || !lse) return ADDER_ERR_NULL_POINTER;
+    if (N <= 0 || classes <= 0) return ADDER_ERR_BAD_SHAPE;
+    if ((long)N * classes > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    const size_t nz = sizeof(float) * (size_t)N * classes, nn = sizeof(float) * (size_t)N;
+    const Span outs[] = {{loss, sizeof(float)}, {lse, nn}};
+    const Span ins[] = {{logits, nz}, {target, sizeof(long long) * (size_t)N}};
+    if (any_alias(outs, ins)) return ADDER_ERR_ALIAS;
+    return launch_ce_fwd(logits, target, loss, lse, N, classes, static_cast<hipStream_t>(stream));
+}
+
+int adder_cross_entropy_bwd_f32(const float *logits, const long long *target, const float *lse, const float *grad_loss,
+                                float *grad_logits, int N, int classes, void *stream) {
+    if (!logits || !target || !lse || !grad_loss || !grad_logits) return ADDER_ERR_NULL_POINTER;
+    if (N <= 0 || classes <= 0) return ADDER_ERR_BAD_SHAPE;
+    if ((long)N * classes > kMaxElems) return ADDER_ERR_TOO_LARGE;
+    const size_t nz = sizeof(float) * (size_t)N * classes, nn = sizeof(float) * (size_t)N;
+    const Span outs[] = {{grad_logits, nz}};
+    const Span ins[] = {{logits, nz}, {target, sizeof(long long) * (size_t)N}, {lse, nn}, {grad_loss, sizeof(float)}};
+    if (any_alias(outs, ins)) return ADDER_ERR_ALIAS;
+    return launch_ce_bwd(logits, target, lse, grad_loss, grad_logits, N, classes, static_cast<hipStream_t>(stream));
+}
+
 int adder_head_supported(int N, int C, int HW, int classes) {
     return (N > 0 && C > 0 && HW > 0 && classes > 0 && head_supported(N, C, HW, classes)) ? 1 : 0;
 }

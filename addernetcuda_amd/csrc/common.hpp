@@ -302,6 +302,10 @@ int launch_head_bwd(const float *dy, const float *z, const float *pooled, const 
                     const float *mean, const float *rstd, float *dz, float *dx, float *dw, float *dgamma, float *dbeta,
                     int N, int C, int HW, int J, hipStream_t s);
 
+int launch_ce_fwd(const float *y, const long long *target, float *loss, float *lse, int N, int J, hipStream_t s);
+int launch_ce_bwd(const float *y, const long long *target, const float *lse, const float *grad_loss, float *gy, int N,
+                  int J, hipStream_t s);
+
 size_t norm_scale_workspace_bytes(long n);
 int launch_norm_scale(float *g, long n, float eta, float eps, void *ws, hipStream_t s);
 static constexpr int kNormBatchMax = ADDER_NORM_BATCH_MAX;

@@ -303,6 +303,75 @@ static void launch_expand(const float *dz, const float *w, float *dx, int N, int
     hipLaunchKernelGGL(head_expand_kernel<HW4>, dim3(N), dim3(kHeadThreads), 0, s, dz, w, dx, C, J);
 }
 
+// ---- the loss of the training script (main.py:66,90: torch.nn.CrossEntropyLoss, mean over the batch) ----------
+// On N x classes logits the framework runs log_softmax and nll_loss forward and backward plus two fills: six launches
+// of 4-8 us.  One workgroup each way here: a thread per image keeps the image's logits in registers.
+static constexpr int kCeThreads = 1024, kCeMaxClasses = 32;
+
+// loss = mean_n (lse_n - y[n, t_n]), lse_n = log sum_j exp(y[n, j]); lse (N) is kept for the backward.
+__global__ __launch_bounds__(kCeThreads) void ce_fwd_kernel(const float *__restrict__ y,
+                                                            const long long *__restrict__ target,
+                                                            float *__restrict__ loss, float *__restrict__ lse, int N,
+                                                            int J) {
+    __shared__ float wsum[kCeThreads / 64];
+    float mine = 0.f;
+    for (int n = threadIdx.x; n < N; n += kCeThreads) {
+        float v[kCeMaxClasses];
+#pragma unroll
+        for (int j = 0; j < kCeMaxClasses; ++j) v[j] = y[(size_t)n * J + min(j, J - 1)];   // (all loads in flight)
+        const int t = (int)min(max(target[n], 0LL), (long long)J - 1);
+        float m = v[0];
+#pragma unroll
+        for (int j = 1; j < kCeMaxClasses; ++j) m = fmaxf(m, v[j]);
+        float sum = 0.f, yt = v[0];
+#pragma unroll
+        for (int j = 0; j < kCeMaxClasses; ++j) {
+            sum += j < J ? expf(v[j] - m) : 0.f;
+            yt = j == t ? v[j] : yt;
+        }
+        const float l = m + logf(sum);
+        lse[n] = l;
+        mine += l - yt;
+    }
+    mine = wave_sum(mine);   // (64 lanes in a fixed butterfly, then the waves in order: the same bits every run)
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.f;
+        for (int w = 0; w < kCeThreads / 64; ++w) total += wsum[w];
+        loss[0] = total / (float)N;
+    }
+}
+
+// grad_logits[n, j] = (exp(y[n, j] - lse_n) - [j == t_n]) * grad_loss / N
+__global__ __launch_bounds__(kCeThreads) void ce_bwd_kernel(const float *__restrict__ y,
+                                                            const long long *__restrict__ target,
+                                                            const float *__restrict__ lse,
+                                                            const float *__restrict__ grad_loss,
+                                                            float *__restrict__ gy, int N, int J) {
+    const float scale = grad_loss[0] / (float)N;
+    const int i = blockIdx.x * kCeThreads + threadIdx.x;
+    if (i < N * J) {
+        const int n = i / J, j = i - n * J;
+        const float p = expf(y[i] - lse[n]);
+        gy[i] = (p - (target[n] == (long long)j ? 1.f : 0.f)) * scale;
+    }
+}
+
+int launch_ce_fwd(const float *y, const long long *target, float *loss, float *lse, int N, int J, hipStream_t s) {
+    if (J > kCeMaxClasses) return ADDER_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(ce_fwd_kernel, dim3(1), dim3(kCeThreads), 0, s, y, target, loss, lse, N, J);
+    return check_launch();
+}
+
+int launch_ce_bwd(const float *y, const long long *target, const float *lse, const float *grad_loss, float *gy, int N,
+                  int J, hipStream_t s) {
+    if (J > kCeMaxClasses) return ADDER_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(ce_bwd_kernel, dim3(ceil_div(N * J, kCeThreads)), dim3(kCeThreads), 0, s, y, target, lse, grad_loss,
+                       gy, N, J);
+    return check_launch();
+}
+
 #define ADDER_HEAD_DISPATCH(fn, ...)                       \
     switch (HW / 4) {                                      \
         case 1: fn<1>(__VA_ARGS__); break;                 \

@@ -110,8 +110,9 @@ def evaluate(net, x_u8, y, batch, bf16=False):
 
 def train_step(net, opt, images, labels, bf16=False):
     from addernetcuda_amd.adder import batched_eta_scaling
+    from addernetcuda_amd.head import cross_entropy
     opt.zero_grad(set_to_none=True)
-    loss = F.cross_entropy(forward_pass(net, images, bf16), labels)
+    loss = cross_entropy(forward_pass(net, images, bf16), labels)   # nn.CrossEntropyLoss of main.py:66,90
     with batched_eta_scaling():   # the adaptive scaling of all adder layers in two launches
         loss.backward()
     opt.step()

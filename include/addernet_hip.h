@@ -28,6 +28,7 @@
  *   [optional]  BatchNorm + residual + ReLU kernels (adder_bn_act_*)
  *   [optional]  BatchNorm backward passes folded into the adder backward kernels (adder_bn_links, *_bn_*)
  *   [optional]  the classifier head of the ResNets: average pool, matrix product, BatchNorm (adder_head_*)
+ *   [optional]  the cross-entropy loss in one launch each way (adder_cross_entropy_*)
  *   [optional]  the momentum-SGD update of all parameters in one launch (adder_sgd_momentum_step_f32)
  */
 #ifndef ADDERNET_HIP_H
@@ -409,6 +410,20 @@ ADDER_API int adder_head_bwd_f32(const float *dy, const float *z, const float *p
                                  const float *gamma, const float *save_mean, const float *save_rstd,
                                  float *dz, float *dx, float *dw, float *dgamma, float *dbeta,
                                  int N, int C, int HW, int classes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * [optional] The loss of the training script (main.py:66,90 of the reference: torch.nn.CrossEntropyLoss with its
+ * defaults -- class indices as targets, mean over the batch) in one launch each way, for at most 32 classes
+ * (ADDER_ERR_UNSUPPORTED above that).  target: N int64 class indices in [0, classes).
+ *   adder_cross_entropy_fwd_f32: loss[0] = mean_n (lse[n] - logits[n, target[n]]), lse[n] = log sum_j exp(logits[n, j]),
+ *     kept for the backward.  adder_cross_entropy_bwd_f32: grad_logits[n, j] =
+ *     (exp(logits[n, j] - lse[n]) - [j == target[n]]) * grad_loss[0] / N, grad_loss one float in device memory.
+ * ---------------------------------------------------------------------- */
+ADDER_API int adder_cross_entropy_fwd_f32(const float *logits, const long long *target, float *loss, float *lse,
+                                          int N, int classes, void *stream);
+ADDER_API int adder_cross_entropy_bwd_f32(const float *logits, const long long *target, const float *lse,
+                                          const float *grad_loss, float *grad_logits, int N, int classes,
+                                          void *stream);
 
 /* ------------------------------------------------------------------------
  * [optional] The parameter update of the training script (main.py:67 of the reference: torch.optim.SGD with

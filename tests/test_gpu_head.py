@@ -124,3 +124,38 @@ def test_refusals(gpu):
     assert lib.adder_head_fwd_f32(*args(t, t), 8, 64, 64, 10, st) == ADDER_ERR_ALIAS
     fc, bn = nn.Conv2d(64, 10, 1, bias=True).to(gpu), nn.BatchNorm2d(10).to(gpu)
     assert not head_applies(torch.zeros(8, 64, 8, 8, device=gpu), fc, bn)      # an fc with a bias
+
+
+@pytest.mark.parametrize("shape", [(256, 10), (7, 3), (1, 1), (1500, 32), (64, 17)], ids=str)
+def test_cross_entropy_matches_torch_in_float64(shape, gpu):
+    from addernetcuda_amd.head import cross_entropy
+    N, J = shape
+    g = torch.Generator().manual_seed(5 + N + J)
+    logits = torch.randn(N, J, generator=g) * 4
+    target = torch.randint(0, J, (N,), generator=g)
+    l64 = logits.double().requires_grad_(True)
+    ref = torch.nn.functional.cross_entropy(l64, target)
+    ref.backward(torch.tensor(0.7, dtype=torch.float64))
+    lg = logits.to(gpu).requires_grad_(True)
+    loss = cross_entropy(lg, target.to(gpu))
+    assert loss.shape == () and loss.grad_fn is not None and "_cross_entropy" in type(loss.grad_fn).__name__
+    loss.backward(torch.tensor(0.7, device=gpu))
+    torch.cuda.synchronize()
+    assert_close(loss, ref.detach(), "loss", rtol=1e-6, atol=1e-6)
+    assert_close(lg.grad, l64.grad, "gradient of the logits", rtol=1e-5, atol=1e-7)
+    # two runs: the same bits
+    lg2 = logits.to(gpu).requires_grad_(True)
+    loss2 = cross_entropy(lg2, target.to(gpu))
+    loss2.backward(torch.tensor(0.7, device=gpu))
+    assert torch.equal(loss2, loss) and torch.equal(lg2.grad, lg.grad)
+
+
+def test_cross_entropy_leaves_the_rest_to_torch(gpu):
+    from addernetcuda_amd.head import cross_entropy
+    logits = torch.randn(8, 100, device=gpu, requires_grad=True)      # more classes than the kernel keeps in registers
+    target = torch.randint(0, 100, (8,), device=gpu)
+    loss = cross_entropy(logits, target)
+    assert "_cross_entropy" not in type(loss.grad_fn).__name__
+    assert torch.equal(loss, torch.nn.functional.cross_entropy(logits, target))
+    cpu = cross_entropy(torch.randn(4, 5), torch.randint(0, 5, (4,)))
+    assert cpu.shape == ()
