@@ -458,7 +458,7 @@ def cpu_model_name():
 
 
 def cpu_layer_baseline(repeats=3):   # ~25 s of host work
-    """BASELINE config 2 on the host: the three 3x3 / stride 1 / pad 1 layer shapes (16, 32, 64 channels at 32, 16, 8
+    """The per-layer benchmark configuration on the host: the three 3x3 / stride 1 / pad 1 layer shapes (16, 32, 64 channels at 32, 16, 8
     pixels, batch 256) through the chunked torch oracle -- unfold (adder.py:32-33), forward (test_cuda.py:18-22),
     grad_W (test_cuda.py:35-41), grad_X (test_cuda.py:57-60), and grad_W with the scaling of adder.py:78 -- each
     the median of `repeats` runs."""
@@ -525,7 +525,7 @@ def cpu_baseline(repeats=15):   # ~10 s of host work
                   f"{repeats} steps = {med * 1e3:.0f} ms, scaled x{BATCH // bs} to batch 256",
         "host_cpus": os.cpu_count(), "cpu_model": cpu_model_name(),
         "layers": cpu_layer_baseline(),
-        "layers_note": "BASELINE config 2 on the host cores: the three stride-1 3x3 shapes at batch 256 through the "
+        "layers_note": "the per-layer benchmark configuration on the host cores: the three stride-1 3x3 shapes at batch 256 through the "
                        "chunked pure-PyTorch oracle (the formulas of adder_cuda/test_cuda.py:18-22,35-41,57-60 and "
                        "adder.py:78 on the unfolded (K, L*N) matrix), median of 3 runs each, all intra-op threads",
     }
